@@ -1,0 +1,202 @@
+/*
+ * vsp_attn.h — C ABI of libvsp_attn.so: the MI355X (gfx950) implementation of
+ * the reference's attention hot path (causal GQA flash-attention prefill,
+ * single-token decode over the KV cache, KV-cache append/read).
+ *
+ * The reference (danielmriley/vesper) has no FFI; its operator seam is a set
+ * of C++ per-backend dispatch functions declared in public headers.  Each
+ * entry point below names the reference interface it replaces (paths relative
+ * to the reference tree).  The C++ mirror of those interfaces — same names,
+ * argument meaning and exceptions — lives in vesper_amd/csrc/adapter/ and is
+ * implemented on top of exactly these calls.
+ *
+ * Conventions
+ *   - plain pointers and sizes only; every pointer in a vsp_tensor / vsp_kv_cache
+ *     is DEVICE memory owned by the caller; the library never allocates, never
+ *     frees and never keeps a pointer after a call returns;
+ *   - all work is enqueued asynchronously on `stream` (a hipStream_t passed as
+ *     void*; NULL = the null stream), the way the reference enqueues on
+ *     Stream::current(Device::HIP) (src/core/stream.cpp:104-166).  No call
+ *     synchronises;
+ *   - strides are in ELEMENTS, like Tensor::strides() (include/vesper/core/tensor.h:30);
+ *   - every call returns a vsp_status; nothing throws across the boundary.
+ *     vsp_status_str() returns, where one exists, the reference's exception text.
+ */
+#ifndef VSP_ATTN_H
+#define VSP_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define VSP_ATTN_ABI_VERSION 1
+
+typedef enum {
+    VSP_OK = 0,
+    /* the reference's own failures (text identical to its exceptions) */
+    VSP_ERR_NDIM = 1,        /* flash_attention: inputs must be 4D [B, H, N, D]        (src/ops/flash_attention.cpp:45-47) */
+    VSP_ERR_SHAPE = 2,       /* flash_attention: Q, K, V must have same shape          (:49-51; GQA-aware, see vsp_attn_prefill) */
+    VSP_ERR_DTYPE = 3,       /* flash_attention: Q, K, V must have same dtype          (:53-55) */
+    VSP_ERR_DROPOUT = 4,     /* flash_attention: dropout_p must be in [0, 1)           (:57-59) */
+    VSP_ERR_NUMEL = 5,       /* copy_from: element count mismatch.                     (src/core/tensor.cpp:198-200) */
+    VSP_ERR_COPY_DTYPE = 6,  /* copy_from: dtype mismatch.                             (src/core/tensor.cpp:201-203) */
+    VSP_ERR_REPEAT_NDIM = 7, /* repeat_kv: input must be 4D [...]                      (src/ops/attention_ops.cpp:97-99) */
+    VSP_ERR_GQA_HEADS = 8,   /* GroupedQueryAttention: num_heads ... divisible by num_kv_heads (src/nn/gqa_attention.cpp:47-51) */
+    VSP_ERR_GQA_EMBED = 9,   /* GroupedQueryAttention: embed_dim ... divisible by num_heads    (:52-56) */
+    VSP_ERR_BROADCAST = 10,  /* causal mask [T,T] cannot be added to scores [T,L]      (src/nn/functional.cpp:406-410) */
+    /* failures that only exist at this boundary */
+    VSP_ERR_NULL = 32,        /* a required pointer is NULL */
+    VSP_ERR_UNSUPPORTED = 33, /* dtype/format/head_dim combination the kernels do not implement */
+    VSP_ERR_STRIDE = 34,      /* innermost stride != 1, or a stride the kernel cannot address */
+    VSP_ERR_ALIGN = 35,       /* a base pointer or row pitch is not 16-byte aligned */
+    VSP_ERR_WORKSPACE = 36,   /* workspace missing or smaller than vsp_attn_workspace_bytes() */
+    VSP_ERR_ARG = 37,         /* an argument is out of range (negative size, len > S_max, ...) */
+    VSP_ERR_LAUNCH = 38       /* the HIP runtime rejected a launch (hipGetLastError text via vsp_last_hip_error) */
+} vsp_status;
+
+typedef enum {
+    VSP_F32 = 0,  /* DType::Float32  (include/vesper/core/dtype.h:9-16) */
+    VSP_BF16 = 1, /* DType::BFloat16: raw bits of include/vesper/core/half.h:157 */
+    VSP_F16 = 2,  /* IEEE binary16 (scales of Q8_0 planes only) */
+    VSP_I8 = 3,
+    VSP_I32 = 4
+} vsp_dtype;
+
+/* A strided view, the part of vesper::Tensor a kernel needs
+ * (data_ptr() already includes the element offset, include/vesper/core/tensor.h:68-80). */
+typedef struct {
+    void* data;
+    int32_t dtype; /* vsp_dtype */
+    int32_t ndim;  /* <= 4 */
+    int64_t shape[4];
+    int64_t stride[4]; /* elements */
+} vsp_tensor;
+
+/* ---- KV cache ---------------------------------------------------------------
+ * Replaces the storage of nn::KVCache (include/vesper/nn/transformer.h:21-39,
+ * src/nn/transformer.cpp:32-93) and nn::GQAKVCache (include/vesper/nn/gqa_attention.h:110-163).
+ * Logical content is the reference's: K and V of shape [B, Hkv, S_max, D], one
+ * current length for the whole batch.  Physical layout per format (S_pad =
+ * S_max rounded up to a multiple of 64; all planes are zero-initialised by
+ * vsp_kv_cache_reset):
+ *
+ *  VSP_KV_F32   the reference's own layout, both planes fp32 row-major
+ *               [B][Hkv][S_max][D]; element (b,h,s,d) at ((b*Hkv+h)*S_max+s)*D+d.
+ *  VSP_KV_BF16  k: bf16 row-major [B][Hkv][S_pad][D]
+ *               v: bf16 token-blocked, transposed inside the block:
+ *                  [B][Hkv][S_pad/8][D][8]; element (b,h,s,d) at
+ *                  (((b*Hkv+h)*(S_pad/8) + s/8)*D + d)*8 + s%8.
+ *               (PV contracts over tokens; with 8 consecutive tokens of one d
+ *               contiguous, a lane's 16-byte load is an MFMA operand as it is.)
+ *  VSP_KV_Q8_0  rows quantised in blocks of 32 along D (ggml block_q8_0
+ *               arithmetic: d = max|x|/127 stored as fp16 RNE, q = roundf(x/d)).
+ *               k:       int8 [B][Hkv][S_pad][D]
+ *               k_scale: fp16 [B][Hkv][S_pad][D/32]
+ *               v:       int8 [B][Hkv][S_pad/16][D][16]   (token-blocked by 16)
+ *               v_scale: fp16 [B][Hkv][S_pad/16][D/32][16]
+ * D must be 64 or 128 for BF16/Q8_0.  Plane sizes: vsp_kv_plane_bytes().
+ */
+typedef enum { VSP_KV_F32 = 0, VSP_KV_BF16 = 1, VSP_KV_Q8_0 = 2 } vsp_kv_format;
+typedef enum { VSP_KV_PLANE_K = 0, VSP_KV_PLANE_V = 1, VSP_KV_PLANE_K_SCALE = 2, VSP_KV_PLANE_V_SCALE = 3 } vsp_kv_plane;
+
+typedef struct {
+    int32_t format; /* vsp_kv_format */
+    int32_t B, Hkv, S_max, D;
+    void* k;
+    void* v;
+    void* k_scale; /* Q8_0 only, else NULL */
+    void* v_scale; /* Q8_0 only, else NULL */
+    int32_t len;   /* the reference's current_len_ (host side, maintained by vsp_kv_append) */
+} vsp_kv_cache;
+
+/* Bytes the caller must allocate for one plane (0 for planes the format lacks). */
+size_t vsp_kv_plane_bytes(int32_t format, int32_t B, int32_t Hkv, int32_t S_max, int32_t D, int32_t plane);
+
+/* KVCache::reset(), src/nn/transformer.cpp:45-54 / GQAKVCache::reset(), src/nn/gqa_attention.cpp:209-214:
+ * zero every plane (a fill kernel, not a memset node, so it may be graph-captured) and set len = 0.
+ * Also the way a freshly allocated cache reaches the constructor's all-zero state (:40-41). */
+int vsp_kv_cache_reset(vsp_kv_cache* cache, void* stream);
+
+/* KVCache::update(new_k,new_v,start_pos) write half, src/nn/transformer.cpp:56-73 (== gqa_attention.cpp:175-194),
+ * replacing ops::index + Tensor::copy_from + copy_strided_hip_dispatch (include/vesper/ops/copy.h:12,
+ * src/ops/hip/copy.hip:16-93).  new_k/new_v: [B,Hkv,T,D], fp32 or bf16, any strides with stride[3]==1.
+ * The slot is [:, :, start_pos:start_pos+T, :] under the reference's Python-slice clamping
+ * (src/ops/view_ops.cpp:270-316); if the clamped slot does not hold exactly the elements of
+ * new_k -> VSP_ERR_NUMEL, nothing written, len unchanged.  Conversion on write: fp32 -> bf16 is the
+ * reference's round-to-nearest-even (include/vesper/core/half.h:162-173); Q8_0 quantises per row.
+ * Afterwards len = max(len, start_pos + T).
+ * start_pos_dev (nullable): device int32[B], per-sequence start positions for ragged batches
+ * (no counterpart in the reference, which has one position for the batch); when given, start_pos
+ * is ignored for placement, each row b is written at start_pos_dev[b] (caller guarantees
+ * 0 <= start_pos_dev[b] and start_pos_dev[b]+T <= S_max) and len is left unchanged. */
+int vsp_kv_append(vsp_kv_cache* cache, const vsp_tensor* new_k, const vsp_tensor* new_v, int64_t start_pos,
+                  const int32_t* start_pos_dev, void* stream);
+
+/* The read half of KVCache::update, :75-92: the reference returns VIEWS [:, :, 0:len, :] of its fp32
+ * storage.  For VSP_KV_F32 the same view can be formed by the caller (vsp_kv_view_f32); for the other
+ * formats this call materialises logical rows [start, start+count) into k_out/v_out
+ * ([B,Hkv,count,D], fp32 or bf16, strided): bf16 planes are copied bit-for-bit (widened exactly for
+ * fp32), Q8_0 planes are dequantised as q * f16->f32(scale).  Used by tests and by callers that
+ * need the reference-shaped tensors; the attention kernels read the planes directly. */
+int vsp_kv_read(const vsp_kv_cache* cache, int64_t start, int64_t count, vsp_tensor* k_out, vsp_tensor* v_out,
+                void* stream);
+/* Q8_0 only: the raw logical blocks, for bit-exact packing checks. qs_out int8 [B,Hkv,count,D],
+ * scale_out fp16 bits [B,Hkv,count,D/32], both contiguous; plane = VSP_KV_PLANE_K or _V. */
+int vsp_kv_read_q8_0(const vsp_kv_cache* cache, int32_t plane, int64_t start, int64_t count, int8_t* qs_out,
+                     uint16_t* scale_out, void* stream);
+/* VSP_KV_F32: fill k_view/v_view with the reference's view [:, :, 0:len, :] (shape, strides, offset 0). */
+int vsp_kv_view_f32(const vsp_kv_cache* cache, vsp_tensor* k_view, vsp_tensor* v_view);
+
+/* ---- prefill ------------------------------------------------------------------
+ * Replaces flash_attention_hip_dispatch (include/vesper/ops/flash_attention.h:74-78, defined at
+ * src/ops/hip/flash_attention.hip:305-331), with repeat_kv_hip_dispatch
+ * (include/vesper/ops/attention_ops.h:35) folded in: q [B,Hq,T,D]; k, v [B,Hkv,L,D] with
+ * Hq % Hkv == 0, query head h reading kv head h / (Hq/Hkv) (src/ops/attention_ops.cpp:47).
+ * out [B,Hq,T,D] same dtype as q; lse [B,Hq,T] fp32 or NULL (= m + log l, src/ops/flash_attention.cpp:359).
+ * dtype bf16 (MFMA, fp32 accumulation) or fp32.  D in {64,128}.  q/k/v/out may be strided
+ * (stride[3]==1, rows 16-byte aligned), e.g. VSP_KV_F32 cache views.
+ * is_causal: key j visible to query t iff j <= t + (L - T): the reference's mask when T == L
+ * (src/ops/flash_attention.cpp:293-296), and its natural extension to a chunk appended at the end
+ * of a longer context.  T > L with is_causal -> VSP_ERR_SHAPE.
+ * Validation order and codes follow src/ops/flash_attention.cpp:45-59. */
+int vsp_attn_prefill(const vsp_tensor* q, const vsp_tensor* k, const vsp_tensor* v, vsp_tensor* out, vsp_tensor* lse,
+                     float scale, int is_causal, float dropout_p, int training, void* stream);
+
+/* ---- decode -------------------------------------------------------------------
+ * Replaces, for T == 1, the op chain scaled_dot_product_attention runs below its flash threshold
+ * (src/nn/functional.cpp:397-421: gemm_batch_hip_dispatch x2, div_scalar, softmax_hip_dispatch)
+ * and the two repeat_kv copies before it (src/nn/gqa_attention.cpp:140-141).
+ * q, out: [B,Hq,1,D] bf16 (fp32 for a VSP_KV_F32 cache).  Every query head attends, unmasked, to
+ * positions [0, L_b) of its kv head, L_b = seq_lens[b] (device int32[B]) or cache->len when
+ * seq_lens is NULL.  L_b == 0 yields zeros.  max_len: host-side upper bound of L_b used to size the
+ * launch (0 = cache->len if seq_lens is NULL, else S_max).
+ * Split-K over the context: partial (m, l, acc) per (b, head, split) go to `workspace`
+ * (>= vsp_attn_decode_workspace_bytes), then a combine kernel reduces them in a fixed order
+ * (bitwise run-to-run deterministic). */
+size_t vsp_attn_decode_workspace_bytes(int32_t B, int32_t Hq, int32_t D, int32_t max_len);
+int vsp_attn_decode(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, int32_t max_len,
+                    vsp_tensor* out, float scale, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- host-side, bit-exact format helpers (pure CPU; exported for tests and callers) ---- */
+uint16_t vsp_f32_to_bf16(float f);   /* include/vesper/core/half.h:162-173 */
+float vsp_bf16_to_f32(uint16_t b);   /* include/vesper/core/half.h:175-181 */
+uint16_t vsp_f32_to_f16(float f);    /* IEEE RNE */
+float vsp_f16_to_f32(uint16_t h);
+void vsp_q8_0_quantize_row(const float* x, int64_t n, uint16_t* scale, int8_t* qs);
+void vsp_q8_0_dequantize_row(const uint16_t* scale, const int8_t* qs, int64_t n, float* x);
+/* The reference's slice clamping for one dimension (src/ops/view_ops.cpp:270-316, step 1). */
+void vsp_slice_bounds(int64_t dim_size, int64_t start, int64_t stop, int64_t* out_start, int64_t* out_len);
+/* GroupedQueryAttention constructor arithmetic and checks (src/nn/gqa_attention.cpp:38-57). */
+int vsp_gqa_config(int64_t embed_dim, int64_t num_heads, int64_t num_kv_heads, int64_t* head_dim, int64_t* num_rep);
+
+const char* vsp_status_str(int status);
+const char* vsp_last_hip_error(void); /* text of the last HIP error seen by this thread ("" if none) */
+int vsp_attn_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VSP_ATTN_H */

@@ -1,0 +1,202 @@
+"""Python view of the reference's operator surface for the attention path, on torch device tensors.
+
+torch is used for device memory and streams only; every computation is a call into libvsp_attn.so.
+Names and argument meaning follow the reference (paths relative to its tree):
+  flash_attention(q,k,v,scale,is_causal,dropout_p,training)  include/vesper/ops/flash_attention.h:34-41
+  scaled_dot_product_attention(q,k,v,is_causal,dropout_p)     include/vesper/nn/functional.h:132-136
+  KVCache / GQAKVCache .update/.reset/.current_seq_len         include/vesper/nn/transformer.h:21-39,
+                                                               include/vesper/nn/gqa_attention.h:110-163
+  attention_core(q,k,v,cache,start_pos)                        steps 4-6 of GroupedQueryAttention::forward,
+                                                               src/nn/gqa_attention.cpp:128-148
+"""
+import ctypes as C
+import math
+
+import torch
+
+from . import _ffi
+from ._ffi import VspError, VspKVCache, VspTensor, check, lib
+
+_DT = {torch.float32: _ffi.F32, torch.bfloat16: _ffi.BF16, torch.float16: _ffi.F16, torch.int8: _ffi.I8,
+       torch.int32: _ffi.I32}
+
+
+def _desc(t):
+    d = VspTensor()
+    d.data = t.data_ptr() if t.numel() > 0 else (t.data_ptr() or 0)
+    if t.dtype not in _DT:
+        raise VspError(_ffi.ERR_UNSUPPORTED)
+    d.dtype = _DT[t.dtype]
+    d.ndim = min(t.dim(), 4)
+    for i in range(min(t.dim(), 4)):
+        d.shape[i] = t.shape[i]
+        d.stride[i] = t.stride(i)
+    if t.dim() > 4:
+        d.ndim = t.dim()  # rejected by the library with the reference's message
+    return d
+
+
+def _stream(t):
+    return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def repeat_kv_is_fused():
+    """ops::repeat_kv (src/ops/attention_ops.cpp:92-155) has no kernel here: query head h reads kv head
+    h // n_rep inside the attention kernels."""
+    return True
+
+
+def flash_attention(q, k, v, scale, is_causal=True, dropout_p=0.0, training=False, return_lse=False):
+    """ops::flash_attention; k, v may have fewer heads than q (GQA)."""
+    if not (q.is_cuda and k.is_cuda and v.is_cuda):
+        raise RuntimeError("flash_attention: unsupported device")  # src/ops/flash_attention.cpp:111-112
+    out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    lse = torch.empty(q.shape[:3], dtype=torch.float32, device=q.device) if (return_lse and q.dim() == 4) else None
+    dq, dk, dv, do = _desc(q), _desc(k), _desc(v), _desc(out)
+    dl = _desc(lse) if lse is not None else None
+    check(lib.vsp_attn_prefill(C.byref(dq), C.byref(dk), C.byref(dv), C.byref(do),
+                               C.byref(dl) if dl is not None else None, float(scale), int(bool(is_causal)),
+                               float(dropout_p), int(bool(training)), _stream(q)))
+    return (out, lse) if return_lse else out
+
+
+class KVCache:
+    """nn::KVCache with selectable storage: fmt 'f32' (the reference's layout), 'bf16' or 'q8_0'."""
+
+    _FMT = {"f32": _ffi.KV_F32, "bf16": _ffi.KV_BF16, "q8_0": _ffi.KV_Q8_0}
+
+    def __init__(self, batch_size, num_heads, max_seq_len, head_dim, device="cuda", fmt="f32"):
+        self.fmt = fmt
+        self.device = torch.device(device)
+        c = VspKVCache()
+        c.format = self._FMT[fmt]
+        c.B, c.Hkv, c.S_max, c.D = batch_size, num_heads, max_seq_len, head_dim
+        self._planes = []
+        for plane in range(4):
+            n = lib.vsp_kv_plane_bytes(c.format, c.B, c.Hkv, c.S_max, c.D, plane)
+            self._planes.append(torch.empty(n, dtype=torch.uint8, device=self.device) if n else None)
+        c.k, c.v, c.k_scale, c.v_scale = [p.data_ptr() if p is not None else None for p in self._planes]
+        c.len = 0
+        self._c = c
+        check(lib.vsp_kv_cache_reset(C.byref(c), _stream(self._planes[0])))  # vesper::zeros, transformer.cpp:40-41
+
+    # -- reference interface
+    def current_seq_len(self):
+        return int(self._c.len)
+
+    def get_max_seq_len(self):
+        return int(self._c.S_max)
+
+    max_seq_len = get_max_seq_len
+
+    def reset(self):
+        check(lib.vsp_kv_cache_reset(C.byref(self._c), _stream(self._planes[0])))
+
+    def update(self, new_k, new_v, start_pos, return_views=True, start_pos_dev=None):
+        dk, dv = _desc(new_k), _desc(new_v)
+        sp = C.c_void_p(start_pos_dev.data_ptr()) if start_pos_dev is not None else None
+        check(lib.vsp_kv_append(C.byref(self._c), C.byref(dk), C.byref(dv), int(start_pos), sp, _stream(new_k)))
+        if not return_views:
+            return None
+        return self.views()
+
+    # -- reads
+    def views(self, dtype=None):
+        """[:, :, 0:len, :] of K and V.  fp32 storage: true views (no copy), like the reference;
+        other formats: materialised in `dtype` (default fp32)."""
+        c = self._c
+        if c.format == _ffi.KV_F32:
+            shape = (c.B, c.Hkv, c.S_max, c.D)
+            k = self._planes[0].view(torch.float32).view(shape)[:, :, :c.len, :]
+            v = self._planes[1].view(torch.float32).view(shape)[:, :, :c.len, :]
+            return k, v
+        return self.read(0, c.len, dtype or torch.float32)
+
+    def read(self, start, count, dtype=torch.float32):
+        c = self._c
+        k = torch.empty((c.B, c.Hkv, count, c.D), dtype=dtype, device=self.device)
+        v = torch.empty_like(k)
+        dk, dv = _desc(k), _desc(v)
+        check(lib.vsp_kv_read(C.byref(c), int(start), int(count), C.byref(dk), C.byref(dv), _stream(k)))
+        return k, v
+
+    def read_q8_0(self, plane, start, count):
+        c = self._c
+        qs = torch.empty((c.B, c.Hkv, count, c.D), dtype=torch.int8, device=self.device)
+        sc = torch.empty((c.B, c.Hkv, count, c.D // 32), dtype=torch.int16, device=self.device)
+        check(lib.vsp_kv_read_q8_0(C.byref(c), plane, int(start), int(count), qs.data_ptr(), sc.data_ptr(), _stream(qs)))
+        return qs, sc
+
+    def raw_plane(self, plane):
+        return self._planes[plane]
+
+    def set_len(self, n):
+        """Bench/test helper: declare `n` tokens valid without appending (planes filled directly)."""
+        self._c.len = int(n)
+
+
+class GQAKVCache(KVCache):
+    """nn::GQAKVCache: same semantics, int64 bookkeeping in the reference."""
+
+
+_WS = {}
+
+
+def _workspace(device, nbytes):
+    key = (device.type, device.index)
+    ws = _WS.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
+        _WS[key] = ws
+    return ws
+
+
+def decode_attention(q, cache, seq_lens=None, max_len=0, scale=None, out=None):
+    """One new token per sequence attending to the cache: q [B,Hq,1,D] -> [B,Hq,1,D]."""
+    c = cache._c
+    if scale is None:
+        scale = 1.0 / math.sqrt(q.shape[-1])  # src/nn/functional.cpp:403
+    if out is None:
+        out = torch.empty_like(q)
+    bound = max_len or (c.S_max if seq_lens is not None else c.len)
+    nbytes = lib.vsp_attn_decode_workspace_bytes(q.shape[0], q.shape[1], q.shape[3], max(int(bound), 1))
+    ws = _workspace(q.device, nbytes)
+    dq, do = _desc(q), _desc(out)
+    sl = C.c_void_p(seq_lens.data_ptr()) if seq_lens is not None else None
+    check(lib.vsp_attn_decode(C.byref(dq), C.byref(c), sl, int(max_len), C.byref(do), float(scale),
+                              C.c_void_p(ws.data_ptr()), ws.numel(), _stream(q)))
+    return out
+
+
+def scaled_dot_product_attention(q, k, v, is_causal=False, dropout_p=0.0):
+    """functional::scaled_dot_product_attention (src/nn/functional.cpp:370-422) on explicit tensors.
+    The reference switches algorithm at T >= 512 for speed; here one kernel serves every T.
+    Like the reference, a causal mask needs T == L (its [T,T] mask does not broadcast otherwise)
+    unless T == 1."""
+    if dropout_p > 0.0:
+        raise VspError(_ffi.ERR_UNSUPPORTED)
+    T, L = q.shape[2], k.shape[2]
+    if is_causal and T != L and T != 1:
+        raise VspError(_ffi.ERR_BROADCAST)
+    scale = 1.0 / math.sqrt(q.shape[-1])
+    return flash_attention(q, k, v, scale, is_causal=bool(is_causal) and T > 1)
+
+
+def attention_core(q, new_k, new_v, cache=None, start_pos=0):
+    """Steps 4-6 of GroupedQueryAttention::forward(x, cache, start_pos), src/nn/gqa_attention.cpp:128-148
+    (== MultiHeadAttention::forward, src/nn/transformer.cpp:190-205, with n_rep = 1):
+    cache.update(k, v, start_pos); repeat_kv (fused); SDPA with use_causal = (T > 1)."""
+    T = q.shape[2]
+    if cache is None:
+        return scaled_dot_product_attention(q, new_k, new_v, is_causal=(T > 1))
+    cache.update(new_k, new_v, start_pos, return_views=False)
+    if T == 1:
+        return decode_attention(q, cache)
+    if cache.fmt == "f32":
+        k, v = cache.views()
+    else:
+        k, v = cache.views(dtype=q.dtype)
+    L = k.shape[2]
+    if L != T:
+        raise VspError(_ffi.ERR_BROADCAST)  # the reference's [T,T] mask cannot be added to [T,L] scores
+    return flash_attention(q, k, v, 1.0 / math.sqrt(q.shape[-1]), is_causal=True)

@@ -1,0 +1,652 @@
+// Single-token decode over the KV cache: split-K over the context + combine.
+//
+// Replaces, for T == 1, what the reference runs below its flash threshold
+// (src/nn/functional.cpp:397-421: matmul, div, softmax, matmul over a materialised score tensor)
+// together with the two repeat_kv copies before it (src/nn/gqa_attention.cpp:140-141).
+//
+// One workgroup (4 wavefronts) handles one (batch row, kv head, context split).  The n_rep query
+// heads that share the kv head ride in the N dimension of 16x16x32 MFMA tiles (padded to 16), so
+// K and V are read from HBM exactly once per kv head:
+//   S^T[key][head]  = K[key][:] . Q^T[:][head]        A = K rows as they lie in HBM (16-byte loads)
+//   O^T[d][head]   += V^T[d][key] . P^T[key][head]    A = V^T, which the token-blocked V plane
+//                                                     stores so that 8/16 tokens of one d are one load
+// A wavefront consumes 64 keys per iteration.  MFMA row i of S^T tile jj (0..3) is key
+// 16*(i/4) + 4*jj + i%4 of the group, which makes the four S values a lane gets from each tile
+// line up with the contraction slots of the PV MFMAs (slot (t, g, e) = key 16*g + 8*t + e) without
+// any cross-lane movement.  Online softmax in fp32, exp2 with the scale folded in.
+#include <stdlib.h>
+
+#include "kv_layout.hpp"
+#include "vsp_common.hpp"
+
+namespace vsp {
+int check_kv_cache(const vsp_kv_cache* c);
+
+namespace {
+
+constexpr int kWaves = 4;
+constexpr int kGroup = 64;  // keys per wave iteration
+
+struct DecodeArgs {
+    const void* q;
+    int64_t sq_b, sq_h;  // q strides (elements) of dims 0, 1
+    const void* k;
+    const void* v;
+    const void* k_scale;
+    const void* v_scale;
+    const int32_t* seq_lens;  // device, or nullptr
+    int32_t len;              // used when seq_lens == nullptr
+    int32_t Hq, Hkv, n_rep;
+    int64_t S;  // physical token capacity of the planes
+    int32_t S_max;  // logical capacity; lengths are clamped to it
+    int32_t chunk;
+    int32_t max_splits;
+    float scale_log2;  // scale * log2(e)
+    float* ws_o;       // [B][Hq][max_splits][D]
+    float* ws_ml;      // [B][Hq][max_splits][2]  (m in log2 domain, l)
+};
+
+__device__ inline float wave_max_over_groups(float x) {
+    x = fmaxf(x, __shfl_xor(x, 16));
+    x = fmaxf(x, __shfl_xor(x, 32));
+    return x;
+}
+__device__ inline float wave_sum_over_groups(float x) {
+    x += __shfl_xor(x, 16);
+    x += __shfl_xor(x, 32);
+    return x;
+}
+
+__device__ inline uint4 mask_tail_u16x8(uint4 v, int nvalid) {
+    // keep the first nvalid 16-bit elements, zero the rest
+    uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int rem = nvalid - 2 * i;
+        w[i] = rem >= 2 ? w[i] : (rem == 1 ? (w[i] & 0xFFFFu) : 0u);
+    }
+    return uint4{w[0], w[1], w[2], w[3]};
+}
+
+// ---------------------------------------------------------------------------------------------
+// bf16 cache
+// ---------------------------------------------------------------------------------------------
+template <int D>
+__global__ void __launch_bounds__(256) decode_bf16_kernel(DecodeArgs a) {
+    constexpr int KS = D / 32;   // MFMA k-steps over the head dim
+    constexpr int DB = D / 16;   // 16-row tiles of O^T
+    const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+    const int L = min(a.seq_lens ? a.seq_lens[b] : a.len, a.S_max);
+    const int chunk_start = split * a.chunk;
+    if (chunk_start >= L) return;
+    const int chunk_end = min(L, chunk_start + a.chunk);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int c = lane & 15, g = lane >> 4;
+
+    // Q^T operands: column c = query head kvh*n_rep + c (zero beyond n_rep)
+    bf16x8_t qf[KS];
+    {
+        const uint16_t* qrow = (const uint16_t*)a.q + (int64_t)b * a.sq_b + (int64_t)(kvh * a.n_rep + min(c, a.n_rep - 1)) * a.sq_h;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            uint4 w = *(const uint4*)(qrow + 32 * ks + 8 * g);
+            if (c >= a.n_rep) w = uint4{0, 0, 0, 0};
+            qf[ks] = __builtin_bit_cast(bf16x8_t, w);
+        }
+    }
+    const uint16_t* Kp = (const uint16_t*)a.k + ((int64_t)b * a.Hkv + kvh) * a.S * D;
+    const uint16_t* Vp = (const uint16_t*)a.v + ((int64_t)b * a.Hkv + kvh) * a.S * D;
+    const int krow = 16 * (c >> 2) + (c & 3);  // this lane's A-operand row: key offset before + 4*jj
+
+    f32x4_t acc[DB];
+#pragma unroll
+    for (int i = 0; i < DB; ++i) acc[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+
+    for (int kbase = chunk_start + wave * kGroup; kbase < chunk_end; kbase += kWaves * kGroup) {
+        // ---- loads: K rows (A operands of S^T), V^T blocks (A operands of O^T)
+        uint4 kf[4][KS];
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            const uint16_t* kr = Kp + (int64_t)(kbase + krow + 4 * jj) * D + 8 * g;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) kf[jj][ks] = *(const uint4*)(kr + 32 * ks);
+        }
+        uint4 vf[DB][2];
+        {
+            const uint16_t* vb = Vp + ((int64_t)(kbase / kVBlkBf16 + 2 * g) * D + c) * kVBlkBf16;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+                    vf[db][t] = *(const uint4*)(vb + ((int64_t)t * D + 16 * db) * kVBlkBf16);
+        }
+        // ---- S^T
+        f32x4_t s[4];
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            s[jj] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+                s[jj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kf[jj][ks]), qf[ks], s[jj], 0, 0, 0);
+        }
+        const bool tail = kbase + kGroup > chunk_end;
+        float mloc = -INFINITY;
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                float t = s[jj][v] * a.scale_log2;
+                if (tail && kbase + 16 * g + 4 * jj + v >= chunk_end) t = -INFINITY;
+                s[jj][v] = t;
+                mloc = fmaxf(mloc, t);
+            }
+        mloc = wave_max_over_groups(mloc);
+        const float m_new = fmaxf(m, mloc);  // finite: the group holds at least one valid key
+        const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+        float lsum = 0.f;
+        uint32_t pw[2][4];
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            float p0 = __builtin_amdgcn_exp2f(s[jj][0] - m_new), p1 = __builtin_amdgcn_exp2f(s[jj][1] - m_new);
+            float p2 = __builtin_amdgcn_exp2f(s[jj][2] - m_new), p3 = __builtin_amdgcn_exp2f(s[jj][3] - m_new);
+            lsum += (p0 + p1) + (p2 + p3);
+            pw[jj >> 1][2 * (jj & 1)] = pack_bf16x2(p0, p1);
+            pw[jj >> 1][2 * (jj & 1) + 1] = pack_bf16x2(p2, p3);
+        }
+        l = l * alpha + lsum;
+        m = m_new;
+        if (tail) {
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int t = 0; t < 2; ++t) vf[db][t] = mask_tail_u16x8(vf[db][t], chunk_end - (kbase + 16 * g + 8 * t));
+        }
+        // ---- O^T
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+            acc[db] *= alpha;
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                bf16x8_t pf = __builtin_bit_cast(bf16x8_t, uint4{pw[t][0], pw[t][1], pw[t][2], pw[t][3]});
+                acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vf[db][t]), pf, acc[db], 0, 0, 0);
+            }
+        }
+    }
+    l = wave_sum_over_groups(l);
+
+    // ---- combine the four wavefronts through LDS, write one partial per (b, head, split)
+    __shared__ float sm_o[kWaves][16][D + 4];
+    __shared__ float sm_m[kWaves][16], sm_l[kWaves][16];
+    if (c < a.n_rep) {
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) sm_o[wave][c][16 * db + 4 * g + v] = acc[db][v];
+        if (g == 0) {
+            sm_m[wave][c] = m;
+            sm_l[wave][c] = l;
+        }
+    }
+    __syncthreads();
+    for (int i = tid; i < a.n_rep * D; i += 256) {
+        const int hc = i / D, d = i % D;
+        float mm = sm_m[0][hc];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) mm = fmaxf(mm, sm_m[w][hc]);
+        float o = 0.f, ll = 0.f;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            const float f = __builtin_amdgcn_exp2f(sm_m[w][hc] - mm);
+            o += f * sm_o[w][hc][d];
+            ll += f * sm_l[w][hc];
+        }
+        const int64_t row = ((int64_t)b * a.Hq + kvh * a.n_rep + hc) * a.max_splits + split;
+        a.ws_o[row * D + d] = o;
+        if (d == 0) {
+            a.ws_ml[row * 2] = mm;
+            a.ws_ml[row * 2 + 1] = ll;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Q8_0 cache: int8 payload widened to fp16 in registers and scaled, fp16 MFMA.
+// ---------------------------------------------------------------------------------------------
+// 4 int8 (one dword, two's complement) -> 4 fp16 holding the same integers.  x ^ 0x80 is the
+// biased value u = q + 128; 0x6400 | u is the fp16 1024 + u; subtracting 1152 is exact.
+__device__ inline void i8x4_to_f16x4(uint32_t w, f16x2_t& lo, f16x2_t& hi) {
+    const uint32_t x = w ^ 0x80808080u;
+    const uint32_t a = __builtin_amdgcn_perm(0x64646464u, x, 0x04010400u);
+    const uint32_t bq = __builtin_amdgcn_perm(0x64646464u, x, 0x04030402u);
+    const f16x2_t bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+    lo = __builtin_bit_cast(f16x2_t, a) - bias;
+    hi = __builtin_bit_cast(f16x2_t, bq) - bias;
+}
+__device__ inline uint32_t f16x2_bits(f16x2_t v) { return __builtin_bit_cast(uint32_t, v); }
+
+template <int D>
+__global__ void __launch_bounds__(256) decode_q8_kernel(DecodeArgs a) {
+    constexpr int KS = D / 32;
+    constexpr int DB = D / 16;
+    constexpr int NH = D / 64;  // 16-byte K loads per row per lane
+    constexpr int NQ = D / kQBlock;
+    const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+    const int L = min(a.seq_lens ? a.seq_lens[b] : a.len, a.S_max);
+    const int chunk_start = split * a.chunk;
+    if (chunk_start >= L) return;
+    const int chunk_end = min(L, chunk_start + a.chunk);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int c = lane & 15, g = lane >> 4;
+
+    // Q^T operands in fp16.  Contraction slot (ks, g, e) is head-dim index
+    // 64*(ks/2) + 16*g + 8*(ks%2) + e, so that one 16-byte K load (16 int8) feeds two k-steps.
+    f16x8_t qf[KS];
+    {
+        const uint16_t* qrow = (const uint16_t*)a.q + (int64_t)b * a.sq_b + (int64_t)(kvh * a.n_rep + min(c, a.n_rep - 1)) * a.sq_h;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            uint4 w = *(const uint4*)(qrow + 64 * (ks >> 1) + 16 * g + 8 * (ks & 1));
+            const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float lo = bf16_bits_to_f32((uint16_t)(ww[i] & 0xFFFFu)), hi = bf16_bits_to_f32((uint16_t)(ww[i] >> 16));
+                lo = fminf(fmaxf(lo, -65504.f), 65504.f);
+                hi = fminf(fmaxf(hi, -65504.f), 65504.f);
+                if (c >= a.n_rep) lo = hi = 0.f;
+                qf[ks][2 * i] = (_Float16)lo;
+                qf[ks][2 * i + 1] = (_Float16)hi;
+            }
+        }
+    }
+    const int64_t head = (int64_t)b * a.Hkv + kvh;
+    const int8_t* Kp = (const int8_t*)a.k + head * a.S * D;
+    const int8_t* Vp = (const int8_t*)a.v + head * a.S * D;
+    const uint16_t* KSp = (const uint16_t*)a.k_scale + head * a.S * NQ;
+    const uint16_t* VSp = (const uint16_t*)a.v_scale + head * a.S * NQ;
+    const int krow = 16 * (c >> 2) + (c & 3);
+
+    f32x4_t acc[DB];
+#pragma unroll
+    for (int i = 0; i < DB; ++i) acc[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+
+    for (int kbase = chunk_start + wave * kGroup; kbase < chunk_end; kbase += kWaves * kGroup) {
+        const bool tail = kbase + kGroup > chunk_end;
+        // ---- loads
+        uint4 kq[4][NH];
+        uint16_t ksc[4][NH];
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            const int64_t key = kbase + krow + 4 * jj;
+#pragma unroll
+            for (int h = 0; h < NH; ++h) {
+                kq[jj][h] = *(const uint4*)(Kp + key * D + 64 * h + 16 * g);
+                ksc[jj][h] = KSp[key * NQ + 2 * h + (g >> 1)];
+            }
+        }
+        uint4 vq[DB];
+        uint4 vsc[NQ][2];
+        {
+            const int64_t blk = kbase / kVBlkQ8 + g;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) vq[db] = *(const uint4*)(Vp + (blk * D + 16 * db + c) * kVBlkQ8);
+#pragma unroll
+            for (int qb = 0; qb < NQ; ++qb) {
+                const uint4* sp = (const uint4*)(VSp + (blk * NQ + qb) * kVBlkQ8);
+                vsc[qb][0] = sp[0];
+                vsc[qb][1] = sp[1];
+            }
+        }
+        // ---- S^T
+        f32x4_t s[4];
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            s[jj] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int h = 0; h < NH; ++h) {
+                const _Float16 sc = __builtin_bit_cast(_Float16, ksc[jj][h]);
+                const f16x2_t sc2 = {sc, sc};
+                const uint32_t w[4] = {kq[jj][h].x, kq[jj][h].y, kq[jj][h].z, kq[jj][h].w};
+                uint32_t o[8];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    f16x2_t lo, hi;
+                    i8x4_to_f16x4(w[i], lo, hi);
+                    o[2 * i] = f16x2_bits(lo * sc2);
+                    o[2 * i + 1] = f16x2_bits(hi * sc2);
+                }
+                f16x8_t k0 = __builtin_bit_cast(f16x8_t, uint4{o[0], o[1], o[2], o[3]});
+                f16x8_t k1 = __builtin_bit_cast(f16x8_t, uint4{o[4], o[5], o[6], o[7]});
+                s[jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(k0, qf[2 * h], s[jj], 0, 0, 0);
+                s[jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(k1, qf[2 * h + 1], s[jj], 0, 0, 0);
+            }
+        }
+        float mloc = -INFINITY;
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                float t = s[jj][v] * a.scale_log2;
+                if (tail && kbase + 16 * g + 4 * jj + v >= chunk_end) t = -INFINITY;
+                s[jj][v] = t;
+                mloc = fmaxf(mloc, t);
+            }
+        mloc = wave_max_over_groups(mloc);
+        const float m_new = fmaxf(m, mloc);
+        const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+        float lsum = 0.f;
+        f16x8_t pf[2];
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const float p = __builtin_amdgcn_exp2f(s[jj][v] - m_new);
+                lsum += p;
+                pf[jj >> 1][4 * (jj & 1) + v] = (_Float16)p;
+            }
+        l = l * alpha + lsum;
+        m = m_new;
+        // ---- O^T: dequantise V^T operands (16 tokens of one d per lane; per-token scales)
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+            acc[db] *= alpha;
+            const int qb = (16 * db) / kQBlock;
+            const uint32_t w[4] = {vq[db].x, vq[db].y, vq[db].z, vq[db].w};
+            const uint32_t scw[8] = {vsc[qb][0].x, vsc[qb][0].y, vsc[qb][0].z, vsc[qb][0].w,
+                                     vsc[qb][1].x, vsc[qb][1].y, vsc[qb][1].z, vsc[qb][1].w};
+            uint32_t o[8];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                f16x2_t lo, hi;
+                i8x4_to_f16x4(w[i], lo, hi);
+                o[2 * i] = f16x2_bits(lo * __builtin_bit_cast(f16x2_t, scw[2 * i]));
+                o[2 * i + 1] = f16x2_bits(hi * __builtin_bit_cast(f16x2_t, scw[2 * i + 1]));
+            }
+            uint4 v0 = uint4{o[0], o[1], o[2], o[3]}, v1 = uint4{o[4], o[5], o[6], o[7]};
+            if (tail) {
+                v0 = mask_tail_u16x8(v0, chunk_end - (kbase + 16 * g));
+                v1 = mask_tail_u16x8(v1, chunk_end - (kbase + 16 * g + 8));
+            }
+            acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, v0), pf[0], acc[db], 0, 0, 0);
+            acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, v1), pf[1], acc[db], 0, 0, 0);
+        }
+    }
+    l = wave_sum_over_groups(l);
+
+    __shared__ float sm_o[kWaves][16][D + 4];
+    __shared__ float sm_m[kWaves][16], sm_l[kWaves][16];
+    if (c < a.n_rep) {
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) sm_o[wave][c][16 * db + 4 * g + v] = acc[db][v];
+        if (g == 0) {
+            sm_m[wave][c] = m;
+            sm_l[wave][c] = l;
+        }
+    }
+    __syncthreads();
+    for (int i = tid; i < a.n_rep * D; i += 256) {
+        const int hc = i / D, d = i % D;
+        float mm = sm_m[0][hc];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) mm = fmaxf(mm, sm_m[w][hc]);
+        float o = 0.f, ll = 0.f;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            const float f = __builtin_amdgcn_exp2f(sm_m[w][hc] - mm);
+            o += f * sm_o[w][hc][d];
+            ll += f * sm_l[w][hc];
+        }
+        const int64_t row = ((int64_t)b * a.Hq + kvh * a.n_rep + hc) * a.max_splits + split;
+        a.ws_o[row * D + d] = o;
+        if (d == 0) {
+            a.ws_ml[row * 2] = mm;
+            a.ws_ml[row * 2 + 1] = ll;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// fp32 cache in the reference's own layout: plain fp32 arithmetic, one workgroup per
+// (batch row, query head, split).  Correctness path for callers that keep the reference's fp32 cache.
+// ---------------------------------------------------------------------------------------------
+template <int MAXD>
+__global__ void __launch_bounds__(256) decode_f32_kernel(DecodeArgs a, int D) {
+    const int split = blockIdx.x, hq = blockIdx.y, b = blockIdx.z;
+    const int L = min(a.seq_lens ? a.seq_lens[b] : a.len, a.S_max);
+    const int chunk_start = split * a.chunk;
+    if (chunk_start >= L) return;
+    const int chunk_end = min(L, chunk_start + a.chunk);
+    const int n = chunk_end - chunk_start;
+    const int kvh = hq / a.n_rep;
+    const int tid = threadIdx.x;
+
+    extern __shared__ float smem[];
+    float* sq = smem;              // [MAXD]
+    float* sp = smem + MAXD;       // [chunk]
+    float* red = sp + a.chunk;     // [256]
+    const float* qrow = (const float*)a.q + (int64_t)b * a.sq_b + (int64_t)hq * a.sq_h;
+    for (int d = tid; d < D; d += 256) sq[d] = qrow[d];
+    __syncthreads();
+    const float* Kp = (const float*)a.k + (((int64_t)b * a.Hkv + kvh) * a.S + chunk_start) * D;
+    const float* Vp = (const float*)a.v + (((int64_t)b * a.Hkv + kvh) * a.S + chunk_start) * D;
+    float mloc = -INFINITY;
+    for (int j = tid; j < n; j += 256) {
+        const float4* kr = (const float4*)(Kp + (int64_t)j * D);
+        float s = 0.f;
+        for (int d4 = 0; d4 < D / 4; ++d4) {
+            const float4 kk = kr[d4];
+            s = fmaf(sq[4 * d4], kk.x, s);
+            s = fmaf(sq[4 * d4 + 1], kk.y, s);
+            s = fmaf(sq[4 * d4 + 2], kk.z, s);
+            s = fmaf(sq[4 * d4 + 3], kk.w, s);
+        }
+        s *= a.scale_log2;
+        sp[j] = s;
+        mloc = fmaxf(mloc, s);
+    }
+    red[tid] = mloc;
+    __syncthreads();
+    for (int st = 128; st > 0; st >>= 1) {
+        if (tid < st) red[tid] = fmaxf(red[tid], red[tid + st]);
+        __syncthreads();
+    }
+    const float m = red[0];
+    __syncthreads();
+    float lloc = 0.f;
+    for (int j = tid; j < n; j += 256) {
+        const float p = exp2f(sp[j] - m);
+        sp[j] = p;
+        lloc += p;
+    }
+    red[tid] = lloc;
+    __syncthreads();
+    for (int st = 128; st > 0; st >>= 1) {
+        if (tid < st) red[tid] += red[tid + st];
+        __syncthreads();
+    }
+    const float l = red[0];
+    __syncthreads();
+    // PV: thread (d, part) sums keys part, part+P, ...; P = 256 / D' where D' = D rounded up to a power of two
+    int Dp = 1;
+    while (Dp < D) Dp <<= 1;
+    const int P = 256 / Dp > 0 ? 256 / Dp : 1;
+    const int d = tid % Dp, part = tid / Dp;
+    float o = 0.f;
+    if (d < D && part < P)
+        for (int j = part; j < n; j += P) o = fmaf(sp[j], Vp[(int64_t)j * D + d], o);
+    __syncthreads();
+    red[tid] = o;
+    __syncthreads();
+    if (tid < D && tid < Dp) {
+        float t = 0.f;
+        for (int p = 0; p < P; ++p) t += red[p * Dp + tid];
+        const int64_t row = ((int64_t)b * a.Hq + hq) * a.max_splits + split;
+        a.ws_o[row * D + tid] = t;
+        if (tid == 0) {
+            a.ws_ml[row * 2] = m;
+            a.ws_ml[row * 2 + 1] = l;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// combine: out[b][h][:] = sum_s w_s O_s / sum_s w_s l_s, w_s = 2^(m_s - max m); fixed order.
+// ---------------------------------------------------------------------------------------------
+template <typename OutT>
+__global__ void __launch_bounds__(256) decode_combine_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
+                                                             const int32_t* __restrict__ seq_lens, int32_t len, int32_t chunk,
+                                                             int32_t max_splits, int32_t Hq, int32_t D, OutT* __restrict__ out,
+                                                             int64_t so_b, int64_t so_h, int32_t S_max) {
+    const int hq = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+    const int L = min(seq_lens ? seq_lens[b] : len, S_max);
+    const int ns = min((L + chunk - 1) / chunk, max_splits);
+    const int64_t row0 = ((int64_t)b * Hq + hq) * max_splits;
+    float M = -INFINITY;
+    for (int s = 0; s < ns; ++s) M = fmaxf(M, ws_ml[(row0 + s) * 2]);
+    float o = 0.f, l = 0.f;
+    for (int s = 0; s < ns; ++s) {
+        const float w = exp2f(ws_ml[(row0 + s) * 2] - M);
+        l += w * ws_ml[(row0 + s) * 2 + 1];
+        if (d < D) o += w * ws_o[(row0 + s) * D + d];
+    }
+    if (d < D) {
+        const float r = ns > 0 ? o / l : 0.f;
+        OutT* p = out + (int64_t)b * so_b + (int64_t)hq * so_h + d;
+        if constexpr (sizeof(OutT) == 4) *p = r;
+        else *p = f32_to_bf16_bits(r);
+    }
+}
+
+int device_cu_count() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            cus = n;
+        else
+            cus = 256;
+    }
+    return cus;
+}
+
+// Tokens per split.  Small enough that the (ragged) work spreads over all CUs with a short tail,
+// large enough that partials stay a few percent of the KV bytes.  Workspace sizing assumes >= 256.
+int pick_chunk(int64_t B, int64_t Hkv, int64_t max_len) {
+    static int forced = -1;
+    if (forced < 0) {
+        const char* e = getenv("VSP_DECODE_CHUNK");
+        forced = e ? atoi(e) : 0;
+        if (forced != 0 && (forced < 256 || forced % 256 != 0 || forced > 8192)) forced = 0;
+    }
+    if (forced > 0) return forced;
+    const int64_t want = 24LL * device_cu_count();
+    for (int chunk : {1024, 512}) {
+        if (B * Hkv * ceil_div(max_len, chunk) >= want) return chunk;
+    }
+    return 256;
+}
+
+}  // namespace
+}  // namespace vsp
+
+using namespace vsp;
+
+extern "C" {
+
+size_t vsp_attn_decode_workspace_bytes(int32_t B, int32_t Hq, int32_t D, int32_t max_len) {
+    if (B <= 0 || Hq <= 0 || D <= 0 || max_len <= 0) return 0;
+    const int64_t splits = ceil_div(max_len, 256);
+    return (size_t)((int64_t)B * Hq * splits * (D + 2) * 4);
+}
+
+int vsp_attn_decode(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, int32_t max_len,
+                    vsp_tensor* out, float scale, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!q || !out) return VSP_ERR_NULL;
+    int rc = check_kv_cache(cache);
+    if (rc != VSP_OK) return rc;
+    if (q->ndim != 4 || out->ndim != 4) return VSP_ERR_NDIM;
+    const int64_t B = q->shape[0], Hq = q->shape[1], T = q->shape[2], D = q->shape[3];
+    if (T != 1 || B != cache->B || D != cache->D) return VSP_ERR_SHAPE;
+    for (int i = 0; i < 4; ++i)
+        if (out->shape[i] != q->shape[i]) return VSP_ERR_SHAPE;
+    if (cache->Hkv <= 0 || Hq <= 0 || Hq % cache->Hkv != 0) return VSP_ERR_GQA_HEADS;
+    const int n_rep = (int)(Hq / cache->Hkv);
+    const int want_dtype = cache->format == VSP_KV_F32 ? VSP_F32 : VSP_BF16;
+    if (q->dtype != out->dtype) return VSP_ERR_DTYPE;
+    if (q->dtype != want_dtype) return VSP_ERR_UNSUPPORTED;
+    if (cache->format != VSP_KV_F32 && n_rep > 16) return VSP_ERR_UNSUPPORTED;
+    if (cache->format == VSP_KV_F32 && D > 256) return VSP_ERR_UNSUPPORTED;
+    if (B == 0) return VSP_OK;
+    if (!q->data || !out->data) return VSP_ERR_NULL;
+    if (q->stride[3] != 1 || out->stride[3] != 1) return VSP_ERR_STRIDE;
+    const int esz = q->dtype == VSP_F32 ? 4 : 2;
+    if (!is_aligned16(q->data) || (q->stride[0] * esz) % 16 || (q->stride[1] * esz) % 16) return VSP_ERR_ALIGN;
+    if (max_len < 0 || max_len > cache->S_max) return VSP_ERR_ARG;
+    if (max_len == 0) max_len = seq_lens ? cache->S_max : cache->len;
+    hipStream_t st = (hipStream_t)stream;
+
+    const int chunk = max_len > 0 ? pick_chunk(B, cache->Hkv, max_len) : 256;
+    const int max_splits = max_len > 0 ? (int)ceil_div(max_len, chunk) : 1;
+    const size_t need = (size_t)(B * Hq * max_splits * (D + 2) * 4);
+    if (max_len > 0) {
+        if (!workspace || workspace_bytes < need) return VSP_ERR_WORKSPACE;
+        if (!is_aligned16(workspace)) return VSP_ERR_ALIGN;
+    }
+    DecodeArgs a;
+    a.q = q->data;
+    a.sq_b = q->stride[0];
+    a.sq_h = q->stride[1];
+    a.k = cache->k;
+    a.v = cache->v;
+    a.k_scale = cache->k_scale;
+    a.v_scale = cache->v_scale;
+    a.seq_lens = seq_lens;
+    a.len = cache->len;
+    a.Hq = (int)Hq;
+    a.Hkv = cache->Hkv;
+    a.n_rep = n_rep;
+    a.S = kv_s_pad(cache->format, cache->S_max);
+    a.S_max = cache->S_max;
+    a.chunk = chunk;
+    a.max_splits = max_splits;
+    a.scale_log2 = scale * kLog2e;
+    a.ws_o = (float*)workspace;
+    a.ws_ml = a.ws_o ? a.ws_o + (size_t)B * Hq * max_splits * D : nullptr;
+
+    if (max_len > 0) {
+        if (cache->format == VSP_KV_BF16) {
+            dim3 grid(max_splits, cache->Hkv, (unsigned)B);
+            if (D == 128) hipLaunchKernelGGL(decode_bf16_kernel<128>, grid, dim3(256), 0, st, a);
+            else hipLaunchKernelGGL(decode_bf16_kernel<64>, grid, dim3(256), 0, st, a);
+        } else if (cache->format == VSP_KV_Q8_0) {
+            dim3 grid(max_splits, cache->Hkv, (unsigned)B);
+            if (D == 128) hipLaunchKernelGGL(decode_q8_kernel<128>, grid, dim3(256), 0, st, a);
+            else hipLaunchKernelGGL(decode_q8_kernel<64>, grid, dim3(256), 0, st, a);
+        } else {
+            dim3 grid(max_splits, (unsigned)Hq, (unsigned)B);
+            const size_t smem = (256 + chunk + 256) * sizeof(float);
+            hipLaunchKernelGGL(decode_f32_kernel<256>, grid, dim3(256), smem, st, a, (int)D);
+        }
+        rc = check_launch();
+        if (rc != VSP_OK) return rc;
+    }
+    dim3 cgrid((unsigned)Hq, (unsigned)B);
+    const int cthreads = D <= 64 ? 64 : (D <= 128 ? 128 : 256);
+    if (out->dtype == VSP_F32)
+        hipLaunchKernelGGL(decode_combine_kernel<float>, cgrid, dim3(cthreads), 0, st, a.ws_o, a.ws_ml, seq_lens,
+                           max_len > 0 ? cache->len : 0, chunk, max_splits, (int)Hq, (int)D, (float*)out->data,
+                           out->stride[0], out->stride[1], cache->S_max);
+    else
+        hipLaunchKernelGGL(decode_combine_kernel<uint16_t>, cgrid, dim3(cthreads), 0, st, a.ws_o, a.ws_ml, seq_lens,
+                           max_len > 0 ? cache->len : 0, chunk, max_splits, (int)Hq, (int)D, (uint16_t*)out->data,
+                           out->stride[0], out->stride[1], cache->S_max);
+    return check_launch();
+}
+
+}  // extern "C"

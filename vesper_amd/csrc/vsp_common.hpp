@@ -1,0 +1,69 @@
+// Shared declarations of libvsp_attn.so: device helpers, argument checks, launch plumbing.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <string.h>
+
+#include "../../include/vsp_attn.h"
+
+namespace vsp {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+// fp32 -> bf16 bits, the reference's round-to-nearest-even
+// (include/vesper/core/half.h:162-173; src/ops/hip/cast.hip:28-34): no NaN special case.
+__host__ __device__ inline uint16_t f32_to_bf16_bits(float f) {
+    uint32_t bits;
+#if defined(__HIP_DEVICE_COMPILE__)
+    bits = __builtin_bit_cast(uint32_t, f);
+#else
+    memcpy(&bits, &f, sizeof bits);
+#endif
+    bits += 0x7FFFu + ((bits >> 16) & 1u);
+    return (uint16_t)(bits >> 16);
+}
+__host__ __device__ inline float bf16_bits_to_f32(uint16_t b) {
+    uint32_t bits = (uint32_t)b << 16;
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_bit_cast(float, bits);
+#else
+    float f;
+    memcpy(&f, &bits, sizeof f);
+    return f;
+#endif
+}
+// two fp32 -> packed bf16x2 (lo = a, hi = b), same rounding
+__device__ inline uint32_t pack_bf16x2(float a, float b) {
+    return (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(b) << 16);
+}
+
+// per-thread last HIP error text (vsp_last_hip_error)
+void set_hip_error(hipError_t e);
+int check_launch();  // VSP_OK or VSP_ERR_LAUNCH after a kernel launch
+
+inline bool is_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+inline int64_t ceil_div(int64_t x, int64_t m) { return (x + m - 1) / m; }
+
+// reference slice clamping for Slice(start, stop), step 1: src/ops/view_ops.cpp:270-316
+inline void slice_bounds(int64_t dim_size, int64_t start, int64_t stop, int64_t* out_start, int64_t* out_len) {
+    if (start < 0) start += dim_size;
+    if (stop < 0) stop += dim_size;
+    start = start < 0 ? 0 : (start > dim_size ? dim_size : start);
+    stop = stop < 0 ? 0 : (stop > dim_size ? dim_size : stop);
+    *out_start = start;
+    *out_len = start >= stop ? 0 : stop - start;
+}
+
+}  // namespace vsp
