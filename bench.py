@@ -1,0 +1,271 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on ONE MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|p4k|c3|c4|c5] [--no-cpu] [--no-extra]
+
+A "step" is one pass of the hot path over one batch of synthetic input that is already resident in
+HBM: one prefill launch (c2, p4k, c3) or one decode call = split-K kernel + combine kernel (c4, c5).
+Prints ONE JSON line.  `value` is the primary workload's throughput (BASELINE config 2 by default:
+causal GQA prefill bf16, B4, 32/8 heads, D128, N2048, in TFLOP/s of algorithmic causal FLOPs
+2*D*B*Hq*N*(N+1)); `other_workloads` carries the remaining BASELINE configs (decode in GB/s of
+algorithmic KV bytes).  `roofline` is for the primary workload's dominant kernel, timed with events
+on the launch stream; `cpu_baseline` is the reference's own CPU path (oracle/_ref, else the oracle
+port) timed on this host on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+HBM_PEAK_GBS = 8000.0
+
+WORKLOADS = {
+    "c2": dict(kind="prefill", B=4, Hq=32, Hkv=8, D=128, N=2048,
+               name="BASELINE config 2: causal GQA prefill bf16, B4, 32 q / 8 kv heads, D128, N2048"),
+    "p4k": dict(kind="prefill", B=2, Hq=32, Hkv=8, D=128, N=4096,
+                name="4k-context point: causal GQA prefill bf16, B2, 32 q / 8 kv heads, D128, N4096"),
+    "c3": dict(kind="prefill", B=1, Hq=32, Hkv=8, D=128, N=8192,
+               name="BASELINE config 3: causal GQA prefill bf16, B1, 32 q / 8 kv heads, D128, N8192"),
+    "c4": dict(kind="decode", fmt="bf16", B=32, Hq=32, Hkv=8, D=128, S=32768, lens=(1024, 32768, 4004),
+               name="BASELINE config 4: batched decode bf16 KV cache, B32, 32 q / 8 kv heads, D128, L~U[1024,32768]"),
+    "c5": dict(kind="decode", fmt="q8_0", B=16, Hq=64, Hkv=8, D=128, S=65536, lens=None,
+               name="BASELINE config 5: decode over Q8_0 KV cache, B16, 64 q / 8 kv heads, D128, L=65536"),
+}
+
+
+def prefill_flops(w):
+    return 2.0 * w["D"] * w["B"] * w["Hq"] * w["N"] * (w["N"] + 1)
+
+
+def decode_bytes(w, lens):
+    row = 2 * w["D"] if w["fmt"] == "bf16" else (w["D"] + 2 * (w["D"] // 32))  # bytes per (token, kv head) per plane
+    return float(sum(2 * w["Hkv"] * int(L) * row for L in lens) + w["B"] * w["Hq"] * w["D"] * (2 + 2))
+
+
+class Runner:
+    """Builds the device-resident inputs of one workload and exposes step()."""
+
+    def __init__(self, key, torch, va):
+        self.w = w = WORKLOADS[key]
+        self.key, self.torch, self.va = key, torch, va
+        dev = torch.device("cuda:0")
+        g = torch.Generator(device="cuda").manual_seed(1000 + sum(map(ord, key)))
+        if w["kind"] == "prefill":
+            B, Hq, Hkv, D, N = w["B"], w["Hq"], w["Hkv"], w["D"], w["N"]
+            mk = lambda h: (torch.randn(B, h, N, D, device=dev, generator=g) * 0.5).to(torch.bfloat16)
+            self.q, self.k, self.v = mk(Hq), mk(Hkv), mk(Hkv)
+            self.scale = 1.0 / math.sqrt(D)
+            self.work = prefill_flops(w)
+            self.unit, self.peak, self.bound = "TFLOP/s", MFMA_BF16_PEAK_TFLOPS, "mfma"
+            self.kernel = "prefill_bf16_kernel<128>"
+        else:
+            import numpy as np
+            B, Hq, Hkv, D, S = w["B"], w["Hq"], w["Hkv"], w["D"], w["S"]
+            if w["lens"]:
+                lo, hi, seed = w["lens"]
+                lens = np.random.default_rng(seed).integers(lo, hi + 1, size=B, dtype=np.int64).astype(np.int32)
+            else:
+                lens = np.full(B, S, np.int32)
+            self.lens = lens
+            self.cache = va.KVCache(B, Hkv, S, D, fmt=w["fmt"])
+            for b in range(B):  # fill through the append path, a batch row at a time (bounded fp32 temporaries)
+                kb = torch.randn(1, Hkv, S, D, device=dev, generator=g)
+                vb = torch.randn(1, Hkv, S, D, device=dev, generator=g)
+                self._append_row(b, kb, vb)
+                del kb, vb
+            self.cache.set_len(S)
+            self.seq_lens = torch.from_numpy(lens).to(dev)
+            self.q = torch.randn(B, Hq, 1, D, device=dev, generator=g).to(torch.bfloat16)
+            self.out = torch.empty_like(self.q)
+            self.scale = 1.0 / math.sqrt(D)
+            self.work = decode_bytes(w, lens)
+            self.unit, self.peak, self.bound = "GB/s", HBM_PEAK_GBS, "hbm"
+            self.kernel = "decode_bf16_kernel<128>" if w["fmt"] == "bf16" else "decode_q8_kernel<128>"
+            self.max_len = int(lens.max())
+
+    def _append_row(self, b, kb, vb):
+        """Append one batch row's K/V [1,Hkv,S,D] at position 0 of row b via per-sequence start positions."""
+        import ctypes as C
+        from vesper_amd import _ffi
+        from vesper_amd.api import _desc, _stream
+        c = self.cache._c
+        sub = _ffi.VspKVCache()
+        for f, _ in _ffi.VspKVCache._fields_:
+            setattr(sub, f, getattr(c, f))
+        # window: same planes offset to row b, batch 1
+        for plane, name in ((0, "k"), (1, "v"), (2, "k_scale"), (3, "v_scale")):
+            nbytes = _ffi.lib.vsp_kv_plane_bytes(c.format, 1, c.Hkv, c.S_max, c.D, plane)
+            base = getattr(c, name)
+            setattr(sub, name, (base + b * nbytes) if base else None)
+        sub.B = 1
+        dk, dv = _desc(kb), _desc(vb)
+        _ffi.check(_ffi.lib.vsp_kv_append(C.byref(sub), C.byref(dk), C.byref(dv), 0, None, _stream(kb)))
+
+    def step(self):
+        if self.w["kind"] == "prefill":
+            return self.va.flash_attention(self.q, self.k, self.v, self.scale, True)
+        return self.va.decode_attention(self.q, self.cache, seq_lens=self.seq_lens, max_len=self.max_len,
+                                        scale=self.scale, out=self.out)
+
+    def rate(self, seconds_per_step):
+        return self.work / seconds_per_step / (1e12 if self.unit == "TFLOP/s" else 1e9)
+
+
+def time_steps(torch, fn, steps, warmup):
+    """warmup untimed, then exactly `steps` steps: wall clock bracketed by synchronize, and device time
+    from events recorded on the launch stream around the same region."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / steps
+    dev = e0.elapsed_time(e1) * 1e-3 / steps
+    return wall, dev
+
+
+def cpu_baseline(key):
+    """The reference's CPU path on a bounded sample of the primary workload, one thread (the path is
+    single-threaded in the reference)."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import numpy as np
+    import _oracle as O
+    w = WORKLOADS[key]
+    use_ref = O.ref is not None
+    kind = "reference" if use_ref else "port"
+    rng = np.random.default_rng(1)
+    if w["kind"] == "prefill":
+        # sample: 8 query heads (2 kv groups) of one batch row at full N: repeat_kv + flash_attention, fp32
+        Hq_s, Hkv_s, N, D = 8, 2, w["N"], w["D"]
+        q = O.bf16_round(rng.standard_normal((1, Hq_s, N, D), dtype=np.float32) * 0.5)
+        k = O.bf16_round(rng.standard_normal((1, Hkv_s, N, D), dtype=np.float32) * 0.5)
+        v = O.bf16_round(rng.standard_normal((1, Hkv_s, N, D), dtype=np.float32) * 0.5)
+        scale = float(np.float32(1.0 / math.sqrt(D)))
+        t0 = time.perf_counter()
+        if use_ref:
+            kr, vr = O.ref_repeat_kv(k, 4), O.ref_repeat_kv(v, 4)
+            O.ref_flash_attention(q, kr, vr, scale, True)
+        else:
+            O.flash_attention(q, O.repeat_kv(k, 4), O.repeat_kv(v, 4), scale, True)
+        dt = time.perf_counter() - t0
+        flops = 2.0 * D * Hq_s * N * (N + 1)
+        return dict(value=flops / dt / 1e12, unit="TFLOP/s", cores=1, kind=kind,
+                    sample=f"1 batch row x {Hq_s} query heads ({Hkv_s} kv heads) of the workload at N={N}: "
+                           f"repeat_kv + flash_attention fp32, {dt:.1f} s; whole workload = x{w['B'] * w['Hq'] // Hq_s}",
+                    seconds=dt)
+    # decode sample: one sequence, one kv group, fp32 cache: repeat_kv + matmul/softmax/matmul branch
+    L, D, n_rep = 8192, w["D"], w["Hq"] // w["Hkv"]
+    q = rng.standard_normal((1, n_rep, 1, D), dtype=np.float32)
+    k = rng.standard_normal((1, 1, L, D), dtype=np.float32)
+    v = rng.standard_normal((1, 1, L, D), dtype=np.float32)
+    reps = 6
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        if use_ref:
+            O.ref_sdpa(q, O.ref_repeat_kv(k, n_rep), O.ref_repeat_kv(v, n_rep), False)
+        else:
+            O.sdpa(q, O.repeat_kv(k, n_rep), O.repeat_kv(v, n_rep), False)
+    dt = (time.perf_counter() - t0) / reps
+    row = 2 * D if w["fmt"] == "bf16" else D + 2 * (D // 32)
+    return dict(value=2 * L * row / dt / 1e9, unit="GB/s", cores=1, kind=kind,
+                sample=f"one sequence x one kv head ({n_rep} query heads), L={L}, fp32 cache as in the reference: "
+                       f"repeat_kv x2 + matmul/div/softmax/matmul, {dt * 1e3:.0f} ms per call x{reps}; "
+                       f"rate in the workload's algorithmic KV bytes",
+                seconds=dt * reps)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="only the primary workload")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch one 1 GiB read + 1 GiB write elementwise kernel (counter calibration for rocprofv3 --pmc)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path shards without communication over "
+              "batch and kv heads; no multi-GPU figure is produced). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import vesper_amd as va  # raises if the HIP library is missing: no fallback
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    props = torch.cuda.get_device_properties(0)
+
+    if args.copy_calibration:
+        src = torch.ones(1 << 28, dtype=torch.int32, device="cuda:0")
+        dst = torch.empty_like(src)
+        torch.add(src, 1, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
+
+    primary = Runner(args.workload, torch, va)
+    wall, dev = time_steps(torch, primary.step, args.steps, args.warmup)
+    value = primary.rate(wall)
+    achieved = primary.rate(dev)
+    result = {
+        "metric": "prefill attn TFLOP/s (% MFMA peak); decode attn HBM GB/s (% of 8 TB/s)",
+        "value": round(value, 3),
+        "unit": primary.unit,
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall * 1e3, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if primary.w.get("fmt", "bf16") == "bf16" else "q8_0 (int8 payload, fp16 MFMA)",
+        "data": "synthetic",
+        "config": {"workload": primary.w["name"], "key": args.workload,
+                   "algorithmic_work_per_step": primary.work,
+                   "work_unit": "FLOP" if primary.bound == "mfma" else "bytes"},
+        "roofline": {"bound": primary.bound, "achieved": round(achieved, 3), "peak": primary.peak,
+                     "unit": primary.unit, "frac": round(achieved / primary.peak, 4), "traffic": None,
+                     "kernel": primary.kernel, "kernel_ms": round(dev * 1e3, 5),
+                     "timing": "HIP events on the launch stream around the timed steps / steps"},
+        "device": {"name": props.name, "cus": props.multi_processor_count,
+                   "peak_used": f"{primary.peak} {primary.unit}"},
+    }
+    del primary
+    torch.cuda.empty_cache()
+
+    if not args.no_extra:
+        others = {}
+        for key in ("c2", "p4k", "c3", "c4", "c5"):
+            if key == args.workload:
+                continue
+            r = Runner(key, torch, va)
+            steps = max(10, args.steps // 2)
+            w_, d_ = time_steps(torch, r.step, steps, max(3, args.warmup // 2))
+            others[key] = {"workload": r.w["name"], "value": round(r.rate(w_), 3), "unit": r.unit,
+                           "ms_per_step": round(w_ * 1e3, 5), "kernel_ms": round(d_ * 1e3, 5),
+                           "roofline_frac": round(r.rate(d_) / r.peak, 4), "bound": r.bound, "steps": steps}
+            del r
+            torch.cuda.empty_cache()
+        result["other_workloads"] = others
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(args.workload)
+        result["cpu_baseline"]["host_cores_available"] = os.cpu_count()
+
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
