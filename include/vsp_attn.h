@@ -52,7 +52,7 @@ typedef enum {
     VSP_ERR_UNSUPPORTED = 33, /* dtype/format/head_dim combination the kernels do not implement */
     VSP_ERR_STRIDE = 34,      /* innermost stride != 1, or a stride the kernel cannot address */
     VSP_ERR_ALIGN = 35,       /* a base pointer or row pitch is not 16-byte aligned */
-    VSP_ERR_WORKSPACE = 36,   /* workspace missing or smaller than vsp_attn_workspace_bytes() */
+    VSP_ERR_WORKSPACE = 36,   /* workspace missing or smaller than vsp_attn_decode_workspace_bytes() */
     VSP_ERR_ARG = 37,         /* an argument is out of range (negative size, len > S_max, ...) */
     VSP_ERR_LAUNCH = 38       /* the HIP runtime rejected a launch (hipGetLastError text via vsp_last_hip_error) */
 } vsp_status;

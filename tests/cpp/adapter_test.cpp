@@ -1,0 +1,243 @@
+// Exercises the C++ mirror of the reference's operator surface (vesper_amd/csrc/adapter/vesper_adapter.hpp)
+// the way the reference's own assert-style tests exercise the original, with the CPU oracle as checker.
+//   adapter_test --cpu-only   host-side checks only (no GPU needed)
+//   adapter_test              everything (needs a GPU)
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "../../oracle/vsp_oracle.h"
+#include "../../vesper_amd/csrc/adapter/vesper_adapter.hpp"
+
+using namespace vesper_amd;
+
+static int g_fail = 0;
+#define CHECK(cond)                                                                  \
+    do {                                                                             \
+        if (!(cond)) {                                                               \
+            std::printf("  CHECK FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond);    \
+            ++g_fail;                                                                \
+        }                                                                            \
+    } while (0)
+
+template <class Ex, class F>
+static std::string thrown(F&& f) {
+    try {
+        f();
+    } catch (const Ex& e) {
+        return e.what();
+    } catch (...) {
+        return "<other exception type>";
+    }
+    return "<nothing thrown>";
+}
+
+static std::vector<float> randn(size_t n, uint64_t seed, float scale = 1.0f) {
+    std::vector<float> x(n);
+    uint64_t s = seed * 0x9E3779B97F4A7C15ull + 1;
+    auto next = [&]() {
+        s ^= s << 13;
+        s ^= s >> 7;
+        s ^= s << 17;
+        return (double)(s >> 11) / 9007199254740992.0;
+    };
+    for (size_t i = 0; i < n; i += 2) {
+        double u1 = next() + 1e-12, u2 = next();
+        double r = std::sqrt(-2.0 * std::log(u1));
+        x[i] = (float)(r * std::cos(6.283185307179586 * u2)) * scale;
+        if (i + 1 < n) x[i + 1] = (float)(r * std::sin(6.283185307179586 * u2)) * scale;
+    }
+    return x;
+}
+static std::vector<float> bf16_round(std::vector<float> x) {
+    for (auto& f : x) f = orc_bf16_to_f32(orc_f32_to_bf16(f));
+    return x;
+}
+static Tensor to_dev(const std::vector<float>& x, std::vector<int64_t> shape, DType dt) {
+    Tensor t = empty(shape, dt);
+    if (dt == DType::Float32) {
+        t.copy_from_host(x.data());
+    } else {
+        std::vector<uint16_t> b(x.size());
+        for (size_t i = 0; i < x.size(); ++i) b[i] = orc_f32_to_bf16(x[i]);
+        t.copy_from_host(b.data());
+    }
+    return t;
+}
+static std::vector<float> to_host(const Tensor& t) {
+    std::vector<float> out(t.numel());
+    if (t.dtype() == DType::Float32) {
+        t.copy_to_host(out.data());
+    } else {
+        std::vector<uint16_t> b(t.numel());
+        t.copy_to_host(b.data());
+        for (size_t i = 0; i < b.size(); ++i) out[i] = orc_bf16_to_f32(b[i]);
+    }
+    return out;
+}
+static double max_abs_diff(const std::vector<float>& a, const float* b, size_t n) {
+    double m = 0;
+    for (size_t i = 0; i < n; ++i) m = std::fmax(m, std::fabs((double)a[i] - (double)b[i]));
+    return m;
+}
+
+// ---- host-only -------------------------------------------------------------------------------------
+static void test_gqa_constructor_validation() {
+    std::printf("test_gqa_constructor_validation\n");
+    nn::GroupedQueryAttentionCore ok(64, 8, 2);
+    CHECK(ok.head_dim() == 8 && ok.num_rep() == 4 && std::fabs(ok.kv_cache_ratio() - 0.25f) < 1e-7f);
+    // src/nn/gqa_attention.cpp:47-57 messages, std::invalid_argument
+    CHECK(thrown<std::invalid_argument>([] { nn::GroupedQueryAttentionCore m(64, 8, 3); }) ==
+          "GroupedQueryAttention: num_heads (8) must be divisible by num_kv_heads (3)");
+    CHECK(thrown<std::invalid_argument>([] { nn::GroupedQueryAttentionCore m(60, 8, 2); }) ==
+          "GroupedQueryAttention: embed_dim (60) must be divisible by num_heads (8)");
+    CHECK(std::fabs(nn::GQAKVCache::memory_savings(32, 8) - 0.75f) < 1e-7f);
+    int64_t s, n;
+    vsp_slice_bounds(10, 8, 12, &s, &n);  // clamped like ops::index
+    CHECK(s == 8 && n == 2);
+    CHECK(vsp_f32_to_bf16(1.00390625f) == orc_f32_to_bf16(1.00390625f));
+}
+
+// ---- GPU -------------------------------------------------------------------------------------------
+static void test_kv_cache_basic() {  // reference tests/test_kv_cache.cpp:8-43
+    std::printf("test_kv_cache_basic\n");
+    const int B = 1, H = 1, S = 10, D = 4;
+    nn::KVCache cache(B, H, S, D, Device::HIP);
+    std::vector<float> ones(B * H * 2 * D, 1.0f), threes(B * H * 1 * D, 3.0f);
+    Tensor k1 = to_dev(ones, {B, H, 2, D}, DType::Float32);
+    auto kv1 = cache.update(k1, k1, 0);
+    CHECK(cache.current_seq_len() == 2);
+    CHECK(kv1.first.shape()[2] == 2);
+    Tensor k2 = to_dev(threes, {B, H, 1, D}, DType::Float32);
+    auto kv2 = cache.update(k2, k2, 2);
+    CHECK(cache.current_seq_len() == 3);
+    CHECK(kv2.first.shape()[2] == 3);
+    CHECK((kv2.first.strides() == std::vector<int64_t>{H * S * D, S * D, D, 1}) && kv2.first.offset() == 0);
+    auto host = to_host(kv2.first);
+    CHECK(host[2 * D] == 3.0f && host[0] == 1.0f && host[D] == 1.0f);
+    CHECK(cache.get_max_seq_len() == 10);
+    // overflow: the reference clamps the slot and copy_from throws
+    CHECK(thrown<std::runtime_error>([&] { cache.update(k1, k1, 9); }) == "copy_from: element count mismatch.");
+    CHECK(cache.current_seq_len() == 3);
+    cache.reset();
+    CHECK(cache.current_seq_len() == 0);
+}
+
+static void test_flash_attention_against_oracle() {
+    std::printf("test_flash_attention_against_oracle\n");
+    const int64_t B = 2, H = 4, N = 96, D = 64;
+    const float scale = 1.0f / std::sqrt((float)D);
+    auto q = randn(B * H * N * D, 1), k = randn(B * H * N * D, 2), v = randn(B * H * N * D, 3);
+    std::vector<float> want(q.size()), lse(B * H * N);
+    for (int causal = 0; causal < 2; ++causal) {
+        orc_flash_attention_f32(q.data(), k.data(), v.data(), want.data(), lse.data(), B, H, N, D, scale, causal);
+        Tensor out = ops::flash_attention(to_dev(q, {B, H, N, D}, DType::Float32), to_dev(k, {B, H, N, D}, DType::Float32),
+                                          to_dev(v, {B, H, N, D}, DType::Float32), scale, causal != 0);
+        CHECK(max_abs_diff(to_host(out), want.data(), want.size()) < 1e-4);
+        auto qb = bf16_round(q), kb = bf16_round(k), vb = bf16_round(v);
+        orc_flash_attention_f32(qb.data(), kb.data(), vb.data(), want.data(), lse.data(), B, H, N, D, scale, causal);
+        Tensor outb = ops::flash_attention(to_dev(qb, {B, H, N, D}, DType::BFloat16), to_dev(kb, {B, H, N, D}, DType::BFloat16),
+                                           to_dev(vb, {B, H, N, D}, DType::BFloat16), scale, causal != 0);
+        CHECK(max_abs_diff(to_host(outb), want.data(), want.size()) < 2e-2);
+    }
+    // the reference's validation messages (src/ops/flash_attention.cpp:45-59)
+    Tensor a = empty({1, 2, 4, 64}, DType::Float32), b = empty({1, 2, 5, 64}, DType::Float32), c3 = empty({2, 4, 64}, DType::Float32);
+    CHECK(thrown<std::runtime_error>([&] { ops::flash_attention(c3, c3, c3, 1.f); }) == "flash_attention: inputs must be 4D [B, H, N, D]");
+    CHECK(thrown<std::runtime_error>([&] { ops::flash_attention(a, b, a, 1.f); }) == "flash_attention: Q, K, V must have same shape");
+    CHECK(thrown<std::runtime_error>([&] { ops::flash_attention(a, a, empty({1, 2, 4, 64}, DType::BFloat16), 1.f); }) ==
+          "flash_attention: Q, K, V must have same dtype");
+    CHECK(thrown<std::runtime_error>([&] { ops::flash_attention(a, a, a, 1.f, true, 1.0f); }) == "flash_attention: dropout_p must be in [0, 1)");
+}
+
+template <typename CacheT>
+static void run_cached_generation(KVFormat fmt, DType dt, double tol, const char* name) {
+    // reference tests/test_kv_cache_chapter33.cpp:66-188 and tests/test_gqa_chapter33.cpp:236-271 (intent):
+    // prefill 8 tokens through the cache, then decode token by token; every step equals the causal full forward.
+    std::printf("test_cached_generation[%s]\n", name);
+    const int64_t B = 2, Hq = 8, Hkv = 2, D = 64, T0 = 8, steps = 5, N = T0 + steps, S_max = 32;
+    nn::GroupedQueryAttentionCore attn(Hq * D, Hq, Hkv);
+    auto q = randn(B * Hq * N * D, 11, 0.5f), k = randn(B * Hkv * N * D, 12, 0.5f), v = randn(B * Hkv * N * D, 13, 0.5f);
+    if (dt == DType::BFloat16) q = bf16_round(q), k = bf16_round(k), v = bf16_round(v);
+    std::vector<float> kq = k, vq = v;
+    if (fmt == KVFormat::Q8_0) {  // the oracle attends over what the cache holds: the dequantised rows
+        std::vector<uint16_t> d(k.size() / 32);
+        std::vector<int8_t> qs(k.size());
+        orc_q8_0_quantize_row(k.data(), (int64_t)k.size(), d.data(), qs.data());
+        orc_q8_0_dequantize_row(d.data(), qs.data(), (int64_t)k.size(), kq.data());
+        orc_q8_0_quantize_row(v.data(), (int64_t)v.size(), d.data(), qs.data());
+        orc_q8_0_dequantize_row(d.data(), qs.data(), (int64_t)v.size(), vq.data());
+    }
+    // oracle: full causal GQA attention over all N tokens (matmul/softmax branch, N < 512)
+    std::vector<float> want(q.size());
+    int64_t st[4] = {Hkv * N * D, N * D, D, 1};
+    CHECK(orc_gqa_attention_f32(q.data(), kq.data(), st, vq.data(), st, want.data(), B, Hq, N, N, D, Hq / Hkv, 1) == 0);
+    auto slice = [&](const std::vector<float>& x, int64_t H, int64_t t0, int64_t t1) {
+        std::vector<float> out((size_t)(B * H * (t1 - t0) * D));
+        for (int64_t b = 0; b < B; ++b)
+            for (int64_t h = 0; h < H; ++h)
+                for (int64_t t = t0; t < t1; ++t)
+                    std::memcpy(&out[(size_t)(((b * H + h) * (t1 - t0) + (t - t0)) * D)], &x[(size_t)(((b * H + h) * N + t) * D)], D * sizeof(float));
+        return out;
+    };
+    CacheT cache(B, Hkv, S_max, D, Device::HIP, fmt);
+    auto step = [&](int64_t t0, int64_t t1) {
+        Tensor tq = to_dev(slice(q, Hq, t0, t1), {B, Hq, t1 - t0, D}, dt);
+        Tensor tk = to_dev(slice(k, Hkv, t0, t1), {B, Hkv, t1 - t0, D}, dt);
+        Tensor tv = to_dev(slice(v, Hkv, t0, t1), {B, Hkv, t1 - t0, D}, dt);
+        Tensor out = attn.forward(tq, tk, tv, &cache, t0);
+        auto got = to_host(out), w = slice(want, Hq, t0, t1);
+        double err = max_abs_diff(got, w.data(), w.size());
+        if (!(err < tol)) std::printf("  step [%ld,%ld): max-abs %.3g\n", (long)t0, (long)t1, err);
+        CHECK(err < tol);
+        CHECK((int64_t)cache.current_seq_len() == t1);
+    };
+    step(0, T0);
+    for (int64_t t = T0; t < N; ++t) step(t, t + 1);
+}
+
+static void test_sdpa_routing() {
+    std::printf("test_sdpa_routing\n");
+    const int64_t B = 1, H = 2, D = 64;
+    // cross shapes, non-causal (reference tests/test_attention_chapter32.cpp:135-162)
+    auto q = randn(B * H * 16 * D, 21), k = randn(B * H * 40 * D, 22), v = randn(B * H * 40 * D, 23);
+    std::vector<float> want(q.size());
+    orc_sdpa_f32(q.data(), k.data(), v.data(), want.data(), B, H, 16, 40, D, 0);
+    Tensor out = nn::functional::scaled_dot_product_attention(to_dev(q, {B, H, 16, D}, DType::Float32), to_dev(k, {B, H, 40, D}, DType::Float32),
+                                                              to_dev(v, {B, H, 40, D}, DType::Float32), false);
+    CHECK(max_abs_diff(to_host(out), want.data(), want.size()) < 1e-4);
+    // causal with T != L does not broadcast in the reference
+    CHECK(thrown<std::runtime_error>([&] {
+              nn::functional::scaled_dot_product_attention(to_dev(q, {B, H, 16, D}, DType::Float32), to_dev(k, {B, H, 40, D}, DType::Float32),
+                                                           to_dev(v, {B, H, 40, D}, DType::Float32), true);
+          }) == "causal mask [T, T] cannot be broadcast onto scores [T, L]");
+    // repeat_kv head map, reference tests/test_gqa_chapter33.cpp:76-118: constant V per kv head
+    std::vector<float> vv(B * 2 * 8 * D);
+    for (size_t i = 0; i < vv.size(); ++i) vv[i] = i < vv.size() / 2 ? 1.0f : 3.0f;
+    auto q8 = randn(B * 8 * 8 * D, 24), k8 = randn(B * 2 * 8 * D, 25);
+    Tensor o8 = nn::functional::scaled_dot_product_attention(to_dev(q8, {B, 8, 8, D}, DType::Float32),
+                                                             ops::repeat_kv(to_dev(k8, {B, 2, 8, D}, DType::Float32), 4),
+                                                             ops::repeat_kv(to_dev(vv, {B, 2, 8, D}, DType::Float32), 4), true);
+    auto h8 = to_host(o8);
+    bool ok = true;
+    for (int64_t h = 0; h < 8; ++h)
+        for (int64_t i = 0; i < 8 * D; ++i) ok = ok && std::fabs(h8[(size_t)(h * 8 * D + i)] - (h < 4 ? 1.0f : 3.0f)) < 1e-5f;
+    CHECK(ok);
+}
+
+int main(int argc, char** argv) {
+    const bool cpu_only = argc > 1 && std::string(argv[1]) == "--cpu-only";
+    test_gqa_constructor_validation();
+    if (!cpu_only) {
+        test_kv_cache_basic();
+        test_flash_attention_against_oracle();
+        run_cached_generation<nn::KVCache>(KVFormat::Float32, DType::Float32, 1e-4, "KVCache fp32");
+        run_cached_generation<nn::GQAKVCache>(KVFormat::BFloat16, DType::BFloat16, 2e-2, "GQAKVCache bf16");
+        run_cached_generation<nn::GQAKVCache>(KVFormat::Q8_0, DType::BFloat16, 2e-2, "GQAKVCache q8_0");
+        test_sdpa_routing();
+    }
+    std::printf(g_fail ? "FAILED: %d check(s)\n" : "all adapter tests passed\n", g_fail);
+    return g_fail ? 1 : 0;
+}

@@ -1,0 +1,392 @@
+// C++ mirror of the reference's operator surface for the attention path, implemented on the C ABI
+// of libvsp_attn.so (include/vsp_attn.h).  Same names, argument meaning and exception types/messages
+// as the reference, so that code written against
+//   vesper::ops::flash_attention / flash_attention_hip_dispatch   include/vesper/ops/flash_attention.h:34-41,74-78
+//   vesper::ops::repeat_kv                                         include/vesper/ops/attention_ops.h:24
+//   vesper::nn::functional::scaled_dot_product_attention           include/vesper/nn/functional.h:132-136
+//   vesper::nn::KVCache / GQAKVCache                               include/vesper/nn/transformer.h:21-39,
+//                                                                  include/vesper/nn/gqa_attention.h:110-163
+//   the attention core of GroupedQueryAttention / MultiHeadAttention::forward(x, cache, start_pos)
+//                                                                  src/nn/gqa_attention.cpp:128-148, src/nn/transformer.cpp:190-205
+// reads the same here.  The Tensor below is the small part of vesper::Tensor those interfaces need
+// (a strided view over shared device storage); a maintainer wiring the library into the reference
+// itself would instead fill vsp_tensor from vesper::Tensor directly.
+// Header-only; link with libvsp_attn.so and the HIP runtime.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdint>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <tuple>
+#include <utility>
+#include <vector>
+
+#include "../../../include/vsp_attn.h"
+
+namespace vesper_amd {
+
+enum class DType { Float32, BFloat16 };
+enum class Device { CPU, HIP };
+enum class KVFormat { Float32 = VSP_KV_F32, BFloat16 = VSP_KV_BF16, Q8_0 = VSP_KV_Q8_0 };
+
+inline size_t GetDTypeSize(DType d) { return d == DType::Float32 ? 4 : 2; }
+
+inline void hip_check(hipError_t e, const char* what) {
+    if (e != hipSuccess) throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(e));
+}
+
+// Maps a vsp_status to the exception the reference throws at the same point
+// (std::invalid_argument in the GroupedQueryAttention constructor, std::runtime_error elsewhere).
+inline void throw_status(int st) {
+    if (st == VSP_OK) return;
+    if (st == VSP_ERR_GQA_HEADS || st == VSP_ERR_GQA_EMBED) throw std::invalid_argument(vsp_status_str(st));
+    std::string msg = vsp_status_str(st);
+    if (st == VSP_ERR_LAUNCH) msg += std::string(": ") + vsp_last_hip_error();
+    throw std::runtime_error(msg);
+}
+
+// The thread's current stream, like Stream::current(Device::HIP) (src/core/stream.cpp:132-166).
+inline hipStream_t& current_stream() {
+    thread_local hipStream_t s = nullptr;
+    return s;
+}
+
+class Storage {
+public:
+    explicit Storage(size_t bytes) : bytes_(bytes) {
+        if (bytes) hip_check(hipMalloc(&ptr_, bytes), "hipMalloc");
+    }
+    ~Storage() {
+        if (ptr_) (void)hipFree(ptr_);
+    }
+    Storage(const Storage&) = delete;
+    Storage& operator=(const Storage&) = delete;
+    void* data() const { return ptr_; }
+    size_t bytes() const { return bytes_; }
+
+private:
+    void* ptr_ = nullptr;
+    size_t bytes_ = 0;
+};
+
+// What a Tensor returned by KVCache::update refers to.
+struct KVCacheState {
+    vsp_kv_cache c{};
+    std::shared_ptr<Storage> planes[4];
+};
+
+class Tensor {
+public:
+    Tensor() = default;
+    // view over existing storage (offset in elements)
+    static Tensor over(std::shared_ptr<Storage> s, DType dt, std::vector<int64_t> shape, std::vector<int64_t> strides,
+                       size_t offset = 0) {
+        Tensor t;
+        t.storage_ = std::move(s);
+        t.dtype_ = dt;
+        t.shape_ = std::move(shape);
+        t.strides_ = std::move(strides);
+        t.offset_ = offset;
+        return t;
+    }
+    static std::vector<int64_t> contiguous_strides(const std::vector<int64_t>& shape) {
+        std::vector<int64_t> st(shape.size(), 1);
+        int64_t s = 1;
+        for (int i = (int)shape.size() - 1; i >= 0; --i) {
+            st[i] = s;
+            s *= shape[i];
+        }
+        return st;
+    }
+    const std::vector<int64_t>& shape() const { return shape_; }
+    const std::vector<int64_t>& strides() const { return strides_; }
+    int64_t ndim() const { return (int64_t)shape_.size(); }
+    DType dtype() const { return dtype_; }
+    Device device() const { return Device::HIP; }
+    size_t offset() const { return offset_; }
+    bool defined() const { return storage_ != nullptr; }
+    size_t numel() const {
+        size_t n = 1;
+        for (auto s : shape_) n *= (size_t)s;
+        return n;
+    }
+    bool is_contiguous() const {
+        int64_t expect = 1;
+        for (int i = (int)shape_.size() - 1; i >= 0; --i) {
+            if (shape_[i] != 1 && strides_[i] != expect) return false;
+            expect *= shape_[i];
+        }
+        return true;
+    }
+    template <typename T>
+    T* data_ptr() const {
+        return (T*)((char*)storage_->data() + offset_ * GetDTypeSize(dtype_));
+    }
+    // host <-> device in contiguous (row-major) order of the view; blocking, like the reference's
+    void copy_from_host(const void* src) { host_copy(const_cast<void*>(src), true); }
+    void copy_to_host(void* dst) const { const_cast<Tensor*>(this)->host_copy(dst, false); }
+    // [:, :, start:stop, :] of a 4-D tensor (the only slicing this path needs)
+    Tensor slice_seq(int64_t start, int64_t stop) const {
+        Tensor t = *this;
+        t.shape_[2] = stop - start;
+        t.offset_ += (size_t)(start * strides_[2]);
+        return t;
+    }
+    vsp_tensor desc() const {
+        vsp_tensor d{};
+        d.data = (storage_ && storage_->data()) ? (void*)data_ptr<char>() : nullptr;
+        d.dtype = dtype_ == DType::Float32 ? VSP_F32 : VSP_BF16;
+        d.ndim = (int32_t)shape_.size();
+        for (size_t i = 0; i < shape_.size() && i < 4; ++i) {
+            d.shape[i] = shape_[i];
+            d.stride[i] = strides_[i];
+        }
+        return d;
+    }
+
+    // set by ops::repeat_kv: logically [B, H*head_rep, S, D], physically the un-repeated tensor
+    int64_t head_rep = 1;
+    // set by KVCache::update: this tensor is the K (is_v == false) or V side of that cache's context
+    std::shared_ptr<KVCacheState> cache;
+    bool is_v = false;
+
+private:
+    void host_copy(void* host, bool to_device) {
+        const size_t esz = GetDTypeSize(dtype_);
+        if (numel() == 0) return;
+        hipStream_t st = current_stream();
+        auto kind = to_device ? hipMemcpyHostToDevice : hipMemcpyDeviceToHost;
+        if (is_contiguous()) {
+            void* dev = (void*)data_ptr<char>();
+            hip_check(hipMemcpyAsync(to_device ? dev : host, to_device ? host : dev, numel() * esz, kind, st), "hipMemcpyAsync");
+        } else {
+            if (strides_.back() != 1) throw std::runtime_error("copy: innermost stride must be 1");
+            const size_t row = (size_t)shape_.back(), rows = numel() / row;
+            for (size_t r = 0; r < rows; ++r) {
+                size_t rem = r, off = 0;
+                for (int d = (int)shape_.size() - 2; d >= 0; --d) {
+                    off += (rem % (size_t)shape_[d]) * (size_t)strides_[d];
+                    rem /= (size_t)shape_[d];
+                }
+                void* dev = data_ptr<char>() + off * esz;
+                void* h = (char*)host + r * row * esz;
+                hip_check(hipMemcpyAsync(to_device ? dev : h, to_device ? h : dev, row * esz, kind, st), "hipMemcpyAsync");
+            }
+        }
+        hip_check(hipStreamSynchronize(st), "hipStreamSynchronize");
+    }
+    std::shared_ptr<Storage> storage_;
+    DType dtype_ = DType::Float32;
+    std::vector<int64_t> shape_, strides_;
+    size_t offset_ = 0;
+};
+
+inline Tensor empty(const std::vector<int64_t>& shape, DType dtype, Device device = Device::HIP) {
+    if (device != Device::HIP) throw std::runtime_error("vesper_amd: only Device::HIP tensors exist on this path");
+    size_t n = 1;
+    for (auto s : shape) n *= (size_t)s;
+    return Tensor::over(std::make_shared<Storage>(n * GetDTypeSize(dtype)), dtype, shape, Tensor::contiguous_strides(shape));
+}
+
+// ------------------------------------------------------------------------------------------------
+namespace nn {
+
+// One template for both reference caches: LenT = int for KVCache, int64_t for GQAKVCache.
+template <typename LenT>
+class KVCacheT {
+public:
+    KVCacheT(LenT batch_size, LenT num_heads, LenT max_seq_len, LenT head_dim, Device device = Device::HIP,
+             KVFormat format = KVFormat::Float32)
+        : st_(std::make_shared<KVCacheState>()) {
+        if (device != Device::HIP) throw std::runtime_error("KVCache: only Device::HIP is implemented here");
+        auto& c = st_->c;
+        c.format = (int32_t)format;
+        c.B = (int32_t)batch_size;
+        c.Hkv = (int32_t)num_heads;
+        c.S_max = (int32_t)max_seq_len;
+        c.D = (int32_t)head_dim;
+        for (int p = 0; p < 4; ++p) {
+            size_t n = vsp_kv_plane_bytes(c.format, c.B, c.Hkv, c.S_max, c.D, p);
+            if (n) st_->planes[p] = std::make_shared<Storage>(n);
+        }
+        c.k = st_->planes[0] ? st_->planes[0]->data() : nullptr;
+        c.v = st_->planes[1] ? st_->planes[1]->data() : nullptr;
+        c.k_scale = st_->planes[2] ? st_->planes[2]->data() : nullptr;
+        c.v_scale = st_->planes[3] ? st_->planes[3]->data() : nullptr;
+        c.len = 0;
+        throw_status(vsp_kv_cache_reset(&c, current_stream()));  // vesper::zeros in the reference constructor
+    }
+
+    // Writes [:, :, start_pos:start_pos+T, :], then returns the active context [:, :, 0:len, :].
+    // Float32 storage: the pair are true strided views of the cache planes, as in the reference.
+    // Other formats: the pair are handles (shape [B,H,len,D], no dense storage) that
+    // scaled_dot_product_attention consumes directly; materialize() makes a real tensor of one.
+    std::pair<Tensor, Tensor> update(const Tensor& new_k, const Tensor& new_v, LenT start_pos) {
+        vsp_tensor dk = new_k.desc(), dv = new_v.desc();
+        throw_status(vsp_kv_append(&st_->c, &dk, &dv, (int64_t)start_pos, nullptr, current_stream()));
+        return {view(false), view(true)};
+    }
+    void reset() { throw_status(vsp_kv_cache_reset(&st_->c, current_stream())); }
+    LenT current_seq_len() const { return (LenT)st_->c.len; }
+    LenT get_max_seq_len() const { return (LenT)st_->c.S_max; }  // KVCache spelling
+    LenT max_seq_len() const { return (LenT)st_->c.S_max; }      // GQAKVCache spelling
+    static float memory_savings(int64_t num_query_heads, int64_t num_kv_heads) {
+        return 1.0f - static_cast<float>(num_kv_heads) / num_query_heads;
+    }
+    KVFormat format() const { return (KVFormat)st_->c.format; }
+    const vsp_kv_cache& raw() const { return st_->c; }
+
+private:
+    Tensor view(bool is_v) const {
+        const auto& c = st_->c;
+        Tensor t;
+        if (c.format == VSP_KV_F32) {
+            std::vector<int64_t> shape = {c.B, c.Hkv, c.S_max, c.D};
+            t = Tensor::over(st_->planes[is_v ? 1 : 0], DType::Float32, shape, Tensor::contiguous_strides(shape)).slice_seq(0, c.len);
+        } else {
+            std::vector<int64_t> shape = {c.B, c.Hkv, c.len, c.D};
+            t = Tensor::over(nullptr, DType::BFloat16, shape, Tensor::contiguous_strides(shape));
+        }
+        t.cache = std::make_shared<KVCacheState>(*st_);  // snapshot of the descriptor (len as of this update)
+        t.is_v = is_v;
+        return t;
+    }
+    std::shared_ptr<KVCacheState> st_;
+};
+
+using KVCache = KVCacheT<int>;
+using GQAKVCache = KVCacheT<int64_t>;
+
+// [:, :, 0:len, :] of a cache handle as a real tensor of `dtype` (copy; Q8_0 is dequantised).
+inline Tensor materialize(const Tensor& handle, DType dtype) {
+    if (!handle.cache || handle.defined()) return handle;
+    const auto& c = handle.cache->c;
+    Tensor out = empty({c.B, c.Hkv, c.len, c.D}, dtype);
+    vsp_tensor d = out.desc();
+    throw_status(vsp_kv_read(&c, 0, c.len, handle.is_v ? nullptr : &d, handle.is_v ? &d : nullptr, current_stream()));
+    out.head_rep = handle.head_rep;
+    return out;
+}
+
+}  // namespace nn
+
+// ------------------------------------------------------------------------------------------------
+namespace ops {
+
+// ops::repeat_kv (src/ops/attention_ops.cpp:92-155).  No copy is made: the result remembers n_rep
+// and the attention kernels map query head h to kv head h / n_rep (src/ops/attention_ops.cpp:47).
+inline Tensor repeat_kv(const Tensor& x, int64_t n_rep) {
+    if (n_rep == 1) return x;
+    if (x.ndim() != 4) throw std::runtime_error("repeat_kv: input must be 4D [Batch, KV_Heads, SeqLen, HeadDim]");
+    Tensor r = x;
+    r.head_rep = x.head_rep * n_rep;
+    return r;
+}
+
+// include/vesper/ops/flash_attention.h:74-78.  output/lse are caller-allocated; lse may be undefined.
+inline void flash_attention_hip_dispatch(const Tensor& q, const Tensor& k, const Tensor& v, Tensor& output, Tensor& lse,
+                                         float scale, bool is_causal, float dropout_p, bool training,
+                                         Tensor* dropout_mask_out) {
+    (void)dropout_mask_out;  // only written when training && dropout_p > 0, which this path rejects
+    Tensor kk = nn::materialize(k, q.dtype()), vv = nn::materialize(v, q.dtype());
+    vsp_tensor dq = q.desc(), dk = kk.desc(), dv = vv.desc(), dout = output.desc(), dl = lse.desc();
+    // a repeat_kv'ed operand must expand to exactly q's head count
+    if (q.ndim() == 4 && kk.ndim() == 4 && (kk.shape()[1] * kk.head_rep != q.shape()[1] || vv.shape()[1] * vv.head_rep != q.shape()[1]))
+        throw_status(VSP_ERR_SHAPE);
+    throw_status(vsp_attn_prefill(&dq, &dk, &dv, &dout, lse.defined() ? &dl : nullptr, scale, is_causal ? 1 : 0, dropout_p,
+                                  training ? 1 : 0, current_stream()));
+}
+
+// include/vesper/ops/flash_attention.h:34-41.
+inline Tensor flash_attention(const Tensor& q, const Tensor& k, const Tensor& v, float scale, bool is_causal = true,
+                              float dropout_p = 0.0f, bool training = false) {
+    if (q.ndim() != 4 || k.ndim() != 4 || v.ndim() != 4) throw_status(VSP_ERR_NDIM);
+    Tensor output = empty(q.shape(), q.dtype());
+    Tensor lse = empty({q.shape()[0], q.shape()[1], q.shape()[2]}, DType::Float32);
+    flash_attention_hip_dispatch(q, k, v, output, lse, scale, is_causal, dropout_p, training, nullptr);
+    return output;
+}
+
+}  // namespace ops
+
+namespace nn {
+namespace functional {
+
+// include/vesper/nn/functional.h:132-136, src/nn/functional.cpp:370-422.  One kernel family serves
+// every sequence length (the reference's switch at 512 is a speed heuristic of its own back ends):
+// T == 1 over a cache handle -> split-K decode; everything else -> the prefill kernel.
+inline Tensor scaled_dot_product_attention(const Tensor& query, const Tensor& key, const Tensor& value, bool is_causal = false,
+                                           double dropout_p = 0.0) {
+    if (dropout_p > 0.0) throw_status(VSP_ERR_UNSUPPORTED);
+    if (query.ndim() != 4 || key.ndim() != 4 || value.ndim() != 4) throw_status(VSP_ERR_NDIM);
+    const int64_t T = query.shape()[2], L = key.shape()[2], D = query.shape()[3];
+    if (is_causal && T != L && T != 1) throw_status(VSP_ERR_BROADCAST);  // [T,T] mask vs [T,L] scores
+    const float scale = 1.0f / std::sqrt(static_cast<float>(D));
+    if (T == 1 && key.cache && value.cache && !key.is_v && value.is_v) {
+        Tensor out = empty(query.shape(), query.dtype());
+        const vsp_kv_cache& c = key.cache->c;
+        const size_t ws_bytes = vsp_attn_decode_workspace_bytes((int32_t)query.shape()[0], (int32_t)query.shape()[1], (int32_t)D,
+                                                               c.len > 0 ? c.len : 1);
+        Storage ws(ws_bytes);
+        vsp_tensor dq = query.desc(), dout = out.desc();
+        throw_status(vsp_attn_decode(&dq, &c, nullptr, 0, &dout, scale, ws.data(), ws_bytes, current_stream()));
+        hip_check(hipStreamSynchronize(current_stream()), "hipStreamSynchronize");  // ws is freed on return
+        return out;
+    }
+    return ops::flash_attention(query, key, value, scale, is_causal && T > 1);
+}
+
+}  // namespace functional
+
+// The attention core shared by GroupedQueryAttention::forward(x, cache, start_pos)
+// (src/nn/gqa_attention.cpp:111-159, steps 4-6) and MultiHeadAttention::forward(x, cache, start_pos)
+// (src/nn/transformer.cpp:166-216): q [B,Hq,T,D], k/v [B,Hkv,T,D] are what the projections + RoPE
+// produced.  The constructor performs the reference constructor's checks and arithmetic.
+class GroupedQueryAttentionCore {
+public:
+    GroupedQueryAttentionCore(int64_t embed_dim, int64_t num_heads, int64_t num_kv_heads)
+        : embed_dim_(embed_dim), num_heads_(num_heads), num_kv_heads_(num_kv_heads) {
+        if (num_heads % num_kv_heads != 0)
+            throw std::invalid_argument("GroupedQueryAttention: num_heads (" + std::to_string(num_heads) +
+                                        ") must be divisible by num_kv_heads (" + std::to_string(num_kv_heads) + ")");
+        if (embed_dim % num_heads != 0)
+            throw std::invalid_argument("GroupedQueryAttention: embed_dim (" + std::to_string(embed_dim) +
+                                        ") must be divisible by num_heads (" + std::to_string(num_heads) + ")");
+        throw_status(vsp_gqa_config(embed_dim, num_heads, num_kv_heads, &head_dim_, &num_rep_));
+    }
+    int64_t embed_dim() const { return embed_dim_; }
+    int64_t num_heads() const { return num_heads_; }
+    int64_t num_kv_heads() const { return num_kv_heads_; }
+    int64_t head_dim() const { return head_dim_; }
+    int64_t num_rep() const { return num_rep_; }
+    float kv_cache_ratio() const { return static_cast<float>(num_kv_heads_) / num_heads_; }
+
+    // forward(x, causal) core, src/nn/gqa_attention.cpp:91-96
+    Tensor forward(const Tensor& q, const Tensor& k, const Tensor& v, bool causal = true) const {
+        return functional::scaled_dot_product_attention(q, ops::repeat_kv(k, num_rep_), ops::repeat_kv(v, num_rep_), causal, 0.0);
+    }
+    // forward(x, cache, start_pos) core, src/nn/gqa_attention.cpp:128-148
+    template <typename CacheT>
+    Tensor forward(const Tensor& q, Tensor k, Tensor v, CacheT* cache, int64_t start_pos = 0) const {
+        const int64_t T = q.shape()[2];
+        if (cache) {
+            auto kv = cache->update(k, v, (decltype(cache->current_seq_len()))start_pos);
+            k = kv.first;
+            v = kv.second;
+        }
+        k = ops::repeat_kv(k, num_rep_);
+        v = ops::repeat_kv(v, num_rep_);
+        const bool use_causal = (T > 1);
+        return functional::scaled_dot_product_attention(q, k, v, use_causal, 0.0);
+    }
+
+private:
+    int64_t embed_dim_, num_heads_, num_kv_heads_, head_dim_ = 0, num_rep_ = 0;
+};
+
+}  // namespace nn
+}  // namespace vesper_amd
