@@ -7,9 +7,15 @@
 // LSE = m + log l; the arithmetic is bf16 MFMA with fp32 accumulation (or fp32 MFMA for fp32 inputs).
 //
 // bf16 kernel.  A workgroup of 4 wavefronts owns 128 consecutive queries of one (batch, query head);
-// each wavefront owns 32 of them.  Key tiles of 64 go through LDS (register-staged prefetch of the
-// next tile while the current one is consumed).  Both GEMMs are computed transposed so that the
-// softmax statistics of a query live in one lane (and its partner 32 lanes away):
+// each wavefront owns 32 of them.  Key tiles of 32 go from global memory straight into LDS (buffer
+// loads with the LDS modifier, two ring slots, the next tile in flight while the current one is
+// consumed, one barrier per tile).  LDS rows are unpadded; 16-byte chunks are XOR-swizzled so that
+// both the ds_read_b128 of K and the transposing reads of V are bank-conflict free.  The vector ALU,
+// not the matrix pipe, is what this kernel runs out of first (VALU and MFMA issue from one SIMD
+// overlap only partly), so the loop is written to keep VALU instructions per MFMA minimal: addresses
+// live in scalar registers, the row sum is a packed dot product, the mask and the rescale are rare
+// branches.  Both GEMMs are computed transposed so that the softmax statistics of a query live in one
+// lane (and its partner 32 lanes away):
 //   S^T[key][q] = K[key][:] . Q^T[:][q]     32x32x16 MFMA, A = K rows from LDS, B = Q^T held in registers
 //   O^T[d][q]  += V^T[d][key] . P^T[key][q]  A = V^T read from the row-major V tile with the
 //                                            transposing LDS read, B = P^T straight from the S^T registers
@@ -40,15 +46,10 @@ struct PrefillArgs {
 };
 
 constexpr int kBM = 128;       // queries per workgroup
-constexpr int kBN = 64;        // keys per tile
 constexpr float kRescaleThreshold = 8.0f;
 
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
-
-__device__ inline uint2 lds_read_tr16_b64(const uint16_t* p) {
-    s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4_t __attribute__((address_space(3)))*)p);
-    return __builtin_bit_cast(uint2, v);
-}
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 
 __device__ inline uint32_t cvt_pk_bf16(float a, float b) {
     typedef float f32x2_t __attribute__((ext_vector_type(2)));
@@ -61,39 +62,66 @@ __device__ inline uint32_t cvt_pk_bf16(float a, float b) {
 __device__ inline float half_swap_max(float x) { return fmaxf(x, __shfl_xor(x, 32)); }
 __device__ inline float half_swap_sum(float x) { return x + __shfl_xor(x, 32); }
 
+// Transposing LDS read issued through inline asm: the compiler cannot prove that a builtin
+// transposing read does not alias an outstanding direct-to-LDS load and would wait for every such
+// load before it.  The asm form carries no such wait; tr_wait() below is the matching
+// "all my LDS reads have returned" fence, tied to the values by data dependence.
+template <int OFFSET_BYTES>
+__device__ inline uint2 lds_read_tr16_b64_asm(uint32_t lds_byte_addr) {
+    uint2 v;
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(lds_byte_addr), "n"(OFFSET_BYTES));
+    return v;
+}
+__device__ inline void tr_wait(uint2& a0, uint2& a1, uint2& a2, uint2& a3, uint2& a4, uint2& a5, uint2& a6, uint2& a7) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3), "+v"(a4), "+v"(a5), "+v"(a6), "+v"(a7));
+}
+__device__ inline void tr_wait(uint2& a0, uint2& a1, uint2& a2, uint2& a3) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3));
+}
+__device__ inline uint32_t lds_addr(const void* p) {
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
+}
+
+constexpr int kUnit = 32;  // keys per tile (one LDS ring slot)
+
 template <int D>
-__global__ void __launch_bounds__(256, 2) prefill_bf16_kernel(PrefillArgs a) {
-    constexpr int KS = D / 16;      // k-steps of S^T over the head dim
-    constexpr int DB = D / 32;      // 32-row tiles of O^T
-    constexpr int KPITCH = D + 8;   // LDS row pitch of the K tile (elements): rows shift by 16 B -> ds_read_b128 conflict-free
-    constexpr int VPITCH = D + 32;  // V tile: rows shift by 64 B -> the 4-row transposing reads are conflict-free
-    constexpr int CPR = D / 8;      // 16-byte chunks per row
-    constexpr int NLD = kBN * CPR / 256;  // chunks per thread per tile
+__global__ void __launch_bounds__(256, 3) prefill_bf16_kernel(PrefillArgs a) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the body uses device-only builtins
+    constexpr int KS = D / 16;
+    constexpr int DB = D / 32;
+    constexpr int CPR = D / 8;
+    constexpr int RP = 256 / (2 * D);
+    constexpr int NR = 1024 / (2 * D);
+    constexpr int NGRP = kUnit / NR;
+    constexpr int NLD = (NGRP + 3) / 4;
+    constexpr int SLOT = kUnit * D;
+    constexpr int NKB = kUnit / 32;   // 32-key S^T blocks per tile
+    constexpr int NJ = kUnit / 16;    // PV k-steps per tile
 
-    __shared__ __attribute__((aligned(16))) uint16_t sK[kBN * KPITCH];
-    __shared__ __attribute__((aligned(16))) uint16_t sV[kBN * VPITCH];
+    __shared__ __attribute__((aligned(1024))) uint16_t sK0[SLOT];
+    __shared__ __attribute__((aligned(1024))) uint16_t sK1[SLOT];
+    __shared__ __attribute__((aligned(1024))) uint16_t sV0[SLOT];
+    __shared__ __attribute__((aligned(1024))) uint16_t sV1[SLOT];
 
-    // heaviest query tiles first (causal work grows with the tile index); heads of one kv group adjacent
     const int bid = blockIdx.x;
     const int qt = a.n_qtiles - 1 - bid / (a.B * a.Hq);
     const int bh = bid % (a.B * a.Hq);
     const int b = bh / a.Hq, hq = bh % a.Hq, kvh = hq / a.n_rep;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int ql = lane & 31, h = lane >> 5;
-    const int q0 = qt * kBM + wave * 32;   // first query of this wavefront
-    const int off = a.L - a.T;             // key j visible to query t iff j <= t + off
+    const int q0 = qt * kBM + wave * 32;
+    const int off = a.L - a.T;
     const int qrow = min(q0 + ql, a.T - 1);
 
     const uint16_t* Qp = (const uint16_t*)a.q + (int64_t)b * a.sq[0] + (int64_t)hq * a.sq[1];
     const uint16_t* Kp = (const uint16_t*)a.k + (int64_t)b * a.sk[0] + (int64_t)kvh * a.sk[1];
     const uint16_t* Vp = (const uint16_t*)a.v + (int64_t)b * a.sv[0] + (int64_t)kvh * a.sv[1];
 
-    // Q^T operands (B of S^T): column ql, contraction slots d = 16*ks + 8*h + e
     bf16x8_t qf[KS];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-    {
+    for (int ks = 0; ks < KS; ++ks) {
         uint4 w = *(const uint4*)(Qp + (int64_t)qrow * a.sq[2] + 16 * ks + 8 * h);
         if (a.negate_q) {
             w.x ^= 0x80008000u;
@@ -104,85 +132,87 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_kernel(PrefillArgs a) {
         qf[ks] = __builtin_bit_cast(bf16x8_t, w);
     }
 
-    // number of key tiles this workgroup / this wavefront needs
     const int wg_qmax = min(qt * kBM + kBM - 1, a.T - 1);
     const int kv_end_wg = a.causal ? min(a.L, wg_qmax + off + 1) : a.L;
-    const int n_tiles = (kv_end_wg + kBN - 1) / kBN;
+    const int n_tiles = (kv_end_wg + kUnit - 1) / kUnit;
     const int wave_qmax = min(q0 + 31, a.T - 1);
-    const int kv_end_wave = a.causal ? min(a.L, wave_qmax + off + 1) : a.L;  // may be <= 0 for waves past T
+    const int kv_end_wave = (q0 < a.T) ? (a.causal ? min(a.L, wave_qmax + off + 1) : a.L) : 0;
 
     f32x16_t acc[DB];
 #pragma unroll
     for (int i = 0; i < DB; ++i)
 #pragma unroll
         for (int j = 0; j < 16; ++j) acc[i][j] = 0.f;
-    float m_ref = -INFINITY;  // reference maximum used in the exponent (log2 domain, scaled)
-    float l = 0.f;            // this lane's share of the row sum
+    float m_ref = -INFINITY;
+    float l = 0.f;
 
-    uint4 stage_k[NLD], stage_v[NLD];
-    auto load_tile = [&](int kt) {
+    // Global -> LDS through buffer loads with the LDS modifier: one wave-wide load fills 1024 contiguous
+    // bytes of LDS (lane i -> bytes [16 i, 16 i + 16)), i.e. NR rows; the swizzle is applied by choosing
+    // which 16-byte chunk of the global row each lane fetches.  The buffer descriptor is rebuilt per tile on
+    // the scalar unit (base = first row of the tile, size = bytes up to the end of the context), so the
+    // per-lane offsets are loop constants and rows past the end of the context read as zeros.
+    const int ld_row = lane / CPR, ld_pos = lane % CPR;
+    uint32_t voffK[NLD], voffV[NLD];
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+        const int r = NR * (wave + 4 * i) + ld_row;
+        voffK[i] = (uint32_t)r * (uint32_t)a.sk[2] * 2u + 16u * (uint32_t)(ld_pos ^ ((r / RP) % CPR));
+        voffV[i] = (uint32_t)r * (uint32_t)a.sv[2] * 2u + 16u * (uint32_t)(ld_pos ^ (((r / RP) % (CPR / 4)) << 2));
+    }
+    const int64_t rowK = a.sk[2] * 2, rowV = a.sv[2] * 2;  // bytes per key row
+    auto load_tile = [&](int t, uint16_t* dstK, uint16_t* dstV) {
+        const int key0 = t * kUnit;
+        const int rows = a.L - key0;  // > 0
+        __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)Kp + (int64_t)key0 * rowK), 0, (int)((int64_t)rows * rowK), 0x00020000);
+        __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)Vp + (int64_t)key0 * rowV), 0, (int)((int64_t)rows * rowV), 0x00020000);
 #pragma unroll
         for (int i = 0; i < NLD; ++i) {
-            const int id = tid + 256 * i, row = id / CPR, cc = id % CPR;
-            const int key = kt * kBN + row;
-            if (key < a.L) {
-                stage_k[i] = *(const uint4*)(Kp + (int64_t)key * a.sk[2] + 8 * cc);
-                stage_v[i] = *(const uint4*)(Vp + (int64_t)key * a.sv[2] + 8 * cc);
-            } else {
-                stage_k[i] = uint4{0, 0, 0, 0};
-                stage_v[i] = uint4{0, 0, 0, 0};
-            }
-        }
-    };
-    auto store_tile = [&]() {
-#pragma unroll
-        for (int i = 0; i < NLD; ++i) {
-            const int id = tid + 256 * i, row = id / CPR, cc = id % CPR;
-            *(uint4*)(sK + row * KPITCH + 8 * cc) = stage_k[i];
-            *(uint4*)(sV + row * VPITCH + 8 * cc) = stage_v[i];
+            const int grp = wave + 4 * i;
+            if (NGRP % 4 != 0 && grp >= NGRP) break;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (__attribute__((address_space(3))) void*)(dstK + grp * 512), 16, voffK[i], 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (__attribute__((address_space(3))) void*)(dstV + grp * 512), 16, voffV[i], 0, 0, 0);
         }
     };
 
-    if (n_tiles > 0) load_tile(0);
-    for (int kt = 0; kt < n_tiles; ++kt) {
-        __syncthreads();  // everyone is done reading the previous tile
-        store_tile();
+    const int kswz = (ql / RP) % CPR;
+    const int i16 = lane & 15;
+    const int vswz = ((i16 >> 2) / RP) % (CPR / 4);
+    const int v_lane_off = (4 * h + (i16 >> 2)) * D + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+
+    auto tile_step = [&](int t, const uint16_t* sK, const uint16_t* sV, uint16_t* nextK, uint16_t* nextV) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if (kt + 1 < n_tiles) load_tile(kt + 1);  // in flight while this tile is consumed
+        if (t + 1 < n_tiles) load_tile(t + 1, nextK, nextV);
+        const int k0 = t * kUnit;
+        if (k0 >= kv_end_wave) return;
 
-        const int k0 = kt * kBN;
-        if (k0 >= kv_end_wave) continue;  // tile entirely masked for this wavefront (uniform per wave)
-
-        // ---- S^T = K . Q^T for the two 32-key halves of the tile
-        f32x16_t s[2];
+        f32x16_t s[NKB];
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
+        for (int kb = 0; kb < NKB; ++kb) {
 #pragma unroll
             for (int j = 0; j < 16; ++j) s[kb][j] = 0.f;
-            const uint16_t* kr = sK + (32 * kb + ql) * KPITCH + 8 * h;
+            const uint16_t* kr = sK + (32 * kb + ql) * D;
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                bf16x8_t kf = __builtin_bit_cast(bf16x8_t, *(const uint4*)(kr + 16 * ks));
+                bf16x8_t kf = __builtin_bit_cast(bf16x8_t, *(const uint4*)(kr + 8 * ((2 * ks + h) ^ kswz)));
                 s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], s[kb], 0, 0, 0);
             }
         }
-        // ---- mask (only tiles that straddle the diagonal or the end of the context)
-        const int q_abs = q0 + ql + off;  // last visible key of this lane's query
-        const bool need_mask = (a.causal && k0 + kBN - 1 > q0 + off) || (k0 + kBN > a.L);
+        const bool need_mask = (a.causal && k0 + kUnit - 1 > q0 + off) || (k0 + kUnit > a.L);
         if (need_mask) {
+            const int q_abs = q0 + ql + off;
             const int lim = a.causal ? min(q_abs, a.L - 1) : a.L - 1;
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+            for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     const int key = k0 + 32 * kb + 8 * (v >> 2) + 4 * h + (v & 3);
                     if (key > lim) s[kb][v] = -INFINITY;
                 }
         }
-        // ---- running maximum (raw scores; scale_log2 > 0 here, a negative scale was folded into Q)
         float mx = s[0][0];
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+        for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
             for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[kb][v]);
         mx = half_swap_max(mx) * a.scale_log2;
@@ -196,35 +226,65 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_kernel(PrefillArgs a) {
                 for (int j = 0; j < 16; ++j) acc[i][j] *= alpha;
             m_ref = m_new;
         }
-        // ---- P^T = exp2(S^T * c - m_ref), packed to bf16 as the B operands of the PV MFMAs
         const float neg_m = (m_ref == -INFINITY) ? 0.f : -m_ref;
-        uint32_t pw[4][4];
+        uint32_t pw[NJ][4];
+        float lsum = 0.f;
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+        for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
             for (int v = 0; v < 16; v += 2) {
                 const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][v], a.scale_log2, neg_m));
                 const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][v + 1], a.scale_log2, neg_m));
-                l += p0 + p1;
-                pw[2 * kb + (v >> 3)][(v & 7) >> 1] = cvt_pk_bf16(p0, p1);
+                const uint32_t pk = cvt_pk_bf16(p0, p1);
+                pw[2 * kb + (v >> 3)][(v & 7) >> 1] = pk;
+                lsum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pk), __builtin_bit_cast(bf16x2_t, 0x3f803f80u), lsum, false);
             }
-        // ---- O^T += V^T . P^T
+        l += lsum;
+        // PV
+        const uint32_t vb = lds_addr(sV) + 2u * (uint32_t)v_lane_off;
+        uint32_t va[DB];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int db = 0; db < DB; ++db) va[db] = vb + 64u * (uint32_t)(db ^ vswz);
+        uint2 tcur[DB][2], tnext[DB][2];
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+            tcur[db][0] = lds_read_tr16_b64_asm<0>(va[db]);
+            tcur[db][1] = lds_read_tr16_b64_asm<8 * D * 2>(va[db]);
+        }
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            if constexpr (DB == 4) tr_wait(tcur[0][0], tcur[0][1], tcur[1][0], tcur[1][1], tcur[2][0], tcur[2][1], tcur[3][0], tcur[3][1]);
+            else tr_wait(tcur[0][0], tcur[0][1], tcur[1][0], tcur[1][1]);
+            if (j + 1 < NJ) {
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    if (j == 0) { tnext[db][0] = lds_read_tr16_b64_asm<16 * D * 2>(va[db]); tnext[db][1] = lds_read_tr16_b64_asm<24 * D * 2>(va[db]); }
+                    if (j == 1) { tnext[db][0] = lds_read_tr16_b64_asm<32 * D * 2>(va[db]); tnext[db][1] = lds_read_tr16_b64_asm<40 * D * 2>(va[db]); }
+                    if (j == 2) { tnext[db][0] = lds_read_tr16_b64_asm<48 * D * 2>(va[db]); tnext[db][1] = lds_read_tr16_b64_asm<56 * D * 2>(va[db]); }
+                }
+            }
             const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, uint4{pw[j][0], pw[j][1], pw[j][2], pw[j][3]});
-            // transposing read: a 16-lane group reads a 4(keys) x 16(d) patch; lane i of the group gets d = i.
-            const uint16_t* vr = sV + (16 * j + 4 * h + ((lane & 15) >> 2)) * VPITCH + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
-                const uint2 lo = lds_read_tr16_b64(vr + 32 * db);
-                const uint2 hi = lds_read_tr16_b64(vr + 8 * VPITCH + 32 * db);
-                const bf16x8_t vf = __builtin_bit_cast(bf16x8_t, uint4{lo.x, lo.y, hi.x, hi.y});
+                const bf16x8_t vf = __builtin_bit_cast(bf16x8_t, uint4{tcur[db][0].x, tcur[db][0].y, tcur[db][1].x, tcur[db][1].y});
                 acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf, acc[db], 0, 0, 0);
             }
+            if (j + 1 < NJ) {
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    tcur[db][0] = tnext[db][0];
+                    tcur[db][1] = tnext[db][1];
+                }
+            }
         }
+    };
+
+    if (n_tiles > 0) load_tile(0, sK0, sV0);
+    for (int t = 0; t < n_tiles; t += 2) {
+        tile_step(t, sK0, sV0, sK1, sV1);
+        if (t + 1 < n_tiles) tile_step(t + 1, sK1, sV1, sK0, sV0);
     }
 
-    // ---- epilogue: O = acc / l, LSE = (m_ref + log2 l) * ln 2
     l = half_swap_sum(l);
     const int qi = q0 + ql;
     if (qi < a.T) {
@@ -236,13 +296,14 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_kernel(PrefillArgs a) {
             for (int vq = 0; vq < 4; ++vq) {
                 const int d = 32 * db + 8 * vq + 4 * h;
                 uint2 w;
-                w.x = (uint32_t)f32_to_bf16_bits(acc[db][4 * vq] * inv_l) | ((uint32_t)f32_to_bf16_bits(acc[db][4 * vq + 1] * inv_l) << 16);
-                w.y = (uint32_t)f32_to_bf16_bits(acc[db][4 * vq + 2] * inv_l) | ((uint32_t)f32_to_bf16_bits(acc[db][4 * vq + 3] * inv_l) << 16);
+                w.x = cvt_pk_bf16(acc[db][4 * vq] * inv_l, acc[db][4 * vq + 1] * inv_l);  // round-to-nearest-even
+                w.y = cvt_pk_bf16(acc[db][4 * vq + 2] * inv_l, acc[db][4 * vq + 3] * inv_l);
                 *(uint2*)(op + d) = w;
             }
         if (a.lse && h == 0)
             a.lse[(int64_t)b * a.sl[0] + (int64_t)hq * a.sl[1] + (int64_t)qi * a.sl[2]] = (m_ref + __builtin_amdgcn_logf(l)) * 0.6931471805599453f;
     }
+#endif
 }
 
 // ---------------------------------------------------------------------------------------------
