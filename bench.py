@@ -146,8 +146,8 @@ def cpu_baseline(key):
     kind = "reference" if use_ref else "port"
     rng = np.random.default_rng(1)
     if w["kind"] == "prefill":
-        # sample: 8 query heads (2 kv groups) of one batch row at full N: repeat_kv + flash_attention, fp32
-        Hq_s, Hkv_s, N, D = 8, 2, w["N"], w["D"]
+        # sample: one full batch row (32 query heads, 8 kv groups) at full N: repeat_kv + flash_attention, fp32
+        Hq_s, Hkv_s, N, D = 32, 8, w["N"], w["D"]
         q = O.bf16_round(rng.standard_normal((1, Hq_s, N, D), dtype=np.float32) * 0.5)
         k = O.bf16_round(rng.standard_normal((1, Hkv_s, N, D), dtype=np.float32) * 0.5)
         v = O.bf16_round(rng.standard_normal((1, Hkv_s, N, D), dtype=np.float32) * 0.5)

@@ -36,7 +36,7 @@ struct DecodeArgs {
     const void* v_scale;
     const int32_t* seq_lens;  // device, or nullptr
     int32_t len;              // used when seq_lens == nullptr
-    int32_t Hq, Hkv, n_rep;
+    int32_t B, Hq, Hkv, n_rep;
     int64_t S;  // physical token capacity of the planes
     int32_t S_max;  // logical capacity; lengths are clamped to it
     int32_t chunk;
@@ -68,20 +68,61 @@ __device__ inline uint4 mask_tail_u16x8(uint4 v, int nvalid) {
     return uint4{w[0], w[1], w[2], w[3]};
 }
 
+
+// Work items are (batch row, split) pairs packed without gaps: item i belongs to the sequence b with
+// offs(b) <= i < offs(b) + nsplits(b), nsplits(b) = ceil(L_b / chunk).  Lengths live on the device, so
+// every workgroup locates its item itself: 64 sequences at a time, one per lane, wave-wide prefix sum.
+// The grid is sized for the worst case; surplus workgroups sit at the END of the grid and exit at once
+// (with the (split, b) grid of a naive mapping the empty workgroups of short sequences would be
+// interleaved with real work and cost launch slots all the way through).
+__device__ inline bool locate_work(const DecodeArgs& a, int item, int lane, int& b, int& split, int& L) {
+    if (!a.seq_lens) {
+        L = min(a.len, a.S_max);
+        const int ns = (L + a.chunk - 1) / a.chunk;
+        if (ns == 0 || item >= ns * a.B) return false;
+        b = item / ns;
+        split = item - b * ns;
+        return true;
+    }
+    int base = 0;
+    for (int b0 = 0; b0 < a.B; b0 += 64) {
+        const int bb = b0 + lane;
+        const int Lb = bb < a.B ? min(max(a.seq_lens[bb], 0), a.S_max) : 0;
+        const int ns = (Lb + a.chunk - 1) / a.chunk;
+        int incl = ns;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int t = __shfl_up(incl, off);
+            if (lane >= off) incl += t;
+        }
+        const int total = __shfl(incl, 63);
+        if (item < base + total) {
+            const unsigned long long m = __ballot(base + incl > item);
+            const int src = __ffsll((long long)m) - 1;
+            b = b0 + src;
+            split = item - (base + __shfl(incl, src) - __shfl(ns, src));
+            L = __shfl(Lb, src);
+            return true;
+        }
+        base += total;
+    }
+    return false;
+}
+
 // ---------------------------------------------------------------------------------------------
 // bf16 cache
 // ---------------------------------------------------------------------------------------------
 template <int D>
-__global__ void __launch_bounds__(256) decode_bf16_kernel(DecodeArgs a) {
+__global__ void __launch_bounds__(256, 2) decode_bf16_kernel(DecodeArgs a) {
     constexpr int KS = D / 32;   // MFMA k-steps over the head dim
     constexpr int DB = D / 16;   // 16-row tiles of O^T
-    const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
-    const int L = min(a.seq_lens ? a.seq_lens[b] : a.len, a.S_max);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kvh = blockIdx.y;
+    int b, split, L;
+    if (!locate_work(a, blockIdx.x, lane, b, split, L)) return;
     const int chunk_start = split * a.chunk;
-    if (chunk_start >= L) return;
     const int chunk_end = min(L, chunk_start + a.chunk);
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c = lane & 15, g = lane >> 4;
 
     // Q^T operands: column c = query head kvh*n_rep + c (zero beyond n_rep)
@@ -104,24 +145,34 @@ __global__ void __launch_bounds__(256) decode_bf16_kernel(DecodeArgs a) {
     for (int i = 0; i < DB; ++i) acc[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, l = 0.f;
 
-    for (int kbase = chunk_start + wave * kGroup; kbase < chunk_end; kbase += kWaves * kGroup) {
-        // ---- loads: K rows (A operands of S^T), V^T blocks (A operands of O^T)
-        uint4 kf[4][KS];
+    // K rows (A operands of S^T) and V^T blocks (A operands of O^T) of one 64-key group.  The loop is
+    // rotated: the loads of group i+1 are issued as soon as group i's registers have been consumed
+    // (K after the S^T MFMAs, V after the O^T MFMAs), so every wavefront keeps HBM requests in flight
+    // while it computes.
+    uint4 kf[4][KS];
+    uint4 vf[DB][2];
+    auto load_k = [&](int kbase) {
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj) {
             const uint16_t* kr = Kp + (int64_t)(kbase + krow + 4 * jj) * D + 8 * g;
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) kf[jj][ks] = *(const uint4*)(kr + 32 * ks);
         }
-        uint4 vf[DB][2];
-        {
-            const uint16_t* vb = Vp + ((int64_t)(kbase / kVBlkBf16 + 2 * g) * D + c) * kVBlkBf16;
+    };
+    auto load_v = [&](int kbase) {
+        const uint16_t* vb = Vp + ((int64_t)(kbase / kVBlkBf16 + 2 * g) * D + c) * kVBlkBf16;
 #pragma unroll
-            for (int db = 0; db < DB; ++db)
+        for (int db = 0; db < DB; ++db)
 #pragma unroll
-                for (int t = 0; t < 2; ++t)
-                    vf[db][t] = *(const uint4*)(vb + ((int64_t)t * D + 16 * db) * kVBlkBf16);
-        }
+            for (int t = 0; t < 2; ++t) vf[db][t] = *(const uint4*)(vb + ((int64_t)t * D + 16 * db) * kVBlkBf16);
+    };
+    const int kfirst = chunk_start + wave * kGroup;
+    if (kfirst < chunk_end) {
+        load_k(kfirst);
+        load_v(kfirst);
+    }
+    for (int kbase = kfirst; kbase < chunk_end; kbase += kWaves * kGroup) {
+        const int knext = kbase + kWaves * kGroup;
         // ---- S^T
         f32x4_t s[4];
 #pragma unroll
@@ -131,6 +182,7 @@ __global__ void __launch_bounds__(256) decode_bf16_kernel(DecodeArgs a) {
             for (int ks = 0; ks < KS; ++ks)
                 s[jj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kf[jj][ks]), qf[ks], s[jj], 0, 0, 0);
         }
+        if (knext < chunk_end) load_k(knext);
         const bool tail = kbase + kGroup > chunk_end;
         float mloc = -INFINITY;
 #pragma unroll
@@ -173,6 +225,7 @@ __global__ void __launch_bounds__(256) decode_bf16_kernel(DecodeArgs a) {
                 acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vf[db][t]), pf, acc[db], 0, 0, 0);
             }
         }
+        if (knext < chunk_end) load_v(knext);
     }
     l = wave_sum_over_groups(l);
 
@@ -227,18 +280,18 @@ __device__ inline void i8x4_to_f16x4(uint32_t w, f16x2_t& lo, f16x2_t& hi) {
 __device__ inline uint32_t f16x2_bits(f16x2_t v) { return __builtin_bit_cast(uint32_t, v); }
 
 template <int D>
-__global__ void __launch_bounds__(256) decode_q8_kernel(DecodeArgs a) {
+__global__ void __launch_bounds__(256, 2) decode_q8_kernel(DecodeArgs a) {
     constexpr int KS = D / 32;
     constexpr int DB = D / 16;
     constexpr int NH = D / 64;  // 16-byte K loads per row per lane
     constexpr int NQ = D / kQBlock;
-    const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
-    const int L = min(a.seq_lens ? a.seq_lens[b] : a.len, a.S_max);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kvh = blockIdx.y;
+    int b, split, L;
+    if (!locate_work(a, blockIdx.x, lane, b, split, L)) return;
     const int chunk_start = split * a.chunk;
-    if (chunk_start >= L) return;
     const int chunk_end = min(L, chunk_start + a.chunk);
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c = lane & 15, g = lane >> 4;
 
     // Q^T operands in fp16.  Contraction slot (ks, g, e) is head-dim index
@@ -273,11 +326,12 @@ __global__ void __launch_bounds__(256) decode_q8_kernel(DecodeArgs a) {
     for (int i = 0; i < DB; ++i) acc[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, l = 0.f;
 
-    for (int kbase = chunk_start + wave * kGroup; kbase < chunk_end; kbase += kWaves * kGroup) {
-        const bool tail = kbase + kGroup > chunk_end;
-        // ---- loads
-        uint4 kq[4][NH];
-        uint16_t ksc[4][NH];
+    // loads of one 64-key group; rotated like the bf16 kernel (K re-issued after S^T, V after O^T)
+    uint4 kq[4][NH];
+    uint16_t ksc[4][NH];
+    uint4 vq[DB];
+    uint4 vsc[NQ][2];
+    auto load_k = [&](int kbase) {
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj) {
             const int64_t key = kbase + krow + 4 * jj;
@@ -287,19 +341,26 @@ __global__ void __launch_bounds__(256) decode_q8_kernel(DecodeArgs a) {
                 ksc[jj][h] = KSp[key * NQ + 2 * h + (g >> 1)];
             }
         }
-        uint4 vq[DB];
-        uint4 vsc[NQ][2];
-        {
-            const int64_t blk = kbase / kVBlkQ8 + g;
+    };
+    auto load_v = [&](int kbase) {
+        const int64_t blk = kbase / kVBlkQ8 + g;
 #pragma unroll
-            for (int db = 0; db < DB; ++db) vq[db] = *(const uint4*)(Vp + (blk * D + 16 * db + c) * kVBlkQ8);
+        for (int db = 0; db < DB; ++db) vq[db] = *(const uint4*)(Vp + (blk * D + 16 * db + c) * kVBlkQ8);
 #pragma unroll
-            for (int qb = 0; qb < NQ; ++qb) {
-                const uint4* sp = (const uint4*)(VSp + (blk * NQ + qb) * kVBlkQ8);
-                vsc[qb][0] = sp[0];
-                vsc[qb][1] = sp[1];
-            }
+        for (int qb = 0; qb < NQ; ++qb) {
+            const uint4* sp = (const uint4*)(VSp + (blk * NQ + qb) * kVBlkQ8);
+            vsc[qb][0] = sp[0];
+            vsc[qb][1] = sp[1];
         }
+    };
+    const int kfirst = chunk_start + wave * kGroup;
+    if (kfirst < chunk_end) {
+        load_k(kfirst);
+        load_v(kfirst);
+    }
+    for (int kbase = kfirst; kbase < chunk_end; kbase += kWaves * kGroup) {
+        const bool tail = kbase + kGroup > chunk_end;
+        const int knext = kbase + kWaves * kGroup;
         // ---- S^T
         f32x4_t s[4];
 #pragma unroll
@@ -324,6 +385,7 @@ __global__ void __launch_bounds__(256) decode_q8_kernel(DecodeArgs a) {
                 s[jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(k1, qf[2 * h + 1], s[jj], 0, 0, 0);
             }
         }
+        if (knext < chunk_end) load_k(knext);
         float mloc = -INFINITY;
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj)
@@ -373,6 +435,7 @@ __global__ void __launch_bounds__(256) decode_q8_kernel(DecodeArgs a) {
             acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, v0), pf[0], acc[db], 0, 0, 0);
             acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, v1), pf[1], acc[db], 0, 0, 0);
         }
+        if (knext < chunk_end) load_v(knext);
     }
     l = wave_sum_over_groups(l);
 
@@ -416,14 +479,14 @@ __global__ void __launch_bounds__(256) decode_q8_kernel(DecodeArgs a) {
 // ---------------------------------------------------------------------------------------------
 template <int MAXD>
 __global__ void __launch_bounds__(256) decode_f32_kernel(DecodeArgs a, int D) {
-    const int split = blockIdx.x, hq = blockIdx.y, b = blockIdx.z;
-    const int L = min(a.seq_lens ? a.seq_lens[b] : a.len, a.S_max);
+    const int tid = threadIdx.x;
+    const int hq = blockIdx.y;
+    int b, split, L;
+    if (!locate_work(a, blockIdx.x, tid & 63, b, split, L)) return;
     const int chunk_start = split * a.chunk;
-    if (chunk_start >= L) return;
     const int chunk_end = min(L, chunk_start + a.chunk);
     const int n = chunk_end - chunk_start;
     const int kvh = hq / a.n_rep;
-    const int tid = threadIdx.x;
 
     extern __shared__ float smem[];
     float* sq = smem;              // [MAXD]
@@ -509,10 +572,26 @@ __global__ void __launch_bounds__(256) decode_combine_kernel(const float* __rest
     float M = -INFINITY;
     for (int s = 0; s < ns; ++s) M = fmaxf(M, ws_ml[(row0 + s) * 2]);
     float o = 0.f, l = 0.f;
-    for (int s = 0; s < ns; ++s) {
+    const float* po = ws_o + row0 * D + (d < D ? d : 0);
+    int s = 0;
+    for (; s + 4 <= ns; s += 4) {  // four independent loads in flight; the sums keep a fixed order
+        const float x0 = po[(int64_t)(s + 0) * D], x1 = po[(int64_t)(s + 1) * D];
+        const float x2 = po[(int64_t)(s + 2) * D], x3 = po[(int64_t)(s + 3) * D];
+        const float w0 = exp2f(ws_ml[(row0 + s + 0) * 2] - M), w1 = exp2f(ws_ml[(row0 + s + 1) * 2] - M);
+        const float w2 = exp2f(ws_ml[(row0 + s + 2) * 2] - M), w3 = exp2f(ws_ml[(row0 + s + 3) * 2] - M);
+        l += w0 * ws_ml[(row0 + s + 0) * 2 + 1];
+        l += w1 * ws_ml[(row0 + s + 1) * 2 + 1];
+        l += w2 * ws_ml[(row0 + s + 2) * 2 + 1];
+        l += w3 * ws_ml[(row0 + s + 3) * 2 + 1];
+        o += w0 * x0;
+        o += w1 * x1;
+        o += w2 * x2;
+        o += w3 * x3;
+    }
+    for (; s < ns; ++s) {
         const float w = exp2f(ws_ml[(row0 + s) * 2] - M);
         l += w * ws_ml[(row0 + s) * 2 + 1];
-        if (d < D) o += w * ws_o[(row0 + s) * D + d];
+        o += w * po[(int64_t)s * D];
     }
     if (d < D) {
         const float r = ns > 0 ? o / l : 0.f;
@@ -535,18 +614,22 @@ int device_cu_count() {
     return cus;
 }
 
-// Tokens per split.  Small enough that the (ragged) work spreads over all CUs with a short tail,
-// large enough that partials stay a few percent of the KV bytes.  Workspace sizing assumes >= 256.
-int pick_chunk(int64_t B, int64_t Hkv, int64_t max_len) {
+// Tokens per split.  Every work item pays a fixed cost (locating itself, loading Q, merging four
+// wavefronts, writing a partial), so splits should be as long as the balance over the chip allows:
+// the largest candidate that still yields at least four work items per CU (counted with the host's
+// upper bound of the lengths).  The quantised kernel has the heavier per-item cost and the lighter
+// stream, hence its larger cap.  Workspace sizing assumes >= 256.
+int pick_chunk(int format, int64_t B, int64_t Hkv, int64_t max_len) {
     static int forced = -1;
     if (forced < 0) {
         const char* e = getenv("VSP_DECODE_CHUNK");
         forced = e ? atoi(e) : 0;
-        if (forced != 0 && (forced < 256 || forced % 256 != 0 || forced > 8192)) forced = 0;
+        if (forced != 0 && (forced < 256 || forced % 256 != 0 || forced > 16384)) forced = 0;
     }
     if (forced > 0) return forced;
-    const int64_t want = 24LL * device_cu_count();
-    for (int chunk : {1024, 512}) {
+    const int64_t want = 4LL * device_cu_count();
+    const int cap = format == VSP_KV_Q8_0 ? 8192 : 1024;
+    for (int chunk = cap; chunk > 256; chunk >>= 1) {
         if (B * Hkv * ceil_div(max_len, chunk) >= want) return chunk;
     }
     return 256;
@@ -591,7 +674,7 @@ int vsp_attn_decode(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_
     if (max_len == 0) max_len = seq_lens ? cache->S_max : cache->len;
     hipStream_t st = (hipStream_t)stream;
 
-    const int chunk = max_len > 0 ? pick_chunk(B, cache->Hkv, max_len) : 256;
+    const int chunk = max_len > 0 ? pick_chunk(cache->format, B, cache->Hkv, max_len) : 256;
     const int max_splits = max_len > 0 ? (int)ceil_div(max_len, chunk) : 1;
     const size_t need = (size_t)(B * Hq * max_splits * (D + 2) * 4);
     if (max_len > 0) {
@@ -608,6 +691,7 @@ int vsp_attn_decode(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_
     a.v_scale = cache->v_scale;
     a.seq_lens = seq_lens;
     a.len = cache->len;
+    a.B = (int)B;
     a.Hq = (int)Hq;
     a.Hkv = cache->Hkv;
     a.n_rep = n_rep;
@@ -621,15 +705,15 @@ int vsp_attn_decode(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_
 
     if (max_len > 0) {
         if (cache->format == VSP_KV_BF16) {
-            dim3 grid(max_splits, cache->Hkv, (unsigned)B);
+            dim3 grid((unsigned)(max_splits * B), cache->Hkv);
             if (D == 128) hipLaunchKernelGGL(decode_bf16_kernel<128>, grid, dim3(256), 0, st, a);
             else hipLaunchKernelGGL(decode_bf16_kernel<64>, grid, dim3(256), 0, st, a);
         } else if (cache->format == VSP_KV_Q8_0) {
-            dim3 grid(max_splits, cache->Hkv, (unsigned)B);
+            dim3 grid((unsigned)(max_splits * B), cache->Hkv);
             if (D == 128) hipLaunchKernelGGL(decode_q8_kernel<128>, grid, dim3(256), 0, st, a);
             else hipLaunchKernelGGL(decode_q8_kernel<64>, grid, dim3(256), 0, st, a);
         } else {
-            dim3 grid(max_splits, (unsigned)Hq, (unsigned)B);
+            dim3 grid((unsigned)(max_splits * B), (unsigned)Hq);
             const size_t smem = (256 + chunk + 256) * sizeof(float);
             hipLaunchKernelGGL(decode_f32_kernel<256>, grid, dim3(256), smem, st, a, (int)D);
         }
