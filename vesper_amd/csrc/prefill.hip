@@ -103,9 +103,21 @@ __global__ void __launch_bounds__(256, 3) prefill_bf16_kernel(PrefillArgs a) {
     __shared__ __attribute__((aligned(1024))) uint16_t sV0[SLOT];
     __shared__ __attribute__((aligned(1024))) uint16_t sV1[SLOT];
 
+    // Block order: heaviest query tiles first (causal work grows with the tile index).  Within one
+    // query-tile row, workgroups are dealt round-robin to the 8 XCDs by the hardware (id % 8); when the
+    // number of (batch, kv head) groups is a multiple of 8, all query heads of a kv group are given ids
+    // of the same residue, so a group's K/V stays in one XCD's L2 instead of being fetched into all eight.
     const int bid = blockIdx.x;
-    const int qt = a.n_qtiles - 1 - bid / (a.B * a.Hq);
-    const int bh = bid % (a.B * a.Hq);
+    const int nbh = a.B * a.Hq;
+    const int qt = a.n_qtiles - 1 - bid / nbh;
+    const int pos = bid % nbh;
+    int bh = pos;
+    const int ngroups = a.B * a.Hkv;
+    if ((ngroups & 7) == 0) {
+        const int xcd = pos & 7, slot = pos >> 3;
+        const int grp = xcd + 8 * (slot / a.n_rep);
+        bh = grp * a.n_rep + slot % a.n_rep;  // == b * Hq + hq, because groups are numbered b * Hkv + kvh
+    }
     const int b = bh / a.Hq, hq = bh % a.Hq, kvh = hq / a.n_rep;
 
     const int tid = threadIdx.x, lane = tid & 63;
