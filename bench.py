@@ -185,6 +185,18 @@ def cpu_baseline(key):
                 seconds=dt * reps)
 
 
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs of this
+# script (summaries under profiles/). The raw counters are scaled by what they read for a 1 GiB read + 1 GiB write
+# elementwise kernel launched by --copy-calibration: FETCH_SIZE x 2.0 = KiB, WRITE_SIZE x 1.0 = KiB. Counters
+# cannot be collected inside a timed run, so these are constants of the workload shapes, not live values.
+MEASURED_TRAFFIC = {
+    "c2": {"fetch_bytes": 64616 * 2 * 1024, "write_bytes": 65730 * 1024, "algorithmic_bytes": 96 * 2**20 + 65 * 2**20},
+    "c3": {"fetch_bytes": 66900 * 2 * 1024, "write_bytes": 65554 * 1024, "algorithmic_bytes": 96 * 2**20 + 65 * 2**20},
+    "c4": {"fetch_bytes": 1280065 * 2 * 1024, "write_bytes": 10880 * 1024, "algorithmic_bytes": 2614935552},
+    "c5": {"fetch_bytes": 1115375 * 2 * 1024, "write_bytes": 4352 * 1024, "algorithmic_bytes": 2282225664},
+}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -236,7 +248,8 @@ def main():
                    "algorithmic_work_per_step": primary.work,
                    "work_unit": "FLOP" if primary.bound == "mfma" else "bytes"},
         "roofline": {"bound": primary.bound, "achieved": round(achieved, 3), "peak": primary.peak,
-                     "unit": primary.unit, "frac": round(achieved / primary.peak, 4), "traffic": None,
+                     "unit": primary.unit, "frac": round(achieved / primary.peak, 4),
+                     "traffic": MEASURED_TRAFFIC.get(args.workload),
                      "kernel": primary.kernel, "kernel_ms": round(dev * 1e3, 5),
                      "timing": "HIP events on the launch stream around the timed steps / steps"},
         "device": {"name": props.name, "cus": props.multi_processor_count,
