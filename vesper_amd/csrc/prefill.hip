@@ -25,6 +25,8 @@
 // the mask is evaluated only on tiles that straddle it.
 #include <math.h>
 
+#include <utility>
+
 #include "vsp_common.hpp"
 
 namespace vsp {
@@ -78,6 +80,27 @@ __device__ inline void tr_wait(uint2& a0, uint2& a1, uint2& a2, uint2& a3, uint2
 __device__ inline void tr_wait(uint2& a0, uint2& a1, uint2& a2, uint2& a3) {
     asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3));
 }
+// Plain 16-byte LDS read through inline asm, for the same reason; lds_wait<N>() waits until at most N of
+// this wave's LDS operations are outstanding (they return in order) and ties the wait to a value.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+template <int OFFSET_BYTES>
+__device__ inline u32x4_t lds_read_b128_asm(uint32_t lds_byte_addr) {
+    u32x4_t v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(lds_byte_addr), "n"(OFFSET_BYTES));
+    return v;
+}
+template <int N>
+__device__ inline void lds_wait(u32x4_t& a0) {
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(a0) : "n"(N));
+}
+template <int... I, class F>
+__device__ inline void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ inline void static_for(F&& f) {
+    static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
 __device__ inline uint32_t lds_addr(const void* p) {
     return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
 }
@@ -98,10 +121,11 @@ __global__ void __launch_bounds__(256, 3) prefill_bf16_kernel(PrefillArgs a) {
     constexpr int NKB = kUnit / 32;   // 32-key S^T blocks per tile
     constexpr int NJ = kUnit / 16;    // PV k-steps per tile
 
-    __shared__ __attribute__((aligned(1024))) uint16_t sK0[SLOT];
-    __shared__ __attribute__((aligned(1024))) uint16_t sK1[SLOT];
-    __shared__ __attribute__((aligned(1024))) uint16_t sV0[SLOT];
-    __shared__ __attribute__((aligned(1024))) uint16_t sV1[SLOT];
+    // Ring slots: K0 | K1 | V0 | V1, SLOT elements each.  Every read of them is issued from inline asm with
+    // the slot as an immediate offset, so the per-lane read addresses are loop constants.
+    __shared__ __attribute__((aligned(1024))) uint16_t smem[4 * SLOT];
+    constexpr int SLOTB = 2 * SLOT;  // bytes per slot
+    const uint32_t lds0 = lds_addr(smem);
 
     // Block order: heaviest query tiles first (causal work grows with the tile index).  Within one
     // query-tile row, workgroups are dealt round-robin to the 8 XCDs by the hardware (id % 8); when the
@@ -172,11 +196,13 @@ __global__ void __launch_bounds__(256, 3) prefill_bf16_kernel(PrefillArgs a) {
         voffV[i] = (uint32_t)r * (uint32_t)a.sv[2] * 2u + 16u * (uint32_t)(ld_pos ^ (((r / RP) % (CPR / 4)) << 2));
     }
     const int64_t rowK = a.sk[2] * 2, rowV = a.sv[2] * 2;  // bytes per key row
-    auto load_tile = [&](int t, uint16_t* dstK, uint16_t* dstV) {
+    auto load_tile = [&](int t, int slot) {
         const int key0 = t * kUnit;
         const int rows = a.L - key0;  // > 0
         __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)Kp + (int64_t)key0 * rowK), 0, (int)((int64_t)rows * rowK), 0x00020000);
         __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)Vp + (int64_t)key0 * rowV), 0, (int)((int64_t)rows * rowV), 0x00020000);
+        uint16_t* dstK = smem + slot * SLOT;
+        uint16_t* dstV = smem + (2 + slot) * SLOT;
 #pragma unroll
         for (int i = 0; i < NLD; ++i) {
             const int grp = wave + 4 * i;
@@ -186,47 +212,56 @@ __global__ void __launch_bounds__(256, 3) prefill_bf16_kernel(PrefillArgs a) {
         }
     };
 
+    // Loop-constant LDS read addresses (slot 0; the slot is an immediate offset on the instruction).
     const int kswz = (ql / RP) % CPR;
+    uint32_t kaddr[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) kaddr[ks] = lds0 + 2u * (uint32_t)(ql * D + 8 * ((2 * ks + h) ^ kswz));
     const int i16 = lane & 15;
     const int vswz = ((i16 >> 2) / RP) % (CPR / 4);
     const int v_lane_off = (4 * h + (i16 >> 2)) * D + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+    uint32_t va[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) va[db] = lds0 + 2u * (uint32_t)v_lane_off + 64u * (uint32_t)(db ^ vswz);
 
-    auto tile_step = [&](int t, const uint16_t* sK, const uint16_t* sV, uint16_t* nextK, uint16_t* nextV) {
+    constexpr int PF = 4;  // K fragments in flight
+
+    auto tile_step = [&](int t, auto slot_c) {
+        constexpr int slot = decltype(slot_c)::value;
+        constexpr int KOFF = slot * SLOTB;
+        constexpr int VOFF = (2 + slot) * SLOTB;
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if (t + 1 < n_tiles) load_tile(t + 1, nextK, nextV);
+        if (t + 1 < n_tiles) load_tile(t + 1, slot ^ 1);
         const int k0 = t * kUnit;
         if (k0 >= kv_end_wave) return;
 
+        static_assert(NKB == 1, "one 32-key block per tile");
         f32x16_t s[NKB];
 #pragma unroll
-        for (int kb = 0; kb < NKB; ++kb) {
-#pragma unroll
-            for (int j = 0; j < 16; ++j) s[kb][j] = 0.f;
-            const uint16_t* kr = sK + (32 * kb + ql) * D;
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                bf16x8_t kf = __builtin_bit_cast(bf16x8_t, *(const uint4*)(kr + 8 * ((2 * ks + h) ^ kswz)));
-                s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], s[kb], 0, 0, 0);
-            }
-        }
+        for (int j = 0; j < 16; ++j) s[0][j] = 0.f;
+        u32x4_t kf[KS];
+        static_for<PF>([&](auto i) { kf[i.value] = lds_read_b128_asm<KOFF>(kaddr[i.value]); });
+        static_for<KS>([&](auto i) {
+            constexpr int ks = i.value;
+            constexpr int issued = (ks + PF < KS) ? ks + PF : KS;
+            lds_wait<issued - ks - 1>(kf[ks]);
+            s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kf[ks]), qf[ks], s[0], 0, 0, 0);
+            if constexpr (ks + PF < KS) kf[ks + PF] = lds_read_b128_asm<KOFF>(kaddr[ks + PF]);
+        });
         const bool need_mask = (a.causal && k0 + kUnit - 1 > q0 + off) || (k0 + kUnit > a.L);
         if (need_mask) {
             const int q_abs = q0 + ql + off;
             const int lim = a.causal ? min(q_abs, a.L - 1) : a.L - 1;
 #pragma unroll
-            for (int kb = 0; kb < NKB; ++kb)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int key = k0 + 32 * kb + 8 * (v >> 2) + 4 * h + (v & 3);
-                    if (key > lim) s[kb][v] = -INFINITY;
-                }
+            for (int v = 0; v < 16; ++v) {
+                const int key = k0 + 8 * (v >> 2) + 4 * h + (v & 3);
+                if (key > lim) s[0][v] = -INFINITY;
+            }
         }
         float mx = s[0][0];
 #pragma unroll
-        for (int kb = 0; kb < NKB; ++kb)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[kb][v]);
+        for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[0][v]);
         mx = half_swap_max(mx) * a.scale_log2;
         if (__any(mx > m_ref + kRescaleThreshold)) {
             const float m_new = fmaxf(m_ref, mx);
@@ -242,37 +277,30 @@ __global__ void __launch_bounds__(256, 3) prefill_bf16_kernel(PrefillArgs a) {
         uint32_t pw[NJ][4];
         float lsum = 0.f;
 #pragma unroll
-        for (int kb = 0; kb < NKB; ++kb)
-#pragma unroll
-            for (int v = 0; v < 16; v += 2) {
-                const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][v], a.scale_log2, neg_m));
-                const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][v + 1], a.scale_log2, neg_m));
-                const uint32_t pk = cvt_pk_bf16(p0, p1);
-                pw[2 * kb + (v >> 3)][(v & 7) >> 1] = pk;
-                lsum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pk), __builtin_bit_cast(bf16x2_t, 0x3f803f80u), lsum, false);
-            }
+        for (int v = 0; v < 16; v += 2) {
+            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[0][v], a.scale_log2, neg_m));
+            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[0][v + 1], a.scale_log2, neg_m));
+            const uint32_t pk = cvt_pk_bf16(p0, p1);
+            pw[v >> 3][(v & 7) >> 1] = pk;
+            lsum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pk), __builtin_bit_cast(bf16x2_t, 0x3f803f80u), lsum, false);
+        }
         l += lsum;
         // PV
-        const uint32_t vb = lds_addr(sV) + 2u * (uint32_t)v_lane_off;
-        uint32_t va[DB];
-#pragma unroll
-        for (int db = 0; db < DB; ++db) va[db] = vb + 64u * (uint32_t)(db ^ vswz);
         uint2 tcur[DB][2], tnext[DB][2];
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
-            tcur[db][0] = lds_read_tr16_b64_asm<0>(va[db]);
-            tcur[db][1] = lds_read_tr16_b64_asm<8 * D * 2>(va[db]);
+            tcur[db][0] = lds_read_tr16_b64_asm<VOFF>(va[db]);
+            tcur[db][1] = lds_read_tr16_b64_asm<VOFF + 8 * D * 2>(va[db]);
         }
-#pragma unroll
-        for (int j = 0; j < NJ; ++j) {
+        static_for<NJ>([&](auto jc) {
+            constexpr int j = jc.value;
             if constexpr (DB == 4) tr_wait(tcur[0][0], tcur[0][1], tcur[1][0], tcur[1][1], tcur[2][0], tcur[2][1], tcur[3][0], tcur[3][1]);
             else tr_wait(tcur[0][0], tcur[0][1], tcur[1][0], tcur[1][1]);
-            if (j + 1 < NJ) {
+            if constexpr (j + 1 < NJ) {
 #pragma unroll
                 for (int db = 0; db < DB; ++db) {
-                    if (j == 0) { tnext[db][0] = lds_read_tr16_b64_asm<16 * D * 2>(va[db]); tnext[db][1] = lds_read_tr16_b64_asm<24 * D * 2>(va[db]); }
-                    if (j == 1) { tnext[db][0] = lds_read_tr16_b64_asm<32 * D * 2>(va[db]); tnext[db][1] = lds_read_tr16_b64_asm<40 * D * 2>(va[db]); }
-                    if (j == 2) { tnext[db][0] = lds_read_tr16_b64_asm<48 * D * 2>(va[db]); tnext[db][1] = lds_read_tr16_b64_asm<56 * D * 2>(va[db]); }
+                    tnext[db][0] = lds_read_tr16_b64_asm<VOFF + (16 * (j + 1)) * D * 2>(va[db]);
+                    tnext[db][1] = lds_read_tr16_b64_asm<VOFF + (16 * (j + 1) + 8) * D * 2>(va[db]);
                 }
             }
             const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, uint4{pw[j][0], pw[j][1], pw[j][2], pw[j][3]});
@@ -281,20 +309,20 @@ __global__ void __launch_bounds__(256, 3) prefill_bf16_kernel(PrefillArgs a) {
                 const bf16x8_t vf = __builtin_bit_cast(bf16x8_t, uint4{tcur[db][0].x, tcur[db][0].y, tcur[db][1].x, tcur[db][1].y});
                 acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf, acc[db], 0, 0, 0);
             }
-            if (j + 1 < NJ) {
+            if constexpr (j + 1 < NJ) {
 #pragma unroll
                 for (int db = 0; db < DB; ++db) {
                     tcur[db][0] = tnext[db][0];
                     tcur[db][1] = tnext[db][1];
                 }
             }
-        }
+        });
     };
 
-    if (n_tiles > 0) load_tile(0, sK0, sV0);
+    if (n_tiles > 0) load_tile(0, 0);
     for (int t = 0; t < n_tiles; t += 2) {
-        tile_step(t, sK0, sV0, sK1, sV1);
-        if (t + 1 < n_tiles) tile_step(t + 1, sK1, sV1, sK0, sV0);
+        tile_step(t, std::integral_constant<int, 0>{});
+        if (t + 1 < n_tiles) tile_step(t + 1, std::integral_constant<int, 1>{});
     }
 
     l = half_swap_sum(l);
