@@ -135,6 +135,28 @@ int vsp_kv_cache_reset(vsp_kv_cache* cache, void* stream);
 int vsp_kv_append(vsp_kv_cache* cache, const vsp_tensor* new_k, const vsp_tensor* new_v, int64_t start_pos,
                   const int32_t* start_pos_dev, void* stream);
 
+/* The step before the cache write in the attention modules, fused with it: rotary position embedding of
+ * q and k (functional::compute_rope_frequencies + functional::apply_rotary_emb,
+ * src/nn/functional.cpp:424-494, as called at src/nn/gqa_attention.cpp:124-130 and
+ * src/nn/transformer.cpp:184-189) followed by KVCache::update's write (above).  One launch replaces the
+ * reference's host-side angle table + upload, ~10 elementwise/stack/permute/contiguous launches per
+ * tensor, and the strided cache copy.
+ *   q [B,Hq,T,D], new_k/new_v [B,Hkv,T,D] (shape must equal the cache's B,Hkv,D): fp32 or bf16, one
+ *   dtype, any strides with stride[3]==1 -- so the three can be strided views of one fused projection
+ *   output [B,T,(Hq+2Hkv)*D] and the reference's transpose copies (src/nn/gqa_attention.cpp:120-122)
+ *   disappear.  q_out [B,Hq,T,D] fp32 or bf16 (may alias q when dtypes match).
+ *   rope_table: device float [table_len][D/2][2] = {cos, sin} of the angle of absolute position p and
+ *   pair i, filled by vsp_rope_fill_table() (8-byte aligned).  Row b, token t uses position
+ *   start_pos + t (or start_pos_dev[b] + t); without start_pos_dev the range must lie inside the
+ *   table (else VSP_ERR_ARG); device-side positions past the table are clamped to its last row.
+ * Arithmetic: pairs (2i, 2i+1); out[2i] = x0*cos - x1*sin, out[2i+1] = x0*sin + x1*cos in fp32 with each
+ * product and sum rounded separately (bit-identical to the reference's separate elementwise ops); bf16
+ * inputs are widened exactly first; conversion into the cache format as in vsp_kv_append.  V is not
+ * rotated.  Slot placement, clamping, errors and the len update are those of vsp_kv_append. */
+int vsp_rope_kv_append(vsp_kv_cache* cache, const vsp_tensor* q, const vsp_tensor* new_k, const vsp_tensor* new_v,
+                       vsp_tensor* q_out, const float* rope_table, int64_t table_len, int64_t start_pos,
+                       const int32_t* start_pos_dev, void* stream);
+
 /* The read half of KVCache::update, :75-92: the reference returns VIEWS [:, :, 0:len, :] of its fp32
  * storage.  For VSP_KV_F32 the same view can be formed by the caller (vsp_kv_view_f32); for the other
  * formats this call materialises logical rows [start, start+count) into k_out/v_out
@@ -187,6 +209,11 @@ uint16_t vsp_f32_to_f16(float f);    /* IEEE RNE */
 float vsp_f16_to_f32(uint16_t h);
 void vsp_q8_0_quantize_row(const float* x, int64_t n, uint16_t* scale, int8_t* qs);
 void vsp_q8_0_dequantize_row(const uint16_t* scale, const int8_t* qs, int64_t n, float* x);
+/* Host-side RoPE table: table[m][i] = {cosf(a), sinf(a)}, a = (float)(start_pos + m) * powf(theta,
+ * -2.0f * i / D), m < count, i < D/2 -- the angles of functional::compute_rope_frequencies
+ * (src/nn/functional.cpp:424-443) through ops::cos / ops::sin (std::cos / std::sin on float,
+ * src/ops/elementwise.cpp:1039-1045).  The caller uploads it once per (D, theta). */
+void vsp_rope_fill_table(float* table, int32_t start_pos, int32_t count, int32_t D, float theta);
 /* The reference's slice clamping for one dimension (src/ops/view_ops.cpp:270-316, step 1). */
 void vsp_slice_bounds(int64_t dim_size, int64_t start, int64_t stop, int64_t* out_start, int64_t* out_len);
 /* GroupedQueryAttention constructor arithmetic and checks (src/nn/gqa_attention.cpp:38-57). */

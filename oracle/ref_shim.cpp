@@ -217,6 +217,48 @@ int vref_gqa_ctor(int64_t embed_dim, int64_t num_heads, int64_t num_kv_heads, in
     });
 }
 
+// functional::compute_rope_frequencies (src/nn/functional.cpp:424-443): angles [seq_len][head_dim/2].
+int vref_rope_frequencies(int seq_len, int head_dim, int start_pos, float theta, float* angles) {
+    return guarded([&] {
+        Tensor f = vesper::nn::functional::compute_rope_frequencies(seq_len, head_dim, start_pos, theta, Device::CPU);
+        to_host(f, angles);
+    });
+}
+// functional::apply_rotary_emb (src/nn/functional.cpp:445-494): x [B,H,S,D], angles [S][D/2].
+int vref_apply_rotary_emb(const float* x, int64_t B, int64_t H, int64_t S, int64_t D, const float* angles,
+                          float* out) {
+    return guarded([&] {
+        Tensor tx = from_host(x, {B, H, S, D});
+        Tensor tf = from_host(angles, {S, D / 2});
+        Tensor o = vesper::nn::functional::apply_rotary_emb(tx, tf);
+        to_host(o, out);
+    });
+}
+// The attention module's own sequence with a cache (src/nn/gqa_attention.cpp:124-141): RoPE on q and k
+// at start_pos, cache update, repeat_kv, attention.  Returns the rotated q and the attention output.
+int vref_gqa_rope_core(void* c, const float* q, const float* new_k, const float* new_v,
+                       int64_t B, int64_t Hq, int64_t Hkv, int64_t T, int64_t D,
+                       int start_pos, float theta, float* q_rot, float* out) {
+    return guarded([&] {
+        auto* cache = static_cast<vesper::nn::KVCache*>(c);
+        Tensor tq = from_host(q, {B, Hq, T, D});
+        Tensor k = from_host(new_k, {B, Hkv, T, D});
+        Tensor v = from_host(new_v, {B, Hkv, T, D});
+        Tensor freqs = vesper::nn::functional::compute_rope_frequencies((int)T, (int)D, start_pos, theta, Device::CPU);
+        tq = vesper::nn::functional::apply_rotary_emb(tq, freqs);
+        k = vesper::nn::functional::apply_rotary_emb(k, freqs);
+        auto kv = cache->update(k, v, start_pos);
+        k = kv.first.contiguous();
+        v = kv.second.contiguous();
+        int64_t n_rep = Hq / Hkv;
+        k = vesper::ops::repeat_kv(k, n_rep);
+        v = vesper::ops::repeat_kv(v, n_rep);
+        Tensor o = vesper::nn::functional::scaled_dot_product_attention(tq, k, v, T > 1, 0.0);
+        to_host(tq, q_rot);
+        to_host(o, out);
+    });
+}
+
 // BFloat16(float) / operator float (include/vesper/core/half.h:162-181).
 uint16_t vref_f32_to_bf16(float f) { return vesper::BFloat16(f).to_bits(); }
 float vref_bf16_to_f32(uint16_t b) { return float(vesper::BFloat16::from_bits(b)); }

@@ -457,3 +457,36 @@ void orc_q8_0_dequantize_row(const uint16_t* d, const int8_t* qs, int64_t n, flo
         for (int j = 0; j < 32; ++j) x[i * 32 + j] = (float)qs[i * 32 + j] * dd;
     }
 }
+
+/* ---- rotary position embedding ----------------------------------------- */
+
+/* src/nn/functional.cpp:424-443.  `-2.0f * i / dim` is evaluated in float left to right
+ * ((-2.0f * (float)i) / (float)dim); std::pow(float, float) is powf; `pos * freq` converts the int
+ * position to float. */
+void orc_rope_angles(int seq_len, int head_dim, int start_pos, float theta, float* angles) {
+    const int half = head_dim / 2;
+    for (int m = 0; m < seq_len; ++m) {
+        const int pos = start_pos + m;
+        for (int i = 0; i < half; ++i) {
+            const float freq = powf(theta, -2.0f * (float)i / (float)head_dim);
+            angles[(int64_t)m * half + i] = (float)pos * freq;
+        }
+    }
+}
+
+/* src/nn/functional.cpp:445-494. */
+void orc_rope_apply_f32(const float* x, int64_t B, int64_t H, int64_t S, int64_t D, const float* angles,
+                        float* out) {
+    const int64_t half = D / 2;
+    for (int64_t bh = 0; bh < B * H; ++bh)
+        for (int64_t s = 0; s < S; ++s)
+            for (int64_t i = 0; i < half; ++i) {
+                const float a = angles[s * half + i];
+                const float c = cosf(a), sn = sinf(a);
+                const int64_t o = (bh * S + s) * D + 2 * i;
+                const float x0 = x[o], x1 = x[o + 1];
+                const float t1 = x0 * c, t2 = x1 * sn, t3 = x0 * sn, t4 = x1 * c;
+                out[o] = t1 - t2;
+                out[o + 1] = t3 + t4;
+            }
+}

@@ -158,6 +158,18 @@ float orc_f16_to_f32(uint16_t h);
 void orc_q8_0_quantize_row(const float* x, int64_t n, uint16_t* d, int8_t* qs);
 void orc_q8_0_dequantize_row(const uint16_t* d, const int8_t* qs, int64_t n, float* x);
 
+/* ---- rotary position embedding (the step before the cache append) ------ */
+
+/* compute_rope_frequencies(seq_len, head_dim, start_pos, theta), src/nn/functional.cpp:424-443:
+ * angles[m][i] = (float)(start_pos + m) * powf(theta, -2.0f * i / head_dim), i < head_dim/2. */
+void orc_rope_angles(int seq_len, int head_dim, int start_pos, float theta, float* angles);
+/* apply_rotary_emb(x, freqs), src/nn/functional.cpp:445-494, x [B,H,S,D] contiguous, angles [S][D/2]:
+ * pairs (2i, 2i+1); c = cosf(angle), s = sinf(angle) (ops::cos / ops::sin = std::cos / std::sin on
+ * float, src/ops/elementwise.cpp:1039-1045); out[2i] = x0*c - x1*s, out[2i+1] = x0*s + x1*c with
+ * every product and the sum rounded separately (separate elementwise ops, no fused multiply-add). */
+void orc_rope_apply_f32(const float* x, int64_t B, int64_t H, int64_t S, int64_t D, const float* angles,
+                        float* out);
+
 #ifdef __cplusplus
 }
 #endif

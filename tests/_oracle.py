@@ -74,6 +74,10 @@ def _load_oracle():
     L.orc_q8_0_quantize_row.restype = None
     L.orc_q8_0_dequantize_row.argtypes = [u16p, i8p, i64, f32p]
     L.orc_q8_0_dequantize_row.restype = None
+    L.orc_rope_angles.argtypes = [C.c_int, C.c_int, C.c_int, C.c_float, f32p]
+    L.orc_rope_angles.restype = None
+    L.orc_rope_apply_f32.argtypes = [f32p] + [i64] * 4 + [f32p, f32p]
+    L.orc_rope_apply_f32.restype = None
     return L
 
 
@@ -258,6 +262,21 @@ def q8_0_dequantize(d, qs):
     return out
 
 
+def rope_angles(seq_len, head_dim, start_pos=0, theta=10000.0):
+    out = np.empty((seq_len, head_dim // 2), np.float32)
+    orc.orc_rope_angles(seq_len, head_dim, start_pos, theta, _p(out))
+    return out
+
+
+def rope_apply(x, angles):
+    x, angles = _f32(x), _f32(angles)
+    B, H, S, D = x.shape
+    assert angles.shape == (S, D // 2)
+    out = np.empty_like(x)
+    orc.orc_rope_apply_f32(_p(x), B, H, S, D, _p(angles), _p(out))
+    return out
+
+
 # ---- the compiled reference (optional) ----------------------------------------------------
 
 def _load_ref():
@@ -287,6 +306,10 @@ def _load_ref():
     L.vref_gqacache_update.argtypes = [C.c_void_p, f32p, f32p] + [i64] * 5 + [f32p, f32p]
     L.vref_gqa_core.argtypes = [C.c_void_p, f32p, f32p, f32p] + [i64] * 5 + [C.c_int, C.c_int, f32p]
     L.vref_gqa_ctor.argtypes = [i64, i64, i64, i64p, i64p]
+    if hasattr(L, "vref_rope_frequencies"):
+        L.vref_rope_frequencies.argtypes = [C.c_int, C.c_int, C.c_int, C.c_float, f32p]
+        L.vref_apply_rotary_emb.argtypes = [f32p] + [i64] * 4 + [f32p, f32p]
+        L.vref_gqa_rope_core.argtypes = [C.c_void_p, f32p, f32p, f32p] + [i64] * 5 + [C.c_int, C.c_float, f32p, f32p]
     L.vref_f32_to_bf16.argtypes = [C.c_float]
     L.vref_f32_to_bf16.restype = C.c_uint16
     L.vref_bf16_to_f32.argtypes = [C.c_uint16]
@@ -386,6 +409,32 @@ class RefKVCache:
         _rchk(ref.vref_gqa_core(self._h, _p(q), _p(new_k), _p(new_v), B, Hq, Hkv, T, D, start_pos,
                                 int(make_contiguous), _p(out)))
         return out
+
+
+    def gqa_rope_core(self, q, new_k, new_v, start_pos, theta=10000.0):
+        """RoPE(q, k) at start_pos -> update -> repeat_kv -> attention; returns (rotated q, output)."""
+        assert not self.gqa
+        q, new_k, new_v = _f32(q), _f32(new_k), _f32(new_v)
+        B, Hq, T, D = q.shape
+        Hkv = new_k.shape[1]
+        q_rot, out = np.empty_like(q), np.empty_like(q)
+        _rchk(ref.vref_gqa_rope_core(self._h, _p(q), _p(new_k), _p(new_v), B, Hq, Hkv, T, D, start_pos,
+                                     theta, _p(q_rot), _p(out)))
+        return q_rot, out
+
+
+def ref_rope_angles(seq_len, head_dim, start_pos=0, theta=10000.0):
+    out = np.empty((seq_len, head_dim // 2), np.float32)
+    _rchk(ref.vref_rope_frequencies(seq_len, head_dim, start_pos, theta, _p(out)))
+    return out
+
+
+def ref_rope_apply(x, angles):
+    x, angles = _f32(x), _f32(angles)
+    B, H, S, D = x.shape
+    out = np.empty_like(x)
+    _rchk(ref.vref_apply_rotary_emb(_p(x), B, H, S, D, _p(angles), _p(out)))
+    return out
 
 
 def ref_gqa_ctor(embed_dim, num_heads, num_kv_heads):

@@ -131,6 +131,32 @@ def gqa_core_cases():
     save("gqa_core", **out)
 
 
+def rope_cases():
+    # functional::compute_rope_frequencies + apply_rotary_emb (src/nn/functional.cpp:424-494): angle tables
+    # at several (seq_len, head_dim, start_pos, theta); rotations of seeded inputs; and the cached attention
+    # sequence with RoPE as GroupedQueryAttention::forward(x, cache, start_pos) runs it
+    # (src/nn/gqa_attention.cpp:124-148): prefill 8 tokens, then 3 single-token steps.
+    out = {}
+    cfgs = [(4, 4, 0, 10000.0), (16, 64, 0, 10000.0), (5, 128, 1000, 10000.0), (3, 128, 32765, 500000.0)]
+    out["cfgs"] = np.array(cfgs, np.float64)
+    for ci, (S, D, sp, th) in enumerate(cfgs):
+        ang = O.ref_rope_angles(S, D, sp, th)
+        x = I.normal(8000 + ci, (2, 3, S, D))
+        out[f"c{ci}_angles"] = ang
+        out[f"c{ci}_x_sha"] = np.frombuffer(bytes.fromhex(I.sha(x)), np.uint8)
+        out[f"c{ci}_out"] = O.ref_rope_apply(x, ang)
+    B, Hq, Hkv, D, S_max = 2, 8, 2, 64, 32
+    c = O.RefKVCache(B, Hkv, S_max, D)
+    out["meta"] = np.array([B, Hq, Hkv, D, S_max], np.int64)
+    pos = 0
+    for si, T in enumerate([8, 1, 1, 1]):
+        q, nk, nv = I.qkv(8100 + 10 * si, B, Hq, Hkv, T, T, D)
+        out[f"s{si}_op"] = np.array([T, pos], np.int64)
+        out[f"s{si}_qrot"], out[f"s{si}_out"] = c.gqa_rope_core(q, nk, nv, pos)
+        pos += T
+    save("rope", **out)
+
+
 def bf16_vectors():
     rng = np.random.default_rng(42)
     bits = np.concatenate([
@@ -152,4 +178,5 @@ if __name__ == "__main__":
     repeat_kv_case()
     kv_cache_cases()
     gqa_core_cases()
+    rope_cases()
     bf16_vectors()

@@ -37,6 +37,7 @@ SYMBOLS = {
     "vsp_kv_plane_bytes": (C.c_size_t, [C.c_int32] * 6),
     "vsp_kv_cache_reset": (C.c_int, [_KP, C.c_void_p]),
     "vsp_kv_append": (C.c_int, [_KP, _TP, _TP, C.c_int64, C.c_void_p, C.c_void_p]),
+    "vsp_rope_kv_append": (C.c_int, [_KP, _TP, _TP, _TP, _TP, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]),
     "vsp_kv_read": (C.c_int, [_KP, C.c_int64, C.c_int64, _TP, _TP, C.c_void_p]),
     "vsp_kv_read_q8_0": (C.c_int, [_KP, C.c_int32, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]),
     "vsp_kv_view_f32": (C.c_int, [_KP, _TP, _TP]),
@@ -49,6 +50,7 @@ SYMBOLS = {
     "vsp_f16_to_f32": (C.c_float, [C.c_uint16]),
     "vsp_q8_0_quantize_row": (None, [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]),
     "vsp_q8_0_dequantize_row": (None, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]),
+    "vsp_rope_fill_table": (None, [C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_float]),
     "vsp_slice_bounds": (None, [C.c_int64, C.c_int64, C.c_int64, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
     "vsp_gqa_config": (C.c_int, [C.c_int64, C.c_int64, C.c_int64, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
     "vsp_status_str": (C.c_char_p, [C.c_int]),

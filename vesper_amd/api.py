@@ -60,6 +60,18 @@ def flash_attention(q, k, v, scale, is_causal=True, dropout_p=0.0, training=Fals
     return (out, lse) if return_lse else out
 
 
+class RopeTable:
+    """{cos, sin} of the angles of functional::compute_rope_frequencies (src/nn/functional.cpp:424-443) for
+    absolute positions [0, length): computed once on the host by the library, kept on the device."""
+
+    def __init__(self, length, head_dim, theta=10000.0, device="cuda"):
+        host = torch.empty((length, head_dim // 2, 2), dtype=torch.float32)
+        lib.vsp_rope_fill_table(C.c_void_p(host.data_ptr()), 0, int(length), int(head_dim), float(theta))
+        self.length, self.head_dim, self.theta = int(length), int(head_dim), float(theta)
+        self.host = host
+        self.table = host.to(device)
+
+
 class KVCache:
     """nn::KVCache with selectable storage: fmt 'f32' (the reference's layout), 'bf16' or 'q8_0'."""
 
@@ -99,6 +111,17 @@ class KVCache:
         if not return_views:
             return None
         return self.views()
+
+    def rope_update(self, q, new_k, new_v, start_pos, rope, out_dtype=None, start_pos_dev=None, return_views=False):
+        """Steps 3-4 of the attention modules' cached forward in one launch (src/nn/gqa_attention.cpp:124-130):
+        q and k rotated by `rope` (a RopeTable) at positions start_pos.., k and v written to the cache.
+        Returns the rotated q (and the cache views when asked)."""
+        q_out = torch.empty(q.shape, dtype=out_dtype or q.dtype, device=q.device)
+        dq, dk, dv, do = _desc(q), _desc(new_k), _desc(new_v), _desc(q_out)
+        sp = C.c_void_p(start_pos_dev.data_ptr()) if start_pos_dev is not None else None
+        check(lib.vsp_rope_kv_append(C.byref(self._c), C.byref(dq), C.byref(dk), C.byref(dv), C.byref(do),
+                                     C.c_void_p(rope.table.data_ptr()), rope.length, int(start_pos), sp, _stream(q)))
+        return (q_out, self.views()) if return_views else q_out
 
     # -- reads
     def views(self, dtype=None):
@@ -182,14 +205,19 @@ def scaled_dot_product_attention(q, k, v, is_causal=False, dropout_p=0.0):
     return flash_attention(q, k, v, scale, is_causal=bool(is_causal) and T > 1)
 
 
-def attention_core(q, new_k, new_v, cache=None, start_pos=0):
+def attention_core(q, new_k, new_v, cache=None, start_pos=0, rope=None, q_dtype=None):
     """Steps 4-6 of GroupedQueryAttention::forward(x, cache, start_pos), src/nn/gqa_attention.cpp:128-148
     (== MultiHeadAttention::forward, src/nn/transformer.cpp:190-205, with n_rep = 1):
-    cache.update(k, v, start_pos); repeat_kv (fused); SDPA with use_causal = (T > 1)."""
+    cache.update(k, v, start_pos); repeat_kv (fused); SDPA with use_causal = (T > 1).
+    With `rope` (a RopeTable) step 3 (:124-127) is included: q and k are rotated at start_pos in the same
+    launch that writes the cache; q continues in `q_dtype` (default: its own)."""
     T = q.shape[2]
     if cache is None:
         return scaled_dot_product_attention(q, new_k, new_v, is_causal=(T > 1))
-    cache.update(new_k, new_v, start_pos, return_views=False)
+    if rope is not None:
+        q = cache.rope_update(q, new_k, new_v, start_pos, rope, out_dtype=q_dtype)
+    else:
+        cache.update(new_k, new_v, start_pos, return_views=False)
     if T == 1:
         return decode_attention(q, cache)
     if cache.fmt == "f32":

@@ -116,6 +116,22 @@ void vsp_q8_0_dequantize_row(const uint16_t* scale, const int8_t* qs, int64_t n,
     }
 }
 
+// compute_rope_frequencies (src/nn/functional.cpp:424-443) followed by ops::cos / ops::sin: float
+// arithmetic throughout, `-2.0f * i / dim` evaluated left to right, the int position converted to float.
+void vsp_rope_fill_table(float* table, int32_t start_pos, int32_t count, int32_t D, float theta) {
+    const int32_t half = D / 2;
+    for (int32_t m = 0; m < count; ++m) {
+        const int32_t pos = start_pos + m;
+        for (int32_t i = 0; i < half; ++i) {
+            const float freq = powf(theta, -2.0f * (float)i / (float)D);
+            const float angle = (float)pos * freq;
+            float* e = table + ((int64_t)m * half + i) * 2;
+            e[0] = cosf(angle);
+            e[1] = sinf(angle);
+        }
+    }
+}
+
 void vsp_slice_bounds(int64_t dim_size, int64_t start, int64_t stop, int64_t* out_start, int64_t* out_len) {
     vsp::slice_bounds(dim_size, start, stop, out_start, out_len);
 }

@@ -45,6 +45,16 @@ struct AppendArgs {
     int64_t slot_start, slot_len;
     const int32_t* start_dev;  // per-batch start positions or nullptr
     int64_t rows;              // B*H*slot_len
+    // Rotary embedding fused into the append (ROPE kernels only): K rows are rotated by the table row of
+    // their destination position; the same launch rotates Q into q_out.
+    const float* table;  // [table_len][D/2][2] = {cos, sin}
+    int64_t table_len;
+    const void* q;
+    void* q_out;
+    int64_t sq[3], so[3];  // q / q_out strides of dims 0..2
+    int64_t Hq, T;
+    int64_t kv_items;      // threads of the K/V part; the Q part follows
+    int32_t q_out_bf16;
 };
 
 template <typename SrcT>
@@ -53,6 +63,50 @@ template <>
 __device__ inline float load_src<float>(const float* p) { return *p; }
 template <>
 __device__ inline float load_src<uint16_t>(const uint16_t* p) { return bf16_bits_to_f32(*p); }
+
+// apply_rotary_emb (src/nn/functional.cpp:445-494) on N consecutive elements starting at even d0 of a row
+// at absolute position pos: pairs (2i, 2i+1), every product and sum rounded on its own as the
+// reference's separate elementwise ops do.  Positions past the table are clamped to its last row.
+template <int N>
+__device__ inline void rope_rotate(float (&x)[N], int64_t d0, int64_t pos, const AppendArgs& a) {
+#pragma clang fp contract(off)  // no fused multiply-add: the products are rounded before the sum
+    if (pos >= a.table_len) pos = a.table_len - 1;
+    if (pos < 0) pos = 0;
+    const float2* t = (const float2*)a.table + pos * (a.D / 2) + d0 / 2;
+#pragma unroll
+    for (int j = 0; j < N / 2; ++j) {
+        const float2 cs = t[j];
+        const float x0 = x[2 * j], x1 = x[2 * j + 1];
+        const float t1 = x0 * cs.x, t2 = x1 * cs.y, t3 = x0 * cs.y, t4 = x1 * cs.x;
+        x[2 * j] = t1 - t2;
+        x[2 * j + 1] = t3 + t4;
+    }
+}
+
+// The Q part of the fused launch: item i rotates 8 consecutive d of one query row.
+template <typename SrcT>
+__device__ inline void rope_q_item(const AppendArgs& a, int64_t i) {
+    const int64_t per_row = a.D / 8;
+    const int64_t r = i / per_row, d0 = (i % per_row) * 8;
+    const int64_t t = r % a.T, bh = r / a.T;
+    const int64_t h = bh % a.Hq, b = bh / a.Hq;
+    const int64_t start = a.start_dev ? (int64_t)a.start_dev[b] : a.slot_start;
+    const SrcT* p = (const SrcT*)a.q + b * a.sq[0] + h * a.sq[1] + t * a.sq[2] + d0;
+    float x[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) x[j] = load_src<SrcT>(p + j);
+    rope_rotate<8>(x, d0, start + t, a);
+    const int64_t o = b * a.so[0] + h * a.so[1] + t * a.so[2] + d0;
+    if (a.q_out_bf16) {
+        uint16_t* dst = (uint16_t*)a.q_out + o;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) dst[j] = f32_to_bf16_bits(x[j]);
+    } else {
+        float* dst = (float*)a.q_out + o;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) dst[j] = x[j];
+    }
+}
 
 // Row r of the slot, in the reference's copy order (src/ops/cpu/copy_cpu.cpp:21-37): linear row
 // index decomposed by the slot shape on the destination side and by the source shape on the
@@ -76,10 +130,17 @@ __device__ inline RowMap map_row(const AppendArgs& a, int64_t r) {
 }
 
 // F32 cache: both planes row-major fp32; a thread moves 4 consecutive d.
-template <typename SrcT>
+template <typename SrcT, bool ROPE>
 __global__ void __launch_bounds__(256) append_f32_kernel(AppendArgs a) {
     const int64_t per_row = a.D / 4;
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if constexpr (ROPE) {
+        if (i >= a.kv_items) {
+            i -= a.kv_items;
+            if (i < a.nB * a.Hq * a.T * (a.D / 8)) rope_q_item<SrcT>(a, i);
+            return;
+        }
+    }
     if (i >= a.rows * per_row) return;
     const int64_t r = i / per_row, d0 = (i % per_row) * 4;
     const RowMap m = map_row(a, r);
@@ -87,31 +148,50 @@ __global__ void __launch_bounds__(256) append_f32_kernel(AppendArgs a) {
     const SrcT* pv = (const SrcT*)a.src_v + m.src_off_v + d0;
     float* dk = (float*)a.k + kv_off_rowmajor(a.H, a.S, a.D, m.b, m.h, m.s, d0);
     float* dv = (float*)a.v + kv_off_rowmajor(a.H, a.S, a.D, m.b, m.h, m.s, d0);
+    float xk[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) xk[j] = load_src<SrcT>(pk + j);
+    if constexpr (ROPE) rope_rotate<4>(xk, d0, m.s, a);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        dk[j] = load_src<SrcT>(pk + j);
+        dk[j] = xk[j];
         dv[j] = load_src<SrcT>(pv + j);
     }
 }
 
 // BF16 cache: K row-major, V token-blocked by 8; a thread converts 8 consecutive d.
-template <typename SrcT>
+template <typename SrcT, bool ROPE>
 __global__ void __launch_bounds__(256) append_bf16_kernel(AppendArgs a) {
     const int64_t per_row = a.D / 8;
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if constexpr (ROPE) {
+        if (i >= a.kv_items) {
+            i -= a.kv_items;
+            if (i < a.nB * a.Hq * a.T * (a.D / 8)) rope_q_item<SrcT>(a, i);
+            return;
+        }
+    }
     if (i >= a.rows * per_row) return;
     const int64_t r = i / per_row, d0 = (i % per_row) * 8;
     const RowMap m = map_row(a, r);
     const SrcT* pk = (const SrcT*)a.src_k + m.src_off_k + d0;
     const SrcT* pv = (const SrcT*)a.src_v + m.src_off_v + d0;
     uint16_t kb[8], vb[8];
+    if constexpr (ROPE) {
+        float xk[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) xk[j] = load_src<SrcT>(pk + j);
+        rope_rotate<8>(xk, d0, m.s, a);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) kb[j] = f32_to_bf16_bits(xk[j]);
+    }
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         if constexpr (sizeof(SrcT) == 2) {
-            kb[j] = pk[j];
+            if constexpr (!ROPE) kb[j] = pk[j];
             vb[j] = pv[j];
         } else {
-            kb[j] = f32_to_bf16_bits(pk[j]);
+            if constexpr (!ROPE) kb[j] = f32_to_bf16_bits(pk[j]);
             vb[j] = f32_to_bf16_bits(pv[j]);
         }
     }
@@ -146,10 +226,17 @@ __device__ inline void quantize_block(const float* x, int8_t* q, uint16_t* scale
     for (int j = 0; j < kQBlock; ++j) q[j] = (int8_t)(int)roundf(__fmul_rn(x[j], id));
 }
 
-template <typename SrcT>
+template <typename SrcT, bool ROPE>
 __global__ void __launch_bounds__(128) append_q8_kernel(AppendArgs a) {
     const int64_t per_row = a.D / kQBlock;
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if constexpr (ROPE) {
+        if (i >= a.kv_items) {
+            i -= a.kv_items;
+            if (i < a.nB * a.Hq * a.T * (a.D / 8)) rope_q_item<SrcT>(a, i);
+            return;
+        }
+    }
     if (i >= a.rows * per_row) return;
     const int64_t r = i / per_row, blk = i % per_row, d0 = blk * kQBlock;
     const RowMap m = map_row(a, r);
@@ -161,6 +248,7 @@ __global__ void __launch_bounds__(128) append_q8_kernel(AppendArgs a) {
     // K: row-major int8, scales [s][blk]
 #pragma unroll
     for (int j = 0; j < kQBlock; ++j) x[j] = load_src<SrcT>(pk + j);
+    if constexpr (ROPE) rope_rotate<kQBlock>(x, d0, m.s, a);
     quantize_block(x, q, &sc);
     {
         uint32_t w[8];
@@ -307,8 +395,17 @@ int vsp_kv_cache_reset(vsp_kv_cache* cache, void* stream) {
     return VSP_OK;
 }
 
-int vsp_kv_append(vsp_kv_cache* cache, const vsp_tensor* new_k, const vsp_tensor* new_v, int64_t start_pos,
-                  const int32_t* start_pos_dev, void* stream) {
+// Shared body of vsp_kv_append and vsp_rope_kv_append (rope != nullptr: rotate K on the way in and Q in
+// the tail of the same launch).
+struct RopeParams {
+    const vsp_tensor* q;
+    vsp_tensor* q_out;
+    const float* table;
+    int64_t table_len;
+};
+
+static int append_impl(vsp_kv_cache* cache, const vsp_tensor* new_k, const vsp_tensor* new_v, int64_t start_pos,
+                       const int32_t* start_pos_dev, const RopeParams* rope, void* stream) {
     int rc = check_cache(cache);
     if (rc != VSP_OK) return rc;
     if (!new_k || !new_v) return VSP_ERR_NULL;
@@ -318,6 +415,25 @@ int vsp_kv_append(vsp_kv_cache* cache, const vsp_tensor* new_k, const vsp_tensor
     for (int i = 0; i < 4; ++i)
         if (new_k->shape[i] < 0 || new_k->shape[i] != new_v->shape[i]) return VSP_ERR_NUMEL;
     const int64_t T = new_k->shape[2];
+    if (rope) {
+        const vsp_tensor* q = rope->q;
+        const vsp_tensor* qo = rope->q_out;
+        if (!q || !qo || !rope->table) return VSP_ERR_NULL;
+        if (q->ndim != 4 || qo->ndim != 4) return VSP_ERR_NDIM;
+        if (q->dtype != new_k->dtype) return VSP_ERR_DTYPE;
+        if (qo->dtype != VSP_F32 && qo->dtype != VSP_BF16) return VSP_ERR_UNSUPPORTED;
+        for (int i = 0; i < 4; ++i)
+            if (q->shape[i] < 0 || q->shape[i] != qo->shape[i]) return VSP_ERR_SHAPE;
+        if (q->shape[0] != new_k->shape[0] || q->shape[2] != T || q->shape[3] != new_k->shape[3]) return VSP_ERR_SHAPE;
+        // the rotated rows must be the cache's rows: no reshaping copy as in plain append
+        if (new_k->shape[0] != cache->B || new_k->shape[1] != cache->Hkv || new_k->shape[3] != cache->D) return VSP_ERR_NUMEL;
+        if (cache->D % 8 != 0) return VSP_ERR_UNSUPPORTED;
+        if (q->stride[3] != 1 || qo->stride[3] != 1) return VSP_ERR_STRIDE;
+        if (((uintptr_t)rope->table & 7) != 0) return VSP_ERR_ALIGN;
+        if (rope->table_len <= 0) return VSP_ERR_ARG;
+        if (!start_pos_dev && (start_pos < 0 || start_pos + T > rope->table_len)) return VSP_ERR_ARG;
+        if (q->shape[0] * q->shape[1] * T * q->shape[3] > 0 && (!q->data || !qo->data)) return VSP_ERR_NULL;
+    }
     // the slot [:, :, start_pos:start_pos+T, :] with the reference's clamping
     int64_t slot_start, slot_len;
     if (start_pos_dev) {
@@ -330,11 +446,14 @@ int vsp_kv_append(vsp_kv_cache* cache, const vsp_tensor* new_k, const vsp_tensor
     const int64_t slot_numel = (int64_t)cache->B * cache->Hkv * slot_len * cache->D;
     const int64_t src_numel = new_k->shape[0] * new_k->shape[1] * new_k->shape[2] * new_k->shape[3];
     if (slot_numel != src_numel) return VSP_ERR_NUMEL;  // copy_from: element count mismatch.
-    if (slot_numel > 0) {
-        if (new_k->shape[3] != cache->D) return VSP_ERR_UNSUPPORTED;  // rows would straddle
-        if (!new_k->data || !new_v->data) return VSP_ERR_NULL;
-        if (new_k->stride[3] != 1 || new_v->stride[3] != 1) return VSP_ERR_STRIDE;
-        AppendArgs a;
+    const int64_t q_items = rope ? rope->q->shape[0] * rope->q->shape[1] * T * (cache->D / 8) : 0;
+    if (slot_numel > 0 || q_items > 0) {
+        if (slot_numel > 0) {
+            if (new_k->shape[3] != cache->D) return VSP_ERR_UNSUPPORTED;  // rows would straddle
+            if (!new_k->data || !new_v->data) return VSP_ERR_NULL;
+            if (new_k->stride[3] != 1 || new_v->stride[3] != 1) return VSP_ERR_STRIDE;
+        }
+        AppendArgs a{};
         a.src_k = new_k->data;
         a.src_v = new_v->data;
         for (int i = 0; i < 3; ++i) {
@@ -356,23 +475,45 @@ int vsp_kv_append(vsp_kv_cache* cache, const vsp_tensor* new_k, const vsp_tensor
         a.slot_len = slot_len;
         a.start_dev = start_pos_dev;
         a.rows = (int64_t)cache->B * cache->Hkv * slot_len;
+        if (rope) {
+            a.table = rope->table;
+            a.table_len = rope->table_len;
+            a.q = rope->q->data;
+            a.q_out = rope->q_out->data;
+            for (int i = 0; i < 3; ++i) {
+                a.sq[i] = rope->q->stride[i];
+                a.so[i] = rope->q_out->stride[i];
+            }
+            a.Hq = rope->q->shape[1];
+            a.T = T;
+            a.q_out_bf16 = rope->q_out->dtype == VSP_BF16;
+        }
         hipStream_t st = (hipStream_t)stream;
         const bool f32src = new_k->dtype == VSP_F32;
+        const bool r = rope != nullptr;
+        auto blocks = [&](int64_t kv_items, int threads) {
+            // the Q part starts at a block boundary so that a block never mixes the two item kinds
+            a.kv_items = ceil_div(kv_items, threads) * threads;
+            return dim3((unsigned)(a.kv_items / threads + ceil_div(q_items, threads)));
+        };
         if (cache->format == VSP_KV_F32) {
-            int64_t n = a.rows * (a.D / 4);
-            dim3 grid((unsigned)ceil_div(n, 256));
-            if (f32src) hipLaunchKernelGGL(append_f32_kernel<float>, grid, dim3(256), 0, st, a);
-            else hipLaunchKernelGGL(append_f32_kernel<uint16_t>, grid, dim3(256), 0, st, a);
+            dim3 grid = blocks(a.rows * (a.D / 4), 256);
+            if (f32src && r) hipLaunchKernelGGL((append_f32_kernel<float, true>), grid, dim3(256), 0, st, a);
+            else if (f32src) hipLaunchKernelGGL((append_f32_kernel<float, false>), grid, dim3(256), 0, st, a);
+            else if (r) hipLaunchKernelGGL((append_f32_kernel<uint16_t, true>), grid, dim3(256), 0, st, a);
+            else hipLaunchKernelGGL((append_f32_kernel<uint16_t, false>), grid, dim3(256), 0, st, a);
         } else if (cache->format == VSP_KV_BF16) {
-            int64_t n = a.rows * (a.D / 8);
-            dim3 grid((unsigned)ceil_div(n, 256));
-            if (f32src) hipLaunchKernelGGL(append_bf16_kernel<float>, grid, dim3(256), 0, st, a);
-            else hipLaunchKernelGGL(append_bf16_kernel<uint16_t>, grid, dim3(256), 0, st, a);
+            dim3 grid = blocks(a.rows * (a.D / 8), 256);
+            if (f32src && r) hipLaunchKernelGGL((append_bf16_kernel<float, true>), grid, dim3(256), 0, st, a);
+            else if (f32src) hipLaunchKernelGGL((append_bf16_kernel<float, false>), grid, dim3(256), 0, st, a);
+            else if (r) hipLaunchKernelGGL((append_bf16_kernel<uint16_t, true>), grid, dim3(256), 0, st, a);
+            else hipLaunchKernelGGL((append_bf16_kernel<uint16_t, false>), grid, dim3(256), 0, st, a);
         } else {
-            int64_t n = a.rows * (a.D / kQBlock);
-            dim3 grid((unsigned)ceil_div(n, 128));
-            if (f32src) hipLaunchKernelGGL(append_q8_kernel<float>, grid, dim3(128), 0, st, a);
-            else hipLaunchKernelGGL(append_q8_kernel<uint16_t>, grid, dim3(128), 0, st, a);
+            dim3 grid = blocks(a.rows * (a.D / kQBlock), 128);
+            if (f32src && r) hipLaunchKernelGGL((append_q8_kernel<float, true>), grid, dim3(128), 0, st, a);
+            else if (f32src) hipLaunchKernelGGL((append_q8_kernel<float, false>), grid, dim3(128), 0, st, a);
+            else if (r) hipLaunchKernelGGL((append_q8_kernel<uint16_t, true>), grid, dim3(128), 0, st, a);
+            else hipLaunchKernelGGL((append_q8_kernel<uint16_t, false>), grid, dim3(128), 0, st, a);
         }
         rc = check_launch();
         if (rc != VSP_OK) return rc;
@@ -383,6 +524,18 @@ int vsp_kv_append(vsp_kv_cache* cache, const vsp_tensor* new_k, const vsp_tensor
         if (nl > cache->len) cache->len = (int32_t)nl;
     }
     return VSP_OK;
+}
+
+int vsp_kv_append(vsp_kv_cache* cache, const vsp_tensor* new_k, const vsp_tensor* new_v, int64_t start_pos,
+                  const int32_t* start_pos_dev, void* stream) {
+    return append_impl(cache, new_k, new_v, start_pos, start_pos_dev, nullptr, stream);
+}
+
+int vsp_rope_kv_append(vsp_kv_cache* cache, const vsp_tensor* q, const vsp_tensor* new_k, const vsp_tensor* new_v,
+                       vsp_tensor* q_out, const float* rope_table, int64_t table_len, int64_t start_pos,
+                       const int32_t* start_pos_dev, void* stream) {
+    RopeParams rp{q, q_out, rope_table, table_len};
+    return append_impl(cache, new_k, new_v, start_pos, start_pos_dev, &rp, stream);
 }
 
 int vsp_kv_read(const vsp_kv_cache* cache, int64_t start, int64_t count, vsp_tensor* k_out, vsp_tensor* v_out,
