@@ -198,6 +198,53 @@ static void run_cached_generation(KVFormat fmt, DType dt, double tol, const char
     for (int64_t t = T0; t < N; ++t) step(t, t + 1);
 }
 
+template <class CacheT>
+static void run_rope_generation(KVFormat fmt, DType qdt, double tol, const char* name) {
+    // GroupedQueryAttention::forward(x, cache, start_pos) from RoPE on (src/nn/gqa_attention.cpp:124-148):
+    // prefill 8 tokens, then token by token; each step equals the causal full forward over rotated q, k.
+    std::printf("test_rope_generation[%s]\n", name);
+    const int64_t B = 2, Hq = 8, Hkv = 2, D = 64, T0 = 8, steps = 4, N = T0 + steps, S_max = 32;
+    nn::GroupedQueryAttentionCore attn(Hq * D, Hq, Hkv);
+    nn::RopeTable rope(S_max, D);
+    auto q = randn(B * Hq * N * D, 31, 0.5f), k = randn(B * Hkv * N * D, 32, 0.5f), v = randn(B * Hkv * N * D, 33, 0.5f);
+    std::vector<float> ang((size_t)(N * D / 2)), qr(q.size()), kr(k.size());
+    orc_rope_angles((int)N, (int)D, 0, 10000.0f, ang.data());
+    orc_rope_apply_f32(q.data(), B, Hq, N, D, ang.data(), qr.data());
+    orc_rope_apply_f32(k.data(), B, Hkv, N, D, ang.data(), kr.data());
+    std::vector<float> want(q.size());
+    int64_t st[4] = {Hkv * N * D, N * D, D, 1};
+    CHECK(orc_gqa_attention_f32(qr.data(), kr.data(), st, v.data(), st, want.data(), B, Hq, N, N, D, Hq / Hkv, 1) == 0);
+    auto slice = [&](const std::vector<float>& x, int64_t H, int64_t t0, int64_t t1) {
+        std::vector<float> out((size_t)(B * H * (t1 - t0) * D));
+        for (int64_t b = 0; b < B; ++b)
+            for (int64_t h = 0; h < H; ++h)
+                for (int64_t t = t0; t < t1; ++t)
+                    std::memcpy(&out[(size_t)(((b * H + h) * (t1 - t0) + (t - t0)) * D)], &x[(size_t)(((b * H + h) * N + t) * D)], D * sizeof(float));
+        return out;
+    };
+    CacheT cache(B, Hkv, S_max, D, Device::HIP, fmt);
+    auto step = [&](int64_t t0, int64_t t1) {
+        Tensor tq = to_dev(slice(q, Hq, t0, t1), {B, Hq, t1 - t0, D}, DType::Float32);
+        Tensor tk = to_dev(slice(k, Hkv, t0, t1), {B, Hkv, t1 - t0, D}, DType::Float32);
+        Tensor tv = to_dev(slice(v, Hkv, t0, t1), {B, Hkv, t1 - t0, D}, DType::Float32);
+        Tensor out = attn.forward_rope(tq, tk, tv, &cache, t0, rope, qdt);
+        auto got = to_host(out), w = slice(want, Hq, t0, t1);
+        double err = max_abs_diff(got, w.data(), w.size());
+        if (!(err < tol)) std::printf("  step [%ld,%ld): max-abs %.3g\n", (long)t0, (long)t1, err);
+        CHECK(err < tol);
+        CHECK((int64_t)cache.current_seq_len() == t1);
+    };
+    step(0, T0);
+    for (int64_t t = T0; t < N; ++t) step(t, t + 1);
+    // positions outside the table are refused, nothing is written
+    nn::RopeTable small(4, D);
+    Tensor tq = to_dev(slice(q, Hq, 0, 8), {B, Hq, 8, D}, DType::Float32);
+    Tensor tk = to_dev(slice(k, Hkv, 0, 8), {B, Hkv, 8, D}, DType::Float32);
+    CacheT c2(B, Hkv, S_max, D, Device::HIP, fmt);
+    CHECK(thrown<std::runtime_error>([&] { attn.forward_rope(tq, tk, tk, &c2, 0, small, qdt); }) != "<nothing thrown>");
+    CHECK(c2.current_seq_len() == 0);
+}
+
 static void test_sdpa_routing() {
     std::printf("test_sdpa_routing\n");
     const int64_t B = 1, H = 2, D = 64;
@@ -236,6 +283,8 @@ int main(int argc, char** argv) {
         run_cached_generation<nn::KVCache>(KVFormat::Float32, DType::Float32, 1e-4, "KVCache fp32");
         run_cached_generation<nn::GQAKVCache>(KVFormat::BFloat16, DType::BFloat16, 2e-2, "GQAKVCache bf16");
         run_cached_generation<nn::GQAKVCache>(KVFormat::Q8_0, DType::BFloat16, 2e-2, "GQAKVCache q8_0");
+        run_rope_generation<nn::KVCache>(KVFormat::Float32, DType::Float32, 1e-4, "KVCache fp32");
+        run_rope_generation<nn::GQAKVCache>(KVFormat::BFloat16, DType::BFloat16, 2e-2, "GQAKVCache bf16");
         test_sdpa_routing();
     }
     std::printf(g_fail ? "FAILED: %d check(s)\n" : "all adapter tests passed\n", g_fail);

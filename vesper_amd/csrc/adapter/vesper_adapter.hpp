@@ -195,6 +195,30 @@ inline Tensor empty(const std::vector<int64_t>& shape, DType dtype, Device devic
 // ------------------------------------------------------------------------------------------------
 namespace nn {
 
+// {cos, sin} of the angles of functional::compute_rope_frequencies (include/vesper/nn/functional.h:148,
+// src/nn/functional.cpp:424-443) for absolute positions [0, max_seq_len): computed once on the host by the
+// library and kept on the device, instead of the reference's per-call host loop + upload.
+class RopeTable {
+public:
+    RopeTable(int64_t max_seq_len, int64_t head_dim, float theta = 10000.0f)
+        : len_(max_seq_len), head_dim_(head_dim), theta_(theta) {
+        if (head_dim % 2 != 0) throw std::runtime_error("RoPE error: head_dim must be even for RoPE");  // src/nn/rope.cpp:98
+        std::vector<float> host((size_t)(max_seq_len * (head_dim / 2) * 2));
+        vsp_rope_fill_table(host.data(), 0, (int32_t)max_seq_len, (int32_t)head_dim, theta);
+        store_ = std::make_shared<Storage>(host.size() * sizeof(float));
+        hip_check(hipMemcpy(store_->data(), host.data(), host.size() * sizeof(float), hipMemcpyHostToDevice), "RopeTable upload");
+    }
+    const float* data() const { return (const float*)store_->data(); }
+    int64_t length() const { return len_; }
+    int64_t head_dim() const { return head_dim_; }
+    float theta() const { return theta_; }
+
+private:
+    std::shared_ptr<Storage> store_;
+    int64_t len_, head_dim_;
+    float theta_;
+};
+
 // One template for both reference caches: LenT = int for KVCache, int64_t for GQAKVCache.
 template <typename LenT>
 class KVCacheT {
@@ -228,6 +252,18 @@ public:
     std::pair<Tensor, Tensor> update(const Tensor& new_k, const Tensor& new_v, LenT start_pos) {
         vsp_tensor dk = new_k.desc(), dv = new_v.desc();
         throw_status(vsp_kv_append(&st_->c, &dk, &dv, (int64_t)start_pos, nullptr, current_stream()));
+        return {view(false), view(true)};
+    }
+    // Steps 3-4 of the cached forward (src/nn/gqa_attention.cpp:124-130) in one launch: q and new_k rotated at
+    // positions start_pos.., new_k/new_v written like update().  q is replaced by its rotated value
+    // (`q_dtype`: what the attention kernels should receive).
+    std::pair<Tensor, Tensor> rope_update(Tensor& q, const Tensor& new_k, const Tensor& new_v, LenT start_pos,
+                                          const RopeTable& rope, DType q_dtype) {
+        Tensor q_out = empty(q.shape(), q_dtype);
+        vsp_tensor dq = q.desc(), dk = new_k.desc(), dv = new_v.desc(), dout = q_out.desc();
+        throw_status(vsp_rope_kv_append(&st_->c, &dq, &dk, &dv, &dout, rope.data(), rope.length(), (int64_t)start_pos,
+                                        nullptr, current_stream()));
+        q = q_out;
         return {view(false), view(true)};
     }
     void reset() { throw_status(vsp_kv_cache_reset(&st_->c, current_stream())); }
@@ -382,6 +418,17 @@ public:
         v = ops::repeat_kv(v, num_rep_);
         const bool use_causal = (T > 1);
         return functional::scaled_dot_product_attention(q, k, v, use_causal, 0.0);
+    }
+
+    // forward(x, cache, start_pos) from step 3 on, src/nn/gqa_attention.cpp:124-148: q/k/v are the projections'
+    // outputs viewed as [B,H,T,D] (any strides), not yet rotated.
+    template <typename CacheT>
+    Tensor forward_rope(Tensor q, const Tensor& k, const Tensor& v, CacheT* cache, int64_t start_pos, const RopeTable& rope,
+                        DType q_dtype) const {
+        if (!cache) throw std::runtime_error("forward_rope: a cache is required");
+        const int64_t T = q.shape()[2];
+        auto kv = cache->rope_update(q, k, v, (decltype(cache->current_seq_len()))start_pos, rope, q_dtype);
+        return functional::scaled_dot_product_attention(q, ops::repeat_kv(kv.first, num_rep_), ops::repeat_kv(kv.second, num_rep_), T > 1, 0.0);
     }
 
 private:
