@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on ONE MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|p4k|c3|c4|c5] [--no-cpu] [--no-extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|p4k|c3|c4|c5|r2] [--no-cpu] [--no-extra]
 
 A "step" is one pass of the hot path over one batch of synthetic input that is already resident in
 HBM: one prefill launch (c2, p4k, c3) or one decode call = split-K kernel + combine kernel (c4, c5).
@@ -36,7 +36,15 @@ WORKLOADS = {
                name="BASELINE config 4: batched decode bf16 KV cache, B32, 32 q / 8 kv heads, D128, L~U[1024,32768]"),
     "c5": dict(kind="decode", fmt="q8_0", B=16, Hq=64, Hkv=8, D=128, S=65536, lens=None,
                name="BASELINE config 5: decode over Q8_0 KV cache, B16, 64 q / 8 kv heads, D128, L=65536"),
+    "r2": dict(kind="rope", fmt="bf16", B=4, Hq=32, Hkv=8, D=128, N=2048,
+               name="RoPE + KV append for config 2: q/k/v bf16 views of one fused projection buffer [B,T,(Hq+2Hkv)D], "
+                    "rotated q out bf16, bf16 cache, B4, 32 q / 8 kv heads, D128, T2048"),
 }
+
+
+def rope_bytes(w):
+    e = 2  # bf16 in, bf16 out
+    return float(w["B"] * w["N"] * w["D"] * e * (2 * w["Hq"] + 4 * w["Hkv"]) + w["N"] * w["D"] * 4)
 
 
 def prefill_flops(w):
@@ -64,6 +72,18 @@ class Runner:
             self.work = prefill_flops(w)
             self.unit, self.peak, self.bound = "TFLOP/s", MFMA_BF16_PEAK_TFLOPS, "mfma"
             self.kernel = "prefill_bf16_kernel<128>"
+        elif w["kind"] == "rope":
+            B, Hq, Hkv, D, N = w["B"], w["Hq"], w["Hkv"], w["D"], w["N"]
+            fused = (torch.randn(B, N, (Hq + 2 * Hkv) * D, device=dev, generator=g) * 0.5).to(torch.bfloat16)
+            self.q = fused[:, :, :Hq * D].view(B, N, Hq, D).transpose(1, 2)
+            self.k = fused[:, :, Hq * D:(Hq + Hkv) * D].view(B, N, Hkv, D).transpose(1, 2)
+            self.v = fused[:, :, (Hq + Hkv) * D:].view(B, N, Hkv, D).transpose(1, 2)
+            self.cache = va.KVCache(B, Hkv, N, D, fmt=w["fmt"])
+            self.rope = va.RopeTable(N, D)
+            self.out = torch.empty(B, Hq, N, D, device=dev, dtype=torch.bfloat16)
+            self.work = rope_bytes(w)
+            self.unit, self.peak, self.bound = "GB/s", HBM_PEAK_GBS, "hbm"
+            self.kernel = "append_bf16_kernel<unsigned short, true>"
         else:
             import numpy as np
             B, Hq, Hkv, D, S = w["B"], w["Hq"], w["Hkv"], w["D"], w["S"]
@@ -110,6 +130,8 @@ class Runner:
     def step(self):
         if self.w["kind"] == "prefill":
             return self.va.flash_attention(self.q, self.k, self.v, self.scale, True)
+        if self.w["kind"] == "rope":
+            return self.cache.rope_update(self.q, self.k, self.v, 0, self.rope, out=self.out)
         return self.va.decode_attention(self.q, self.cache, seq_lens=self.seq_lens, max_len=self.max_len,
                                         scale=self.scale, out=self.out)
 
@@ -260,7 +282,7 @@ def main():
 
     if not args.no_extra:
         others = {}
-        for key in ("c2", "p4k", "c3", "c4", "c5"):
+        for key in ("c2", "p4k", "c3", "c4", "c5", "r2"):
             if key == args.workload:
                 continue
             r = Runner(key, torch, va)

@@ -187,6 +187,20 @@ int vsp_kv_view_f32(const vsp_kv_cache* cache, vsp_tensor* k_view, vsp_tensor* v
 int vsp_attn_prefill(const vsp_tensor* q, const vsp_tensor* k, const vsp_tensor* v, vsp_tensor* out, vsp_tensor* lse,
                      float scale, int is_causal, float dropout_p, int training, void* stream);
 
+/* Chunked / offset prefill straight over the cache planes (no counterpart in the reference, whose causal mask is
+ * [T,T] and cannot be added to [T,L] scores, src/nn/functional.cpp:406-410; the semantics are the rows
+ * [L-T, L) of the reference's full causal forward over L tokens, src/ops/flash_attention.cpp:218-364):
+ * q [B,Hq,T,D] holds the LAST T tokens of each context, whose K/V are already in the cache
+ * (vsp_kv_append / vsp_rope_kv_append first).  Context length: cache->len, or seq_lens[b] (device int32[B],
+ * T <= seq_lens[b] <= S_max; values are clamped to that range) for ragged batches.  Query t attends keys
+ * j <= L_b - T + t when is_causal, all L_b keys otherwise.
+ *   VSP_KV_F32 : q/out fp32, fp32 arithmetic.   VSP_KV_BF16 : q/out bf16; K rows and token-blocked V are
+ *   consumed in place (V^T operands are plain 16-byte reads of the blocked plane).
+ *   VSP_KV_Q8_0: VSP_ERR_UNSUPPORTED (materialise the context with vsp_kv_read and call vsp_attn_prefill).
+ * Tokens past L_b in the planes are never used, whatever they hold.  lse as in vsp_attn_prefill. */
+int vsp_attn_prefill_cached(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, vsp_tensor* out,
+                            vsp_tensor* lse, float scale, int is_causal, void* stream);
+
 /* ---- decode -------------------------------------------------------------------
  * Replaces, for T == 1, the op chain scaled_dot_product_attention runs below its flash threshold
  * (src/nn/functional.cpp:397-421: gemm_batch_hip_dispatch x2, div_scalar, softmax_hip_dispatch)

@@ -1,0 +1,138 @@
+"""Chunked prefill over the cache planes (vsp_attn_prefill_cached) on the GPU.  The reference has no chunked
+causal attention; the expected values are rows [L-T, L) of its full causal forward over L tokens (the oracle's
+flash_attention, bit-exact to the compiled reference), on the values the cache holds."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import _gpu as G
+import _inputs as I
+import _oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def va():
+    import vesper_amd
+    return vesper_amd
+
+
+def _expected(q_full, k, v, L, T, causal=True):
+    """Rows [L-T, L) of attention over the first L tokens, fp32 oracle."""
+    n = q_full.shape[1] // k.shape[1]
+    kk, vv = O.repeat_kv(k[:, :, :L], n), O.repeat_kv(v[:, :, :L], n)
+    scale = float(np.float32(1.0 / math.sqrt(q_full.shape[-1])))
+    if causal:
+        return O.flash_attention(q_full[:, :, :L], kk, vv, scale, True)[:, :, L - T:]
+    return O.sdpa(q_full[:, :, L - T:L], kk, vv, False)
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,L,T,D,S_max", [(1, 4, 2, 96, 32, 128, 128), (2, 8, 2, 201, 73, 128, 260),
+                                                 (1, 4, 4, 130, 130, 64, 130), (1, 2, 1, 333, 1, 64, 400),
+                                                 (1, 8, 2, 1100, 300, 128, 1100)])
+def test_bf16_planes_against_oracle_and_dense_kernel(va, B, Hq, Hkv, L, T, D, S_max):
+    q, k, v = [O.bf16_round(x * np.float32(0.5)) for x in I.qkv(3000 + L, B, Hq, Hkv, L, L, D)]
+    c = va.KVCache(B, Hkv, S_max, D, fmt="bf16")
+    # the context arrives in two appends, the second being the chunk
+    if L > T:
+        c.update(G.to_bf16_dev(k[:, :, :L - T]), G.to_bf16_dev(v[:, :, :L - T]), 0, return_views=False)
+    c.update(G.to_bf16_dev(k[:, :, L - T:]), G.to_bf16_dev(v[:, :, L - T:]), L - T, return_views=False)
+    qd = G.to_bf16_dev(q[:, :, L - T:])
+    out, lse = c.prefill(qd, return_lse=True)
+    want = _expected(q, k, v, L, T)
+    G.assert_bf16_close(G.bf16_to_np(out), want, "vs oracle")
+    # the dense kernel (row-major V through the transposing LDS read) on the read-back context: an independent path
+    kd, vd = c.read(0, L, torch.bfloat16)
+    dense, lse2 = va.flash_attention(qd, kd, vd, 1.0 / math.sqrt(D), True, return_lse=True)
+    err = np.abs(G.bf16_to_np(out) - G.bf16_to_np(dense))
+    assert err.max() <= 2e-2
+    assert np.allclose(lse.cpu().numpy(), lse2.cpu().numpy(), atol=2e-3)
+    # non-causal: every query sees all L keys
+    out_nc = c.prefill(qd, is_causal=False)
+    G.assert_bf16_close(G.bf16_to_np(out_nc), _expected(q, k, v, L, T, causal=False), "non-causal")
+
+
+def test_stale_tokens_past_the_context_are_never_used(va):
+    B, Hq, Hkv, L, T, D, S_max = 1, 4, 2, 77, 40, 128, 192
+    q, k, v = [O.bf16_round(x) for x in I.qkv(3100, B, Hq, Hkv, L, L, D)]
+    c = va.KVCache(B, Hkv, S_max, D, fmt="bf16")
+    # poison every plane byte (bf16 NaN pattern 0x7fc0), then write only the context
+    for p in (0, 1):
+        c.raw_plane(p).view(torch.int16).fill_(0x7fc0)
+    c.update(G.to_bf16_dev(k), G.to_bf16_dev(v), 0, return_views=False)
+    out = c.prefill(G.to_bf16_dev(q[:, :, L - T:]))
+    got = G.bf16_to_np(out)
+    assert np.isfinite(got).all()
+    G.assert_bf16_close(got, _expected(q, k, v, L, T), "poisoned tail")
+
+
+def test_per_sequence_lengths(va):
+    B, Hq, Hkv, T, D, S_max = 3, 4, 2, 24, 128, 160
+    lens = np.array([24, 131, 90], np.int32)
+    qs, ks, vs = [], [], []
+    c = va.KVCache(B, Hkv, S_max, D, fmt="bf16")
+    kfull = np.zeros((B, Hkv, S_max, D), np.float32)
+    vfull = np.zeros_like(kfull)
+    qchunk = np.zeros((B, Hq, T, D), np.float32)
+    for b in range(B):
+        q, k, v = [O.bf16_round(x * np.float32(0.7)) for x in I.qkv(3200 + b, 1, Hq, Hkv, int(lens[b]), int(lens[b]), D)]
+        qs.append(q), ks.append(k), vs.append(v)
+        kfull[b, :, :lens[b]], vfull[b, :, :lens[b]] = k[0], v[0]
+        qchunk[b] = q[0, :, lens[b] - T:]
+    c.update(G.to_bf16_dev(kfull), G.to_bf16_dev(vfull), 0, return_views=False)
+    sl = torch.from_numpy(lens).to(G.dev())
+    out = G.bf16_to_np(c.prefill(G.to_bf16_dev(qchunk), seq_lens=sl))
+    for b in range(B):
+        G.assert_bf16_close(out[b:b + 1], _expected(qs[b], ks[b], vs[b], int(lens[b]), T), f"row {b}")
+
+
+def test_f32_cache_planes(va):
+    B, Hq, Hkv, L, T, D, S_max = 2, 4, 2, 150, 50, 64, 200
+    q, k, v = I.qkv(3300, B, Hq, Hkv, L, L, D)
+    c = va.KVCache(B, Hkv, S_max, D, fmt="f32")
+    c.update(G.f32_dev(k), G.f32_dev(v), 0, return_views=False)
+    out = c.prefill(G.f32_dev(q[:, :, L - T:]))
+    G.assert_f32_close(out.cpu().numpy(), _expected(q, k, v, L, T), "f32 planes")
+    lens = torch.tensor([150, 99], dtype=torch.int32, device=G.dev())
+    out2 = c.prefill(G.f32_dev(np.stack([q[0, :, 100:150], q[1, :, 49:99]])), seq_lens=lens).cpu().numpy()
+    G.assert_f32_close(out2[0:1], _expected(q[0:1], k[0:1], v[0:1], 150, 50), "row 0")
+    G.assert_f32_close(out2[1:2], _expected(q[1:2], k[1:2], v[1:2], 99, 50), "row 1")
+
+
+def test_chunked_equals_one_shot_at_config2_size(va):
+    # BASELINE config 2 shape, prefilled in two chunks of 1024 through the cache: same rows as the dense launch
+    B, Hq, Hkv, N, D = 4, 32, 8, 2048, 128
+    g = torch.Generator(device="cuda").manual_seed(5)
+    mk = lambda h: (torch.randn(B, h, N, D, device=G.dev(), generator=g) * 0.5).to(torch.bfloat16)
+    q, k, v = mk(Hq), mk(Hkv), mk(Hkv)
+    dense = va.flash_attention(q, k, v, 1.0 / math.sqrt(D), True)
+    c = va.KVCache(B, Hkv, N, D, fmt="bf16")
+    outs = []
+    for t0 in (0, 1024):
+        c.update(k[:, :, t0:t0 + 1024], v[:, :, t0:t0 + 1024], t0, return_views=False)
+        outs.append(c.prefill(q[:, :, t0:t0 + 1024]))
+    got = torch.cat(outs, dim=2).float()
+    err = (got - dense.float()).abs()
+    assert err.max().item() <= 2e-2 and err.mean().item() <= 2e-3
+    again = c.prefill(q[:, :, 1024:])
+    assert torch.equal(again, outs[1])  # run-to-run deterministic
+
+
+def test_argument_errors(va):
+    c8 = va.KVCache(1, 2, 64, 64, fmt="q8_0")
+    q = torch.zeros(1, 4, 8, 64, device=G.dev(), dtype=torch.bfloat16)
+    with pytest.raises(va.VspError):
+        c8.prefill(q)
+    c = va.KVCache(1, 2, 64, 64, fmt="bf16")
+    with pytest.raises(va.VspError):      # chunk longer than the context (len == 0)
+        c.prefill(q)
+    c.update(torch.zeros(1, 2, 16, 64, device=G.dev(), dtype=torch.bfloat16),
+             torch.zeros(1, 2, 16, 64, device=G.dev(), dtype=torch.bfloat16), 0, return_views=False)
+    with pytest.raises(va.VspError):      # fp32 q over a bf16 cache
+        c.prefill(q.float())
+    with pytest.raises(va.VspError):      # head count not a multiple of the cache's
+        c.prefill(torch.zeros(1, 3, 8, 64, device=G.dev(), dtype=torch.bfloat16))
+    assert c.prefill(q).shape == q.shape

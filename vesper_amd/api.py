@@ -112,16 +112,30 @@ class KVCache:
             return None
         return self.views()
 
-    def rope_update(self, q, new_k, new_v, start_pos, rope, out_dtype=None, start_pos_dev=None, return_views=False):
+    def rope_update(self, q, new_k, new_v, start_pos, rope, out_dtype=None, start_pos_dev=None, return_views=False,
+                    out=None):
         """Steps 3-4 of the attention modules' cached forward in one launch (src/nn/gqa_attention.cpp:124-130):
         q and k rotated by `rope` (a RopeTable) at positions start_pos.., k and v written to the cache.
         Returns the rotated q (and the cache views when asked)."""
-        q_out = torch.empty(q.shape, dtype=out_dtype or q.dtype, device=q.device)
+        q_out = out if out is not None else torch.empty(q.shape, dtype=out_dtype or q.dtype, device=q.device)
         dq, dk, dv, do = _desc(q), _desc(new_k), _desc(new_v), _desc(q_out)
         sp = C.c_void_p(start_pos_dev.data_ptr()) if start_pos_dev is not None else None
         check(lib.vsp_rope_kv_append(C.byref(self._c), C.byref(dq), C.byref(dk), C.byref(dv), C.byref(do),
                                      C.c_void_p(rope.table.data_ptr()), rope.length, int(start_pos), sp, _stream(q)))
         return (q_out, self.views()) if return_views else q_out
+
+    def prefill(self, q, seq_lens=None, is_causal=True, scale=None, return_lse=False):
+        """Attention of the last T tokens (q [B,Hq,T,D]) over the cached context, read in place from the planes:
+        chunked prefill.  seq_lens: device int32[B] per-row context lengths (default: the cache's one length)."""
+        out = torch.empty_like(q)
+        lse = torch.empty(q.shape[:3], dtype=torch.float32, device=q.device) if return_lse else None
+        dq, do = _desc(q), _desc(out)
+        dl = _desc(lse) if lse is not None else None
+        sl = C.c_void_p(seq_lens.data_ptr()) if seq_lens is not None else None
+        sc = float(scale) if scale is not None else 1.0 / math.sqrt(q.shape[-1])
+        check(lib.vsp_attn_prefill_cached(C.byref(dq), C.byref(self._c), sl, C.byref(do),
+                                          C.byref(dl) if dl is not None else None, sc, int(bool(is_causal)), _stream(q)))
+        return (out, lse) if return_lse else out
 
     # -- reads
     def views(self, dtype=None):

@@ -27,6 +27,7 @@
 
 #include <utility>
 
+#include "kv_layout.hpp"
 #include "vsp_common.hpp"
 
 namespace vsp {
@@ -44,6 +45,8 @@ struct PrefillArgs {
     int32_t causal;
     int32_t n_qtiles;
     int32_t negate_q;  // scale < 0: flip the sign of Q (exact) and use |scale|
+    int32_t s_pad;     // cache-plane mode: padded token capacity of the planes
+    const int32_t* seq_lens;  // cache-plane mode: per-batch context lengths (device) or nullptr
     float scale_log2;  // |scale| * log2(e) for bf16; scale * log2(e) for fp32
 };
 
@@ -93,6 +96,12 @@ template <int N>
 __device__ inline void lds_wait(u32x4_t& a0) {
     asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(a0) : "n"(N));
 }
+__device__ inline void lds_wait0(u32x4_t& a0, u32x4_t& a1, u32x4_t& a2, u32x4_t& a3) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3));
+}
+__device__ inline void lds_wait0(u32x4_t& a0, u32x4_t& a1) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a0), "+v"(a1));
+}
 template <int... I, class F>
 __device__ inline void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
     (f(std::integral_constant<int, I>{}), ...);
@@ -107,7 +116,12 @@ __device__ inline uint32_t lds_addr(const void* p) {
 
 constexpr int kUnit = 32;  // keys per tile (one LDS ring slot)
 
-template <int D>
+// VBLK: K and V are the planes of a bf16 KV cache (K row-major, V token-blocked by 8) instead of dense
+// tensors, and the context length may come per batch row from a device array.  With 8 tokens of one d
+// contiguous, a V^T operand is a plain 16-byte LDS read (no transposing read, no swizzle); to make the
+// softmax registers line up with those 8 consecutive tokens, lane i of the K operand holds key
+// (i with bits 2 and 3 swapped) of the tile.
+template <int D, bool VBLK>
 __global__ void __launch_bounds__(256, 3) prefill_bf16_kernel(PrefillArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the body uses device-only builtins
     constexpr int KS = D / 16;
@@ -143,12 +157,14 @@ __global__ void __launch_bounds__(256, 3) prefill_bf16_kernel(PrefillArgs a) {
         bh = grp * a.n_rep + slot % a.n_rep;  // == b * Hq + hq, because groups are numbered b * Hkv + kvh
     }
     const int b = bh / a.Hq, hq = bh % a.Hq, kvh = hq / a.n_rep;
+    int L = a.L;
+    if (VBLK && a.seq_lens) L = min(max(a.seq_lens[b], a.T), a.L);  // a.L = capacity bound in this mode
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int ql = lane & 31, h = lane >> 5;
     const int q0 = qt * kBM + wave * 32;
-    const int off = a.L - a.T;
+    const int off = L - a.T;
     const int qrow = min(q0 + ql, a.T - 1);
 
     const uint16_t* Qp = (const uint16_t*)a.q + (int64_t)b * a.sq[0] + (int64_t)hq * a.sq[1];
@@ -169,10 +185,10 @@ __global__ void __launch_bounds__(256, 3) prefill_bf16_kernel(PrefillArgs a) {
     }
 
     const int wg_qmax = min(qt * kBM + kBM - 1, a.T - 1);
-    const int kv_end_wg = a.causal ? min(a.L, wg_qmax + off + 1) : a.L;
+    const int kv_end_wg = a.causal ? min(L, wg_qmax + off + 1) : L;
     const int n_tiles = (kv_end_wg + kUnit - 1) / kUnit;
     const int wave_qmax = min(q0 + 31, a.T - 1);
-    const int kv_end_wave = (q0 < a.T) ? (a.causal ? min(a.L, wave_qmax + off + 1) : a.L) : 0;
+    const int kv_end_wave = (q0 < a.T) ? (a.causal ? min(L, wave_qmax + off + 1) : L) : 0;
 
     f32x16_t acc[DB];
 #pragma unroll
@@ -193,14 +209,18 @@ __global__ void __launch_bounds__(256, 3) prefill_bf16_kernel(PrefillArgs a) {
     for (int i = 0; i < NLD; ++i) {
         const int r = NR * (wave + 4 * i) + ld_row;
         voffK[i] = (uint32_t)r * (uint32_t)a.sk[2] * 2u + 16u * (uint32_t)(ld_pos ^ ((r / RP) % CPR));
-        voffV[i] = (uint32_t)r * (uint32_t)a.sv[2] * 2u + 16u * (uint32_t)(ld_pos ^ (((r / RP) % (CPR / 4)) << 2));
+        if constexpr (VBLK) voffV[i] = (uint32_t)(wave + 4 * i) * 1024u + 16u * (uint32_t)lane;  // the tile is contiguous
+        else voffV[i] = (uint32_t)r * (uint32_t)a.sv[2] * 2u + 16u * (uint32_t)(ld_pos ^ (((r / RP) % (CPR / 4)) << 2));
     }
     const int64_t rowK = a.sk[2] * 2, rowV = a.sv[2] * 2;  // bytes per key row
     auto load_tile = [&](int t, int slot) {
         const int key0 = t * kUnit;
-        const int rows = a.L - key0;  // > 0
+        const int rows = L - key0;  // > 0
         __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)Kp + (int64_t)key0 * rowK), 0, (int)((int64_t)rows * rowK), 0x00020000);
-        __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)Vp + (int64_t)key0 * rowV), 0, (int)((int64_t)rows * rowV), 0x00020000);
+        // VBLK: 32 tokens = 4 token blocks = kUnit * D contiguous elements; bound = the rest of this head's plane
+        const int64_t v_base = VBLK ? (int64_t)key0 * D * 2 : (int64_t)key0 * rowV;
+        const int64_t v_bytes = VBLK ? ((int64_t)a.s_pad - key0) * D * 2 : (int64_t)rows * rowV;
+        __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)Vp + v_base), 0, (int)v_bytes, 0x00020000);
         uint16_t* dstK = smem + slot * SLOT;
         uint16_t* dstV = smem + (2 + slot) * SLOT;
 #pragma unroll
@@ -213,16 +233,18 @@ __global__ void __launch_bounds__(256, 3) prefill_bf16_kernel(PrefillArgs a) {
     };
 
     // Loop-constant LDS read addresses (slot 0; the slot is an immediate offset on the instruction).
-    const int kswz = (ql / RP) % CPR;
+    const int krow = VBLK ? ((ql & ~12) | ((ql & 4) << 1) | ((ql & 8) >> 1)) : ql;  // tile row this lane's S^T row holds
+    const int kswz = (krow / RP) % CPR;
     uint32_t kaddr[KS];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) kaddr[ks] = lds0 + 2u * (uint32_t)(ql * D + 8 * ((2 * ks + h) ^ kswz));
+    for (int ks = 0; ks < KS; ++ks) kaddr[ks] = lds0 + 2u * (uint32_t)(krow * D + 8 * ((2 * ks + h) ^ kswz));
     const int i16 = lane & 15;
     const int vswz = ((i16 >> 2) / RP) % (CPR / 4);
     const int v_lane_off = (4 * h + (i16 >> 2)) * D + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
     uint32_t va[DB];
 #pragma unroll
-    for (int db = 0; db < DB; ++db) va[db] = lds0 + 2u * (uint32_t)v_lane_off + 64u * (uint32_t)(db ^ vswz);
+    for (int db = 0; db < DB; ++db)
+        va[db] = VBLK ? lds0 + 16u * (uint32_t)(h * D + ql) : lds0 + 2u * (uint32_t)v_lane_off + 64u * (uint32_t)(db ^ vswz);
 
     constexpr int PF = 4;  // K fragments in flight
 
@@ -249,13 +271,13 @@ __global__ void __launch_bounds__(256, 3) prefill_bf16_kernel(PrefillArgs a) {
             s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kf[ks]), qf[ks], s[0], 0, 0, 0);
             if constexpr (ks + PF < KS) kf[ks + PF] = lds_read_b128_asm<KOFF>(kaddr[ks + PF]);
         });
-        const bool need_mask = (a.causal && k0 + kUnit - 1 > q0 + off) || (k0 + kUnit > a.L);
+        const bool need_mask = (a.causal && k0 + kUnit - 1 > q0 + off) || (k0 + kUnit > L);
         if (need_mask) {
             const int q_abs = q0 + ql + off;
-            const int lim = a.causal ? min(q_abs, a.L - 1) : a.L - 1;
+            const int lim = a.causal ? min(q_abs, L - 1) : L - 1;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const int key = k0 + 8 * (v >> 2) + 4 * h + (v & 3);
+                const int key = VBLK ? k0 + 16 * (v >> 3) + 8 * h + (v & 7) : k0 + 8 * (v >> 2) + 4 * h + (v & 3);
                 if (key > lim) s[0][v] = -INFINITY;
             }
         }
@@ -286,6 +308,41 @@ __global__ void __launch_bounds__(256, 3) prefill_bf16_kernel(PrefillArgs a) {
         }
         l += lsum;
         // PV
+        if constexpr (VBLK) {
+            u32x4_t vcur[DB], vnext[DB];
+            static_for<DB>([&](auto dbc) { vcur[dbc.value] = lds_read_b128_asm<VOFF + 512 * dbc.value>(va[dbc.value]); });
+            const bool tail = k0 + kUnit > L;  // the planes hold stale tokens past L: P is 0 there, V must not be NaN
+            static_for<NJ>([&](auto jc) {
+                constexpr int j = jc.value;
+                if constexpr (DB == 4) lds_wait0(vcur[0], vcur[1], vcur[2], vcur[3]);
+                else lds_wait0(vcur[0], vcur[1]);
+                if constexpr (j + 1 < NJ)
+                    static_for<DB>([&](auto dbc) {
+                        vnext[dbc.value] = lds_read_b128_asm<VOFF + (2 * (j + 1) * D + 32 * dbc.value) * 16>(va[dbc.value]);
+                    });
+                if (tail) {
+                    const int nvalid = L - (k0 + 16 * j + 8 * h);  // slots e >= nvalid are past the context
+#pragma unroll
+                    for (int db = 0; db < DB; ++db)
+#pragma unroll
+                        for (int w = 0; w < 4; ++w) {
+                            uint32_t x = vcur[db][w];
+                            if (2 * w + 1 >= nvalid) x &= 0x0000ffffu;
+                            if (2 * w >= nvalid) x = 0;
+                            vcur[db][w] = x;
+                        }
+                }
+                const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, uint4{pw[j][0], pw[j][1], pw[j][2], pw[j][3]});
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+                    acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, vcur[db]), pf, acc[db], 0, 0, 0);
+                if constexpr (j + 1 < NJ) {
+#pragma unroll
+                    for (int db = 0; db < DB; ++db) vcur[db] = vnext[db];
+                }
+            });
+            return;
+        }
         uint2 tcur[DB][2], tnext[DB][2];
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
@@ -362,10 +419,11 @@ __global__ void __launch_bounds__(256) prefill_f32_kernel(PrefillArgs a) {
     const int qt = a.n_qtiles - 1 - bid / (a.B * a.Hq);
     const int bh = bid % (a.B * a.Hq);
     const int b = bh / a.Hq, hq = bh % a.Hq, kvh = hq / a.n_rep;
+    const int L = a.seq_lens ? min(max(a.seq_lens[b], a.T), a.L) : a.L;  // per-row context length (cache mode)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int ql = lane & 31, h = lane >> 5;
     const int q0 = qt * kBM + wave * 32;
-    const int off = a.L - a.T;
+    const int off = L - a.T;
     const int qrow = min(q0 + ql, a.T - 1);
 
     const float* Qp = (const float*)a.q + (int64_t)b * a.sq[0] + (int64_t)hq * a.sq[1] + (int64_t)qrow * a.sq[2];
@@ -378,10 +436,10 @@ __global__ void __launch_bounds__(256) prefill_f32_kernel(PrefillArgs a) {
     for (int ks = 0; ks < D / 2; ++ks) qf[ks] = Qp[2 * ks + h];
 
     const int wg_qmax = min(qt * kBM + kBM - 1, a.T - 1);
-    const int kv_end_wg = a.causal ? min(a.L, wg_qmax + off + 1) : a.L;
+    const int kv_end_wg = a.causal ? min(L, wg_qmax + off + 1) : L;
     const int n_tiles = (kv_end_wg + BN - 1) / BN;
     const int wave_qmax = min(q0 + 31, a.T - 1);
-    const int kv_end_wave = a.causal ? min(a.L, wave_qmax + off + 1) : a.L;
+    const int kv_end_wave = a.causal ? min(L, wave_qmax + off + 1) : L;
 
     f32x16_t acc[DB];
 #pragma unroll
@@ -394,8 +452,8 @@ __global__ void __launch_bounds__(256) prefill_f32_kernel(PrefillArgs a) {
         __syncthreads();
         for (int id = tid; id < BN * D; id += 256) {
             const int row = id / D, col = id % D, key = kt * BN + row;
-            sK[row * PITCH + col] = key < a.L ? Kp[(int64_t)key * a.sk[2] + col] : 0.f;
-            sV[row * PITCH + col] = key < a.L ? Vp[(int64_t)key * a.sv[2] + col] : 0.f;
+            sK[row * PITCH + col] = key < L ? Kp[(int64_t)key * a.sk[2] + col] : 0.f;
+            sV[row * PITCH + col] = key < L ? Vp[(int64_t)key * a.sv[2] + col] : 0.f;
         }
         __syncthreads();
         const int k0 = kt * BN;
@@ -407,7 +465,7 @@ __global__ void __launch_bounds__(256) prefill_f32_kernel(PrefillArgs a) {
 #pragma unroll
         for (int ks = 0; ks < D / 2; ++ks)
             s = __builtin_amdgcn_mfma_f32_32x32x2f32(sK[ql * PITCH + 2 * ks + h], qf[ks], s, 0, 0, 0);
-        const int lim = a.causal ? min(q0 + ql + off, a.L - 1) : a.L - 1;
+        const int lim = a.causal ? min(q0 + ql + off, L - 1) : L - 1;
         float mx = -INFINITY;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
@@ -465,10 +523,92 @@ int check_tensor4(const vsp_tensor* t, int esz) {
     return VSP_OK;
 }
 
+int launch_prefill(const PrefillArgs& a, int dtype, int64_t D, bool cache_planes, void* stream) {
+    const int64_t blocks = (int64_t)a.n_qtiles * a.B * a.Hq;
+    if (blocks > INT32_MAX) return VSP_ERR_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    dim3 grid((unsigned)blocks), block(256);
+    if (dtype == VSP_BF16) {
+        if (cache_planes) {
+            if (D == 128) hipLaunchKernelGGL((prefill_bf16_kernel<128, true>), grid, block, 0, st, a);
+            else hipLaunchKernelGGL((prefill_bf16_kernel<64, true>), grid, block, 0, st, a);
+        } else {
+            if (D == 128) hipLaunchKernelGGL((prefill_bf16_kernel<128, false>), grid, block, 0, st, a);
+            else hipLaunchKernelGGL((prefill_bf16_kernel<64, false>), grid, block, 0, st, a);
+        }
+    } else {
+        if (D == 128) hipLaunchKernelGGL(prefill_f32_kernel<128>, grid, block, 0, st, a);
+        else hipLaunchKernelGGL(prefill_f32_kernel<64>, grid, block, 0, st, a);
+    }
+    return check_launch();
+}
+
 }  // namespace
+
+int check_kv_cache(const vsp_kv_cache* c);  // kv_cache.hip
+
 }  // namespace vsp
 
 using namespace vsp;
+
+extern "C" int vsp_attn_prefill_cached(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens,
+                                       vsp_tensor* out, vsp_tensor* lse, float scale, int is_causal, void* stream) {
+    if (!q || !out) return VSP_ERR_NULL;
+    int rc = check_kv_cache(cache);
+    if (rc != VSP_OK) return rc;
+    if (q->ndim != 4 || out->ndim != 4) return VSP_ERR_NDIM;
+    const int64_t B = q->shape[0], Hq = q->shape[1], T = q->shape[2], D = q->shape[3];
+    const int64_t Hkv = cache->Hkv;
+    if (B != cache->B || D != cache->D) return VSP_ERR_SHAPE;
+    if (Hkv <= 0 ? Hq != 0 : (Hq % Hkv != 0)) return VSP_ERR_SHAPE;
+    const int64_t L = seq_lens ? cache->S_max : cache->len;  // with seq_lens: the bound the device values are clamped to
+    if (T > L) return VSP_ERR_SHAPE;                          // the chunk is part of the context
+    for (int i = 0; i < 4; ++i)
+        if (out->shape[i] != q->shape[i]) return VSP_ERR_SHAPE;
+    if (out->dtype != q->dtype) return VSP_ERR_DTYPE;
+    if (cache->format == VSP_KV_Q8_0) return VSP_ERR_UNSUPPORTED;  // read the context out with vsp_kv_read first
+    if (q->dtype != (cache->format == VSP_KV_F32 ? VSP_F32 : VSP_BF16)) return VSP_ERR_DTYPE;
+    if (lse) {
+        if (lse->ndim != 3 || lse->shape[0] != B || lse->shape[1] != Hq || lse->shape[2] != T) return VSP_ERR_SHAPE;
+        if (lse->dtype != VSP_F32) return VSP_ERR_DTYPE;
+    }
+    if (B * Hq * T * D == 0) return VSP_OK;
+    if (D != 64 && D != 128) return VSP_ERR_UNSUPPORTED;
+    if (!(fabsf(scale) > 0.0f) || !(fabsf(scale) < INFINITY)) return VSP_ERR_ARG;
+    const int esz = q->dtype == VSP_F32 ? 4 : 2;
+    if ((rc = check_tensor4(q, esz)) != VSP_OK || (rc = check_tensor4(out, esz)) != VSP_OK) return rc;
+    if (lse && !lse->data) return VSP_ERR_NULL;
+    if (T > INT32_MAX / 2) return VSP_ERR_ARG;
+
+    PrefillArgs a{};
+    a.q = q->data;
+    a.k = cache->k;
+    a.v = cache->v;
+    a.out = out->data;
+    a.lse = lse ? (float*)lse->data : nullptr;
+    const int64_t s_phys = kv_s_pad(cache->format, cache->S_max);
+    for (int i = 0; i < 3; ++i) {
+        a.sq[i] = q->stride[i];
+        a.so[i] = out->stride[i];
+        a.sl[i] = lse ? lse->stride[i] : 0;
+    }
+    a.sk[0] = a.sv[0] = Hkv * s_phys * D;
+    a.sk[1] = a.sv[1] = s_phys * D;
+    a.sk[2] = a.sv[2] = D;
+    a.B = (int)B;
+    a.Hq = (int)Hq;
+    a.Hkv = (int)Hkv;
+    a.n_rep = (int)(Hq / Hkv);
+    a.T = (int)T;
+    a.L = (int)L;
+    a.s_pad = (int)s_phys;
+    a.seq_lens = seq_lens;
+    a.causal = is_causal ? 1 : 0;
+    a.n_qtiles = (int)ceil_div(T, kBM);
+    a.negate_q = (q->dtype == VSP_BF16 && scale < 0.0f) ? 1 : 0;
+    a.scale_log2 = (q->dtype == VSP_BF16 ? fabsf(scale) : scale) * kLog2e;
+    return launch_prefill(a, q->dtype, D, cache->format == VSP_KV_BF16, stream);
+}
 
 extern "C" int vsp_attn_prefill(const vsp_tensor* q, const vsp_tensor* k, const vsp_tensor* v, vsp_tensor* out,
                                 vsp_tensor* lse, float scale, int is_causal, float dropout_p, int training,
@@ -508,7 +648,7 @@ extern "C" int vsp_attn_prefill(const vsp_tensor* q, const vsp_tensor* k, const 
     if (lse && !lse->data) return VSP_ERR_NULL;
     if (T > INT32_MAX / 2 || L > INT32_MAX / 2) return VSP_ERR_ARG;
 
-    PrefillArgs a;
+    PrefillArgs a{};
     a.q = q->data;
     a.k = k->data;
     a.v = v->data;
@@ -531,16 +671,5 @@ extern "C" int vsp_attn_prefill(const vsp_tensor* q, const vsp_tensor* k, const 
     a.n_qtiles = (int)ceil_div(T, kBM);
     a.negate_q = (q->dtype == VSP_BF16 && scale < 0.0f) ? 1 : 0;
     a.scale_log2 = (q->dtype == VSP_BF16 ? fabsf(scale) : scale) * kLog2e;
-    const int64_t blocks = (int64_t)a.n_qtiles * B * Hq;
-    if (blocks > INT32_MAX) return VSP_ERR_ARG;
-    hipStream_t st = (hipStream_t)stream;
-    dim3 grid((unsigned)blocks), block(256);
-    if (q->dtype == VSP_BF16) {
-        if (D == 128) hipLaunchKernelGGL(prefill_bf16_kernel<128>, grid, block, 0, st, a);
-        else hipLaunchKernelGGL(prefill_bf16_kernel<64>, grid, block, 0, st, a);
-    } else {
-        if (D == 128) hipLaunchKernelGGL(prefill_f32_kernel<128>, grid, block, 0, st, a);
-        else hipLaunchKernelGGL(prefill_f32_kernel<64>, grid, block, 0, st, a);
-    }
-    return check_launch();
+    return launch_prefill(a, q->dtype, D, false, stream);
 }
