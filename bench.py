@@ -36,6 +36,12 @@ WORKLOADS = {
                name="BASELINE config 4: batched decode bf16 KV cache, B32, 32 q / 8 kv heads, D128, L~U[1024,32768]"),
     "c5": dict(kind="decode", fmt="q8_0", B=16, Hq=64, Hkv=8, D=128, S=65536, lens=None,
                name="BASELINE config 5: decode over Q8_0 KV cache, B16, 64 q / 8 kv heads, D128, L=65536"),
+    "c2c": dict(kind="prefill_cached", fmt="bf16", B=4, Hq=32, Hkv=8, D=128, N=2048,
+                name="config 2 through the cache: causal GQA prefill bf16 reading K/V from the bf16 cache planes, "
+                     "B4, 32 q / 8 kv heads, D128, N2048"),
+    "c3c": dict(kind="prefill_cached", fmt="bf16", B=1, Hq=32, Hkv=8, D=128, N=8192,
+                name="config 3 through the cache: causal GQA prefill bf16 reading K/V from the bf16 cache planes, "
+                     "B1, 32 q / 8 kv heads, D128, N8192"),
     "r2": dict(kind="rope", fmt="bf16", B=4, Hq=32, Hkv=8, D=128, N=2048,
                name="RoPE + KV append for config 2: q/k/v bf16 views of one fused projection buffer [B,T,(Hq+2Hkv)D], "
                     "rotated q out bf16, bf16 cache, B4, 32 q / 8 kv heads, D128, T2048"),
@@ -71,7 +77,16 @@ class Runner:
             self.scale = 1.0 / math.sqrt(D)
             self.work = prefill_flops(w)
             self.unit, self.peak, self.bound = "TFLOP/s", MFMA_BF16_PEAK_TFLOPS, "mfma"
-            self.kernel = "prefill_bf16_kernel<128>"
+            self.kernel = "prefill_bf16_kernel<128, false>"
+        elif w["kind"] == "prefill_cached":
+            B, Hq, Hkv, D, N = w["B"], w["Hq"], w["Hkv"], w["D"], w["N"]
+            mk = lambda h: (torch.randn(B, h, N, D, device=dev, generator=g) * 0.5).to(torch.bfloat16)
+            self.q = mk(Hq)
+            self.cache = va.KVCache(B, Hkv, N, D, fmt=w["fmt"])
+            self.cache.update(mk(Hkv), mk(Hkv), 0, return_views=False)
+            self.work = prefill_flops(w)
+            self.unit, self.peak, self.bound = "TFLOP/s", MFMA_BF16_PEAK_TFLOPS, "mfma"
+            self.kernel = "prefill_bf16_kernel<128, true>"
         elif w["kind"] == "rope":
             B, Hq, Hkv, D, N = w["B"], w["Hq"], w["Hkv"], w["D"], w["N"]
             fused = (torch.randn(B, N, (Hq + 2 * Hkv) * D, device=dev, generator=g) * 0.5).to(torch.bfloat16)
@@ -130,6 +145,8 @@ class Runner:
     def step(self):
         if self.w["kind"] == "prefill":
             return self.va.flash_attention(self.q, self.k, self.v, self.scale, True)
+        if self.w["kind"] == "prefill_cached":
+            return self.cache.prefill(self.q)
         if self.w["kind"] == "rope":
             return self.cache.rope_update(self.q, self.k, self.v, 0, self.rope, out=self.out)
         return self.va.decode_attention(self.q, self.cache, seq_lens=self.seq_lens, max_len=self.max_len,
@@ -282,7 +299,7 @@ def main():
 
     if not args.no_extra:
         others = {}
-        for key in ("c2", "p4k", "c3", "c4", "c5", "r2"):
+        for key in ("c2", "p4k", "c3", "c4", "c5", "c2c", "c3c", "r2"):
             if key == args.workload:
                 continue
             r = Runner(key, torch, va)
