@@ -196,10 +196,15 @@ int vsp_attn_prefill(const vsp_tensor* q, const vsp_tensor* k, const vsp_tensor*
  * j <= L_b - T + t when is_causal, all L_b keys otherwise.
  *   VSP_KV_F32 : q/out fp32, fp32 arithmetic.   VSP_KV_BF16 : q/out bf16; K rows and token-blocked V are
  *   consumed in place (V^T operands are plain 16-byte reads of the blocked plane).
- *   VSP_KV_Q8_0: VSP_ERR_UNSUPPORTED (materialise the context with vsp_kv_read and call vsp_attn_prefill).
+ *   VSP_KV_Q8_0: q/out bf16; rows [0, L) are first dequantised to dense bf16 in `workspace`
+ *                (vsp_attn_prefill_cached_workspace_bytes() bytes, 16-byte aligned; else VSP_ERR_WORKSPACE) and
+ *                the dense kernel runs over that: prefill is compute-bound, the read-out is ~0.2 % of its time.
+ *                The other formats need no workspace (NULL, 0).
  * Tokens past L_b in the planes are never used, whatever they hold.  lse as in vsp_attn_prefill. */
+size_t vsp_attn_prefill_cached_workspace_bytes(const vsp_kv_cache* cache, int with_seq_lens);
 int vsp_attn_prefill_cached(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, vsp_tensor* out,
-                            vsp_tensor* lse, float scale, int is_causal, void* stream);
+                            vsp_tensor* lse, float scale, int is_causal, void* workspace, size_t workspace_bytes,
+                            void* stream);
 
 /* ---- decode -------------------------------------------------------------------
  * Replaces, for T == 1, the op chain scaled_dot_product_attention runs below its flash threshold

@@ -121,11 +121,33 @@ def test_chunked_equals_one_shot_at_config2_size(va):
     assert torch.equal(again, outs[1])  # run-to-run deterministic
 
 
+def test_q8_0_cache(va):
+    # the oracle attends over what the cache holds: the dequantised rows
+    B, Hq, Hkv, L, T, D, S_max = 2, 8, 2, 140, 60, 128, 200
+    q, k, v = [O.bf16_round(x * np.float32(0.5)) for x in I.qkv(3400, B, Hq, Hkv, L, L, D)]
+    c = va.KVCache(B, Hkv, S_max, D, fmt="q8_0")
+    c.update(G.to_bf16_dev(k), G.to_bf16_dev(v), 0, return_views=False)
+    kq, vq = O.q8_0_dequantize(*O.q8_0_quantize(k)), O.q8_0_dequantize(*O.q8_0_quantize(v))
+    out = c.prefill(G.to_bf16_dev(q[:, :, L - T:]))
+    G.assert_bf16_close(G.bf16_to_np(out), _expected(q, kq, vq, L, T), "q8_0 planes")
+    lens = torch.tensor([140, 75], dtype=torch.int32, device=G.dev())
+    qc = np.stack([q[0, :, 80:140], q[1, :, 15:75]])
+    out2 = G.bf16_to_np(c.prefill(G.to_bf16_dev(qc), seq_lens=lens))
+    G.assert_bf16_close(out2[0:1], _expected(q[0:1], kq[0:1], vq[0:1], 140, 60), "row 0")
+    G.assert_bf16_close(out2[1:2], _expected(q[1:2], kq[1:2], vq[1:2], 75, 60), "row 1")
+    # a missing workspace is an error, not a silent fallback
+    import ctypes as C
+    from vesper_amd import _ffi
+    from vesper_amd.api import _desc, _stream
+    qd = G.to_bf16_dev(q[:, :, L - T:])
+    od = torch.empty_like(qd)
+    dq, do = _desc(qd), _desc(od)
+    rc = _ffi.lib.vsp_attn_prefill_cached(C.byref(dq), C.byref(c._c), None, C.byref(do), None, 0.1, 1, None, 0, _stream(qd))
+    assert rc == _ffi.ERR_WORKSPACE
+
+
 def test_argument_errors(va):
-    c8 = va.KVCache(1, 2, 64, 64, fmt="q8_0")
     q = torch.zeros(1, 4, 8, 64, device=G.dev(), dtype=torch.bfloat16)
-    with pytest.raises(va.VspError):
-        c8.prefill(q)
     c = va.KVCache(1, 2, 64, 64, fmt="bf16")
     with pytest.raises(va.VspError):      # chunk longer than the context (len == 0)
         c.prefill(q)

@@ -133,8 +133,11 @@ class KVCache:
         dl = _desc(lse) if lse is not None else None
         sl = C.c_void_p(seq_lens.data_ptr()) if seq_lens is not None else None
         sc = float(scale) if scale is not None else 1.0 / math.sqrt(q.shape[-1])
+        nws = lib.vsp_attn_prefill_cached_workspace_bytes(C.byref(self._c), int(seq_lens is not None))
+        ws = torch.empty(nws, dtype=torch.uint8, device=q.device) if nws else None
         check(lib.vsp_attn_prefill_cached(C.byref(dq), C.byref(self._c), sl, C.byref(do),
-                                          C.byref(dl) if dl is not None else None, sc, int(bool(is_causal)), _stream(q)))
+                                          C.byref(dl) if dl is not None else None, sc, int(bool(is_causal)),
+                                          C.c_void_p(ws.data_ptr()) if ws is not None else None, nws, _stream(q)))
         return (out, lse) if return_lse else out
 
     # -- reads

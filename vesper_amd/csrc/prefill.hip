@@ -158,7 +158,7 @@ __global__ void __launch_bounds__(256, 3) prefill_bf16_kernel(PrefillArgs a) {
     }
     const int b = bh / a.Hq, hq = bh % a.Hq, kvh = hq / a.n_rep;
     int L = a.L;
-    if (VBLK && a.seq_lens) L = min(max(a.seq_lens[b], a.T), a.L);  // a.L = capacity bound in this mode
+    if (a.seq_lens) L = min(max(a.seq_lens[b], a.T), a.L);  // cache mode: a.L is the bound the device values are clamped to
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -551,8 +551,18 @@ int check_kv_cache(const vsp_kv_cache* c);  // kv_cache.hip
 
 using namespace vsp;
 
+extern "C" size_t vsp_attn_prefill_cached_workspace_bytes(const vsp_kv_cache* cache, int with_seq_lens) {
+    if (!cache || cache->format != VSP_KV_Q8_0) return 0;
+    const int64_t rows = with_seq_lens ? cache->S_max : cache->len;
+    return (size_t)2 * (size_t)cache->B * (size_t)cache->Hkv * (size_t)rows * (size_t)cache->D * 2;  // K and V, bf16
+}
+
+extern "C" int vsp_kv_read(const vsp_kv_cache* cache, int64_t start, int64_t count, vsp_tensor* k_out, vsp_tensor* v_out,
+                           void* stream);
+
 extern "C" int vsp_attn_prefill_cached(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens,
-                                       vsp_tensor* out, vsp_tensor* lse, float scale, int is_causal, void* stream) {
+                                       vsp_tensor* out, vsp_tensor* lse, float scale, int is_causal, void* workspace,
+                                       size_t workspace_bytes, void* stream) {
     if (!q || !out) return VSP_ERR_NULL;
     int rc = check_kv_cache(cache);
     if (rc != VSP_OK) return rc;
@@ -566,7 +576,6 @@ extern "C" int vsp_attn_prefill_cached(const vsp_tensor* q, const vsp_kv_cache* 
     for (int i = 0; i < 4; ++i)
         if (out->shape[i] != q->shape[i]) return VSP_ERR_SHAPE;
     if (out->dtype != q->dtype) return VSP_ERR_DTYPE;
-    if (cache->format == VSP_KV_Q8_0) return VSP_ERR_UNSUPPORTED;  // read the context out with vsp_kv_read first
     if (q->dtype != (cache->format == VSP_KV_F32 ? VSP_F32 : VSP_BF16)) return VSP_ERR_DTYPE;
     if (lse) {
         if (lse->ndim != 3 || lse->shape[0] != B || lse->shape[1] != Hq || lse->shape[2] != T) return VSP_ERR_SHAPE;
@@ -586,11 +595,34 @@ extern "C" int vsp_attn_prefill_cached(const vsp_tensor* q, const vsp_kv_cache* 
     a.v = cache->v;
     a.out = out->data;
     a.lse = lse ? (float*)lse->data : nullptr;
-    const int64_t s_phys = kv_s_pad(cache->format, cache->S_max);
+    int64_t s_phys = kv_s_pad(cache->format, cache->S_max);
     for (int i = 0; i < 3; ++i) {
         a.sq[i] = q->stride[i];
         a.so[i] = out->stride[i];
         a.sl[i] = lse ? lse->stride[i] : 0;
+    }
+    if (cache->format == VSP_KV_Q8_0) {
+        // Compute-bound path: dequantising inside the MFMA loop would add vector-ALU work to a kernel that is
+        // already short of it, while reading the context out once costs ~0.2 % of the attention time.  The rows
+        // [0, L) are dequantised to dense bf16 in the workspace and the dense kernel runs over that.
+        const size_t need = vsp_attn_prefill_cached_workspace_bytes(cache, seq_lens != nullptr);
+        if (!workspace || workspace_bytes < need) return VSP_ERR_WORKSPACE;
+        if (!is_aligned16(workspace)) return VSP_ERR_ALIGN;
+        vsp_tensor kt{}, vt{};
+        kt.dtype = vt.dtype = VSP_BF16;
+        kt.ndim = vt.ndim = 4;
+        const int64_t shp[4] = {B, Hkv, L, D};
+        for (int i = 0; i < 4; ++i) kt.shape[i] = vt.shape[i] = shp[i];
+        kt.stride[3] = vt.stride[3] = 1;
+        kt.stride[2] = vt.stride[2] = D;
+        kt.stride[1] = vt.stride[1] = L * D;
+        kt.stride[0] = vt.stride[0] = Hkv * L * D;
+        kt.data = workspace;
+        vt.data = (char*)workspace + need / 2;
+        if ((rc = vsp_kv_read(cache, 0, L, &kt, &vt, stream)) != VSP_OK) return rc;
+        a.k = kt.data;
+        a.v = vt.data;
+        s_phys = L;
     }
     a.sk[0] = a.sv[0] = Hkv * s_phys * D;
     a.sk[1] = a.sv[1] = s_phys * D;
