@@ -130,8 +130,8 @@ int vsp_kv_cache_reset(vsp_kv_cache* cache, void* stream);
  * Afterwards len = max(len, start_pos + T).
  * start_pos_dev (nullable): device int32[B], per-sequence start positions for ragged batches
  * (no counterpart in the reference, which has one position for the batch); when given, start_pos
- * is ignored for placement, each row b is written at start_pos_dev[b] (caller guarantees
- * 0 <= start_pos_dev[b] and start_pos_dev[b]+T <= S_max) and len is left unchanged. */
+ * is ignored for placement, each row b is written at start_pos_dev[b] (0 <= start_pos_dev[b],
+ * start_pos_dev[b]+T <= S_max; tokens that would land outside the planes are dropped) and len is left unchanged. */
 int vsp_kv_append(vsp_kv_cache* cache, const vsp_tensor* new_k, const vsp_tensor* new_v, int64_t start_pos,
                   const int32_t* start_pos_dev, void* stream);
 
@@ -200,11 +200,19 @@ int vsp_attn_prefill(const vsp_tensor* q, const vsp_tensor* k, const vsp_tensor*
  *                (vsp_attn_prefill_cached_workspace_bytes() bytes, 16-byte aligned; else VSP_ERR_WORKSPACE) and
  *                the dense kernel runs over that: prefill is compute-bound, the read-out is ~0.2 % of its time.
  *                The other formats need no workspace (NULL, 0).
- * Tokens past L_b in the planes are never used, whatever they hold.  lse as in vsp_attn_prefill. */
+ * Tokens past L_b in the planes are never used, whatever they hold.  lse as in vsp_attn_prefill.
+ * chunk_lens (nullable): device int32[B], n_b <= T valid query rows per sequence (ragged chunks in one call):
+ * query t < n_b sits at position L_b - n_b + t; rows t >= n_b of `out` are unspecified. */
 size_t vsp_attn_prefill_cached_workspace_bytes(const vsp_kv_cache* cache, int with_seq_lens);
-int vsp_attn_prefill_cached(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, vsp_tensor* out,
-                            vsp_tensor* lse, float scale, int is_causal, void* workspace, size_t workspace_bytes,
-                            void* stream);
+int vsp_attn_prefill_cached(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens,
+                            const int32_t* chunk_lens, vsp_tensor* out, vsp_tensor* lse, float scale, int is_causal,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
+/* Ragged batches keep their lengths on the device (the reference's caches have one host-side length for the
+ * whole batch, src/nn/transformer.cpp:73): after vsp_kv_append / vsp_rope_kv_append with start_pos_dev = seq_lens,
+ * this advances them in stream order: seq_lens[b] = min(seq_lens[b] + n_b, S_max), n_b = n_new[b] clamped to
+ * [0, T], or T when n_new is NULL.  The same array is what vsp_attn_decode and vsp_attn_prefill_cached take. */
+int vsp_seq_lens_advance(int32_t* seq_lens, const int32_t* n_new, int32_t T, int32_t B, int32_t S_max, void* stream);
 
 /* ---- decode -------------------------------------------------------------------
  * Replaces, for T == 1, the op chain scaled_dot_product_attention runs below its flash threshold

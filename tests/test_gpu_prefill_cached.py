@@ -142,7 +142,7 @@ def test_q8_0_cache(va):
     qd = G.to_bf16_dev(q[:, :, L - T:])
     od = torch.empty_like(qd)
     dq, do = _desc(qd), _desc(od)
-    rc = _ffi.lib.vsp_attn_prefill_cached(C.byref(dq), C.byref(c._c), None, C.byref(do), None, 0.1, 1, None, 0, _stream(qd))
+    rc = _ffi.lib.vsp_attn_prefill_cached(C.byref(dq), C.byref(c._c), None, None, C.byref(do), None, 0.1, 1, None, 0, _stream(qd))
     assert rc == _ffi.ERR_WORKSPACE
 
 

@@ -124,7 +124,7 @@ class KVCache:
                                      C.c_void_p(rope.table.data_ptr()), rope.length, int(start_pos), sp, _stream(q)))
         return (q_out, self.views()) if return_views else q_out
 
-    def prefill(self, q, seq_lens=None, is_causal=True, scale=None, return_lse=False):
+    def prefill(self, q, seq_lens=None, is_causal=True, scale=None, return_lse=False, chunk_lens=None):
         """Attention of the last T tokens (q [B,Hq,T,D]) over the cached context, read in place from the planes:
         chunked prefill.  seq_lens: device int32[B] per-row context lengths (default: the cache's one length)."""
         out = torch.empty_like(q)
@@ -132,10 +132,11 @@ class KVCache:
         dq, do = _desc(q), _desc(out)
         dl = _desc(lse) if lse is not None else None
         sl = C.c_void_p(seq_lens.data_ptr()) if seq_lens is not None else None
+        cl = C.c_void_p(chunk_lens.data_ptr()) if chunk_lens is not None else None
         sc = float(scale) if scale is not None else 1.0 / math.sqrt(q.shape[-1])
         nws = lib.vsp_attn_prefill_cached_workspace_bytes(C.byref(self._c), int(seq_lens is not None))
         ws = torch.empty(nws, dtype=torch.uint8, device=q.device) if nws else None
-        check(lib.vsp_attn_prefill_cached(C.byref(dq), C.byref(self._c), sl, C.byref(do),
+        check(lib.vsp_attn_prefill_cached(C.byref(dq), C.byref(self._c), sl, cl, C.byref(do),
                                           C.byref(dl) if dl is not None else None, sc, int(bool(is_causal)),
                                           C.c_void_p(ws.data_ptr()) if ws is not None else None, nws, _stream(q)))
         return (out, lse) if return_lse else out
@@ -177,6 +178,46 @@ class KVCache:
 
 class GQAKVCache(KVCache):
     """nn::GQAKVCache: same semantics, int64 bookkeeping in the reference."""
+
+
+class RaggedKVCache(KVCache):
+    """A cache whose rows have their own lengths, kept in a device int32[B] array (the reference's caches have
+    one host-side length for the batch).  Every step is asynchronous: nothing is read back to the host.
+    `upper` is a host-side upper bound of the longest row, used only to size work (grids, workspaces)."""
+
+    def __init__(self, batch_size, num_heads, max_seq_len, head_dim, device="cuda", fmt="bf16"):
+        super().__init__(batch_size, num_heads, max_seq_len, head_dim, device=device, fmt=fmt)
+        self.seq_lens = torch.zeros(batch_size, dtype=torch.int32, device=self.device)
+        self.upper = 0
+
+    def reset_rows(self, rows):
+        """Forget the given rows (a finished request leaves the batch); their tokens become stale, not zero."""
+        self.seq_lens[torch.as_tensor(rows, device=self.device, dtype=torch.long)] = 0
+
+    def _advance(self, n_new, T, ref):
+        nn_ = C.c_void_p(n_new.data_ptr()) if n_new is not None else None
+        check(lib.vsp_seq_lens_advance(C.c_void_p(self.seq_lens.data_ptr()), nn_, int(T), self._c.B, self._c.S_max,
+                                       _stream(ref)))
+        self.upper = min(self.upper + int(T), self._c.S_max)
+
+    def append(self, new_k, new_v, n_new=None, q=None, rope=None, q_dtype=None):
+        """Row b's first n_new[b] (default: all T) tokens go to positions seq_lens[b]..; with `rope`, q and k are
+        rotated at those positions in the same launch and the rotated q is returned."""
+        T = new_k.shape[2]
+        if rope is not None:
+            out = self.rope_update(q, new_k, new_v, 0, rope, out_dtype=q_dtype, start_pos_dev=self.seq_lens)
+        else:
+            self.update(new_k, new_v, 0, return_views=False, start_pos_dev=self.seq_lens)
+            out = None
+        self._advance(n_new, T, new_k)
+        return out
+
+    def decode(self, q, scale=None, out=None):
+        return decode_attention(q, self, seq_lens=self.seq_lens, max_len=max(self.upper, 1), scale=scale, out=out)
+
+    def prefill_chunk(self, q, n_new=None, scale=None):
+        """Attention of the chunk just appended (q [B,Hq,T,D], row b valid for n_new[b] rows) over each row's context."""
+        return self.prefill(q, seq_lens=self.seq_lens, chunk_lens=n_new, scale=scale)
 
 
 _WS = {}

@@ -144,6 +144,7 @@ __global__ void __launch_bounds__(256) append_f32_kernel(AppendArgs a) {
     if (i >= a.rows * per_row) return;
     const int64_t r = i / per_row, d0 = (i % per_row) * 4;
     const RowMap m = map_row(a, r);
+    if (m.s < 0 || m.s >= a.S) return;  // a device-side position outside the planes: drop the token, never write out of bounds
     const SrcT* pk = (const SrcT*)a.src_k + m.src_off_k + d0;
     const SrcT* pv = (const SrcT*)a.src_v + m.src_off_v + d0;
     float* dk = (float*)a.k + kv_off_rowmajor(a.H, a.S, a.D, m.b, m.h, m.s, d0);
@@ -174,6 +175,7 @@ __global__ void __launch_bounds__(256) append_bf16_kernel(AppendArgs a) {
     if (i >= a.rows * per_row) return;
     const int64_t r = i / per_row, d0 = (i % per_row) * 8;
     const RowMap m = map_row(a, r);
+    if (m.s < 0 || m.s >= a.S) return;  // a device-side position outside the planes: drop the token, never write out of bounds
     const SrcT* pk = (const SrcT*)a.src_k + m.src_off_k + d0;
     const SrcT* pv = (const SrcT*)a.src_v + m.src_off_v + d0;
     uint16_t kb[8], vb[8];
@@ -240,6 +242,7 @@ __global__ void __launch_bounds__(128) append_q8_kernel(AppendArgs a) {
     if (i >= a.rows * per_row) return;
     const int64_t r = i / per_row, blk = i % per_row, d0 = blk * kQBlock;
     const RowMap m = map_row(a, r);
+    if (m.s < 0 || m.s >= a.S) return;  // a device-side position outside the planes: drop the token, never write out of bounds
     const SrcT* pk = (const SrcT*)a.src_k + m.src_off_k + d0;
     const SrcT* pv = (const SrcT*)a.src_v + m.src_off_v + d0;
     float x[kQBlock];
@@ -350,6 +353,15 @@ __global__ void __launch_bounds__(256) read_q8_raw_kernel(const int8_t* __restri
         qs_out[i] = qs[kv_off_vblocked(H, S, D, kVBlkQ8, b, h, s, d)];
         if (d % kQBlock == 0) sc_out[i / kQBlock] = sc[kv_off_vscale(H, S, D, b, h, s, d / kQBlock)];
     }
+}
+
+// lens[b] = min(lens[b] + (n_new ? clamp(n_new[b], 0, T) : T), S_max)
+__global__ void __launch_bounds__(256) advance_lens_kernel(int32_t* __restrict__ lens, const int32_t* __restrict__ n_new,
+                                                           int32_t T, int32_t B, int32_t S_max) {
+    const int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= B) return;
+    const int n = n_new ? min(max(n_new[b], 0), T) : T;
+    lens[b] = min(lens[b] + n, S_max);
 }
 
 int check_cache(const vsp_kv_cache* c) {
@@ -536,6 +548,15 @@ int vsp_rope_kv_append(vsp_kv_cache* cache, const vsp_tensor* q, const vsp_tenso
                        const int32_t* start_pos_dev, void* stream) {
     RopeParams rp{q, q_out, rope_table, table_len};
     return append_impl(cache, new_k, new_v, start_pos, start_pos_dev, &rp, stream);
+}
+
+int vsp_seq_lens_advance(int32_t* seq_lens, const int32_t* n_new, int32_t T, int32_t B, int32_t S_max, void* stream) {
+    if (B < 0 || T < 0 || S_max < 0) return VSP_ERR_ARG;
+    if (B == 0) return VSP_OK;
+    if (!seq_lens) return VSP_ERR_NULL;
+    hipLaunchKernelGGL(advance_lens_kernel, dim3((unsigned)ceil_div(B, 256)), dim3(256), 0, (hipStream_t)stream, seq_lens,
+                       n_new, T, B, S_max);
+    return check_launch();
 }
 
 int vsp_kv_read(const vsp_kv_cache* cache, int64_t start, int64_t count, vsp_tensor* k_out, vsp_tensor* v_out,

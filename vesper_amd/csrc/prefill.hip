@@ -47,6 +47,7 @@ struct PrefillArgs {
     int32_t negate_q;  // scale < 0: flip the sign of Q (exact) and use |scale|
     int32_t s_pad;     // cache-plane mode: padded token capacity of the planes
     const int32_t* seq_lens;  // cache-plane mode: per-batch context lengths (device) or nullptr
+    const int32_t* chunk_lens;  // cache-plane mode: per-batch number of valid query rows (device) or nullptr
     float scale_log2;  // |scale| * log2(e) for bf16; scale * log2(e) for fp32
 };
 
@@ -158,13 +159,16 @@ __global__ void __launch_bounds__(256, 3) prefill_bf16_kernel(PrefillArgs a) {
     }
     const int b = bh / a.Hq, hq = bh % a.Hq, kvh = hq / a.n_rep;
     int L = a.L;
-    if (a.seq_lens) L = min(max(a.seq_lens[b], a.T), a.L);  // cache mode: a.L is the bound the device values are clamped to
+    // cache mode: per-row context length (clamped to the bound a.L) and per-row chunk length n <= T:
+    // query t < n sits at absolute position L - n + t; rows t >= n carry no query and their output is unspecified
+    const int n_chunk = a.chunk_lens ? min(max(a.chunk_lens[b], 0), a.T) : a.T;
+    if (a.seq_lens) L = min(max(a.seq_lens[b], n_chunk), a.L);
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int ql = lane & 31, h = lane >> 5;
     const int q0 = qt * kBM + wave * 32;
-    const int off = L - a.T;
+    const int off = L - n_chunk;
     const int qrow = min(q0 + ql, a.T - 1);
 
     const uint16_t* Qp = (const uint16_t*)a.q + (int64_t)b * a.sq[0] + (int64_t)hq * a.sq[1];
@@ -385,7 +389,7 @@ __global__ void __launch_bounds__(256, 3) prefill_bf16_kernel(PrefillArgs a) {
     l = half_swap_sum(l);
     const int qi = q0 + ql;
     if (qi < a.T) {
-        const float inv_l = 1.0f / l;
+        const float inv_l = l > 0.f ? 1.0f / l : 0.f;  // an empty context (cache mode, length 0) gives zeros
         uint16_t* op = (uint16_t*)a.out + (int64_t)b * a.so[0] + (int64_t)hq * a.so[1] + (int64_t)qi * a.so[2];
 #pragma unroll
         for (int db = 0; db < DB; ++db)
@@ -419,11 +423,12 @@ __global__ void __launch_bounds__(256) prefill_f32_kernel(PrefillArgs a) {
     const int qt = a.n_qtiles - 1 - bid / (a.B * a.Hq);
     const int bh = bid % (a.B * a.Hq);
     const int b = bh / a.Hq, hq = bh % a.Hq, kvh = hq / a.n_rep;
-    const int L = a.seq_lens ? min(max(a.seq_lens[b], a.T), a.L) : a.L;  // per-row context length (cache mode)
+    const int n_chunk = a.chunk_lens ? min(max(a.chunk_lens[b], 0), a.T) : a.T;  // cache mode, as in the bf16 kernel
+    const int L = a.seq_lens ? min(max(a.seq_lens[b], n_chunk), a.L) : a.L;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int ql = lane & 31, h = lane >> 5;
     const int q0 = qt * kBM + wave * 32;
-    const int off = L - a.T;
+    const int off = L - n_chunk;
     const int qrow = min(q0 + ql, a.T - 1);
 
     const float* Qp = (const float*)a.q + (int64_t)b * a.sq[0] + (int64_t)hq * a.sq[1] + (int64_t)qrow * a.sq[2];
@@ -503,7 +508,7 @@ __global__ void __launch_bounds__(256) prefill_f32_kernel(PrefillArgs a) {
     l = half_swap_sum(l);
     const int qi = q0 + ql;
     if (qi < a.T) {
-        const float inv_l = 1.0f / l;
+        const float inv_l = l > 0.f ? 1.0f / l : 0.f;  // an empty context (cache mode, length 0) gives zeros
         float* op = (float*)a.out + (int64_t)b * a.so[0] + (int64_t)hq * a.so[1] + (int64_t)qi * a.so[2];
 #pragma unroll
         for (int db = 0; db < DB; ++db)
@@ -561,8 +566,8 @@ extern "C" int vsp_kv_read(const vsp_kv_cache* cache, int64_t start, int64_t cou
                            void* stream);
 
 extern "C" int vsp_attn_prefill_cached(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens,
-                                       vsp_tensor* out, vsp_tensor* lse, float scale, int is_causal, void* workspace,
-                                       size_t workspace_bytes, void* stream) {
+                                       const int32_t* chunk_lens, vsp_tensor* out, vsp_tensor* lse, float scale,
+                                       int is_causal, void* workspace, size_t workspace_bytes, void* stream) {
     if (!q || !out) return VSP_ERR_NULL;
     int rc = check_kv_cache(cache);
     if (rc != VSP_OK) return rc;
@@ -635,6 +640,7 @@ extern "C" int vsp_attn_prefill_cached(const vsp_tensor* q, const vsp_kv_cache* 
     a.L = (int)L;
     a.s_pad = (int)s_phys;
     a.seq_lens = seq_lens;
+    a.chunk_lens = chunk_lens;
     a.causal = is_causal ? 1 : 0;
     a.n_qtiles = (int)ceil_div(T, kBM);
     a.negate_q = (q->dtype == VSP_BF16 && scale < 0.0f) ? 1 : 0;
