@@ -1,0 +1,70 @@
+"""The decode step (RoPE + append at device-side positions, length advance, split-K decode, combine) recorded
+into a HIP graph and replayed: every entry point is asynchronous, allocates nothing and records no memset node, so a
+serving loop can replay one graph per token.  Each replay is checked against the same step run eagerly, with the
+program's own eager work and synchronisations between replays."""
+import numpy as np
+import pytest
+import torch
+
+import _gpu as G
+import _inputs as I
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def va():
+    import vesper_amd
+    return vesper_amd
+
+
+@pytest.mark.parametrize("fmt", ["bf16", "q8_0"])
+def test_decode_step_replays_bit_identically(va, fmt):
+    B, Hq, Hkv, D, S_max, steps = 4, 16, 4, 128, 512, 4
+    rope = va.RopeTable(S_max, D)
+    prompts = [100, 37, 250, 5]
+
+    def make_cache():
+        c = va.RaggedKVCache(B, Hkv, S_max, D, fmt=fmt)
+        P = max(prompts)
+        q, k, v = I.qkv(5000, B, Hq, Hkv, P, P, D, scale=0.5)
+        c.append(G.f32_dev(k), G.f32_dev(v), n_new=torch.tensor(prompts, dtype=torch.int32, device=G.dev()),
+                 q=G.f32_dev(q), rope=rope, q_dtype=torch.bfloat16)
+        c.upper = P + steps  # host-side bound for the whole replayed range: the graph's grid must cover it
+        return c
+
+    toks = [I.qkv(5100 + 7 * i, B, Hq, Hkv, 1, 1, D, scale=0.5) for i in range(steps)]
+
+    # eager run
+    ce = make_cache()
+    eager = []
+    for q, k, v in toks:
+        qr = ce.append(G.f32_dev(k), G.f32_dev(v), q=G.f32_dev(q), rope=rope, q_dtype=torch.bfloat16)
+        eager.append(ce.decode(qr).clone())
+    torch.cuda.synchronize()
+
+    # graph run: static input/output buffers, one capture, one replay per token
+    cg = make_cache()
+    sq = torch.empty(B, Hq, 1, D, device=G.dev())
+    sk = torch.empty(B, Hkv, 1, D, device=G.dev())
+    sv = torch.empty(B, Hkv, 1, D, device=G.dev())
+    q_rot = torch.empty(B, Hq, 1, D, device=G.dev(), dtype=torch.bfloat16)
+    out = torch.empty_like(q_rot)
+    va.decode_attention(q_rot, cg, seq_lens=cg.seq_lens, max_len=cg.upper, out=out)  # sizes the shared workspace
+    lens0 = cg.seq_lens.clone()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            cg.rope_update(sq, sk, sv, 0, rope, start_pos_dev=cg.seq_lens, out=q_rot)
+            cg._advance(None, 1, sq)
+            va.decode_attention(q_rot, cg, seq_lens=cg.seq_lens, max_len=cg.upper, out=out)
+    torch.cuda.synchronize()
+    cg.seq_lens.copy_(lens0)  # capture does not execute; make sure the lengths are the prompt lengths
+    for i, (q, k, v) in enumerate(toks):
+        sq.copy_(G.f32_dev(q)), sk.copy_(G.f32_dev(k)), sv.copy_(G.f32_dev(v))  # eager work between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager[i]), f"replay {i}"
+    assert cg.seq_lens.cpu().tolist() == [p + steps for p in prompts]
