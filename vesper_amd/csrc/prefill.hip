@@ -65,7 +65,14 @@ __device__ inline uint32_t cvt_pk_bf16(float a, float b) {
 }
 
 // Reductions over the two half-waves (lane l and lane l ^ 32 hold the two halves of a query's keys).
-__device__ inline float half_swap_max(float x) { return fmaxf(x, __shfl_xor(x, 32)); }
+// v_permlane32_swap exchanges the upper half of its first operand with the lower half of its second; with a
+// copy of x in a second register both halves end up holding (lo[l], hi[l]) pairs: no LDS round trip.
+__device__ inline float half_swap_max(float x) {
+    float y;
+    // two wait states between a vector-ALU write and a permlane swap that reads it
+    asm volatile("v_mov_b32 %1, %0\n\ts_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(x), "=&v"(y));
+    return fmaxf(x, y);
+}
 __device__ inline float half_swap_sum(float x) { return x + __shfl_xor(x, 32); }
 
 // Transposing LDS read issued through inline asm: the compiler cannot prove that a builtin
