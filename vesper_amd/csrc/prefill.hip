@@ -85,11 +85,13 @@ __device__ inline uint2 lds_read_tr16_b64_asm(uint32_t lds_byte_addr) {
     asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(lds_byte_addr), "n"(OFFSET_BYTES));
     return v;
 }
-__device__ inline void tr_wait(uint2& a0, uint2& a1, uint2& a2, uint2& a3, uint2& a4, uint2& a5, uint2& a6, uint2& a7) {
-    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3), "+v"(a4), "+v"(a5), "+v"(a6), "+v"(a7));
+// `tie` is a value computed just before the point where the wait should sit: without it the compiler is free to
+// hoist the wait above independent vector-ALU work, which would expose the LDS latency the early read hides.
+__device__ inline void tr_wait(uint32_t& tie, uint2& a0, uint2& a1, uint2& a2, uint2& a3, uint2& a4, uint2& a5, uint2& a6, uint2& a7) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(tie), "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3), "+v"(a4), "+v"(a5), "+v"(a6), "+v"(a7));
 }
-__device__ inline void tr_wait(uint2& a0, uint2& a1, uint2& a2, uint2& a3) {
-    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3));
+__device__ inline void tr_wait(uint32_t& tie, uint2& a0, uint2& a1, uint2& a2, uint2& a3) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(tie), "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3));
 }
 // Plain 16-byte LDS read through inline asm, for the same reason; lds_wait<N>() waits until at most N of
 // this wave's LDS operations are outstanding (they return in order) and ties the wait to a value.
@@ -104,11 +106,11 @@ template <int N>
 __device__ inline void lds_wait(u32x4_t& a0) {
     asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(a0) : "n"(N));
 }
-__device__ inline void lds_wait0(u32x4_t& a0, u32x4_t& a1, u32x4_t& a2, u32x4_t& a3) {
-    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3));
+__device__ inline void lds_wait0(uint32_t& tie, u32x4_t& a0, u32x4_t& a1, u32x4_t& a2, u32x4_t& a3) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(tie), "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3));
 }
-__device__ inline void lds_wait0(u32x4_t& a0, u32x4_t& a1) {
-    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a0), "+v"(a1));
+__device__ inline void lds_wait0(uint32_t& tie, u32x4_t& a0, u32x4_t& a1) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(tie), "+v"(a0), "+v"(a1));
 }
 template <int... I, class F>
 __device__ inline void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
@@ -282,6 +284,18 @@ __global__ void __launch_bounds__(256, 3) prefill_bf16_kernel(PrefillArgs a) {
             s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kf[ks]), qf[ks], s[0], 0, 0, 0);
             if constexpr (ks + PF < KS) kf[ks + PF] = lds_read_b128_asm<KOFF>(kaddr[ks + PF]);
         });
+        // the first V fragments are requested now, so that their LDS latency passes under the softmax
+        u32x4_t vcur[DB];
+        uint2 tcur[DB][2];
+        if constexpr (VBLK) {
+            static_for<DB>([&](auto dbc) { vcur[dbc.value] = lds_read_b128_asm<VOFF + 512 * dbc.value>(va[dbc.value]); });
+        } else {
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                tcur[db][0] = lds_read_tr16_b64_asm<VOFF>(va[db]);
+                tcur[db][1] = lds_read_tr16_b64_asm<VOFF + 8 * D * 2>(va[db]);
+            }
+        }
         const bool need_mask = (a.causal && k0 + kUnit - 1 > q0 + off) || (k0 + kUnit > L);
         if (need_mask) {
             const int q_abs = q0 + ql + off;
@@ -320,13 +334,12 @@ __global__ void __launch_bounds__(256, 3) prefill_bf16_kernel(PrefillArgs a) {
         l += lsum;
         // PV
         if constexpr (VBLK) {
-            u32x4_t vcur[DB], vnext[DB];
-            static_for<DB>([&](auto dbc) { vcur[dbc.value] = lds_read_b128_asm<VOFF + 512 * dbc.value>(va[dbc.value]); });
+            u32x4_t vnext[DB];
             const bool tail = k0 + kUnit > L;  // the planes hold stale tokens past L: P is 0 there, V must not be NaN
             static_for<NJ>([&](auto jc) {
                 constexpr int j = jc.value;
-                if constexpr (DB == 4) lds_wait0(vcur[0], vcur[1], vcur[2], vcur[3]);
-                else lds_wait0(vcur[0], vcur[1]);
+                if constexpr (DB == 4) lds_wait0(pw[j][3], vcur[0], vcur[1], vcur[2], vcur[3]);
+                else lds_wait0(pw[j][3], vcur[0], vcur[1]);
                 if constexpr (j + 1 < NJ)
                     static_for<DB>([&](auto dbc) {
                         vnext[dbc.value] = lds_read_b128_asm<VOFF + (2 * (j + 1) * D + 32 * dbc.value) * 16>(va[dbc.value]);
@@ -354,16 +367,11 @@ __global__ void __launch_bounds__(256, 3) prefill_bf16_kernel(PrefillArgs a) {
             });
             return;
         }
-        uint2 tcur[DB][2], tnext[DB][2];
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-            tcur[db][0] = lds_read_tr16_b64_asm<VOFF>(va[db]);
-            tcur[db][1] = lds_read_tr16_b64_asm<VOFF + 8 * D * 2>(va[db]);
-        }
+        uint2 tnext[DB][2];
         static_for<NJ>([&](auto jc) {
             constexpr int j = jc.value;
-            if constexpr (DB == 4) tr_wait(tcur[0][0], tcur[0][1], tcur[1][0], tcur[1][1], tcur[2][0], tcur[2][1], tcur[3][0], tcur[3][1]);
-            else tr_wait(tcur[0][0], tcur[0][1], tcur[1][0], tcur[1][1]);
+            if constexpr (DB == 4) tr_wait(pw[j][3], tcur[0][0], tcur[0][1], tcur[1][0], tcur[1][1], tcur[2][0], tcur[2][1], tcur[3][0], tcur[3][1]);
+            else tr_wait(pw[j][3], tcur[0][0], tcur[0][1], tcur[1][0], tcur[1][1]);
             if constexpr (j + 1 < NJ) {
 #pragma unroll
                 for (int db = 0; db < DB; ++db) {
