@@ -156,9 +156,26 @@ class Runner:
         return self.work / seconds_per_step / (1e12 if self.unit == "TFLOP/s" else 1e9)
 
 
-def time_steps(torch, fn, steps, warmup):
-    """warmup untimed, then exactly `steps` steps: wall clock bracketed by synchronize, and device time
-    from events recorded on the launch stream around the same region."""
+CONDITION_SECONDS = 0.3
+
+
+def condition(torch, fn, seconds=CONDITION_SECONDS):
+    """Untimed: keep the GPU busy with the workload for a fixed wall time before the warm-up steps.  The part
+    raises its clocks over the first ~50 ms of sustained load (a 0.14 ms kernel takes 0.20 ms right after an
+    idle period and settles after ~300 launches); a serving process is always in the settled state, and a
+    warm-up counted in steps would measure the ramp for short kernels."""
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
+
+
+def time_steps(torch, fn, steps, warmup, conditioning=True):
+    """clock conditioning and `warmup` steps untimed, then exactly `steps` steps: wall clock bracketed by
+    synchronize, and device time from events recorded on the launch stream around the same region."""
+    if conditioning:
+        condition(torch, fn)
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -244,6 +261,8 @@ def main():
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="only the primary workload")
+    ap.add_argument("--no-conditioning", action="store_true",
+                    help="skip the fixed 0.3 s of untimed load that lets the clocks settle before the warm-up steps")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one 1 GiB read + 1 GiB write elementwise kernel (counter calibration for rocprofv3 --pmc)")
     args = ap.parse_args()
@@ -267,7 +286,7 @@ def main():
         del src, dst
 
     primary = Runner(args.workload, torch, va)
-    wall, dev = time_steps(torch, primary.step, args.steps, args.warmup)
+    wall, dev = time_steps(torch, primary.step, args.steps, args.warmup, not args.no_conditioning)
     value = primary.rate(wall)
     achieved = primary.rate(dev)
     result = {
@@ -291,6 +310,7 @@ def main():
                      "traffic": MEASURED_TRAFFIC.get(args.workload),
                      "kernel": primary.kernel, "kernel_ms": round(dev * 1e3, 5),
                      "timing": "HIP events on the launch stream around the timed steps / steps"},
+        "clock_conditioning_s": 0.0 if args.no_conditioning else CONDITION_SECONDS,
         "device": {"name": props.name, "cus": props.multi_processor_count,
                    "peak_used": f"{primary.peak} {primary.unit}"},
     }
@@ -304,7 +324,7 @@ def main():
                 continue
             r = Runner(key, torch, va)
             steps = max(10, args.steps // 2)
-            w_, d_ = time_steps(torch, r.step, steps, max(3, args.warmup // 2))
+            w_, d_ = time_steps(torch, r.step, steps, max(3, args.warmup // 2), not args.no_conditioning)
             others[key] = {"workload": r.w["name"], "value": round(r.rate(w_), 3), "unit": r.unit,
                            "ms_per_step": round(w_ * 1e3, 5), "kernel_ms": round(d_ * 1e3, 5),
                            "roofline_frac": round(r.rate(d_) / r.peak, 4), "bound": r.bound, "steps": steps}
