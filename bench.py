@@ -5,9 +5,9 @@
 
 A "step" is one pass of the hot path over one batch of synthetic input that is already resident in
 HBM: one prefill launch (c2, p4k, c3) or one decode call = split-K kernel + combine kernel (c4, c5).
-Prints ONE JSON line.  `value` is the primary workload's throughput (BASELINE config 2 by default:
+Prints ONE JSON line.  `value` is the primary workload's throughput (benchmark config 2 by default:
 causal GQA prefill bf16, B4, 32/8 heads, D128, N2048, in TFLOP/s of algorithmic causal FLOPs
-2*D*B*Hq*N*(N+1)); `other_workloads` carries the remaining BASELINE configs (decode in GB/s of
+2*D*B*Hq*N*(N+1)); `other_workloads` carries the remaining benchmark configs (decode in GB/s of
 algorithmic KV bytes).  `roofline` is for the primary workload's dominant kernel, timed with events
 on the launch stream; `cpu_baseline` is the reference's own CPU path (oracle/_ref, else the oracle
 port) timed on this host on a bounded sample of the same workload.

@@ -1,11 +1,11 @@
 """Helpers shared by the GPU parity tests: bit-level conversions between torch device tensors and the
-numpy arrays the oracle consumes, and the tolerances BASELINE states."""
+numpy arrays the oracle consumes, and the tolerances the benchmark definition states."""
 import numpy as np
 import torch
 
 import _oracle as O
 
-# BASELINE tolerances: bf16 max-abs 2e-2 / mean-abs 2e-3; fp32 1e-4 relative
+# benchmark tolerances: bf16 max-abs 2e-2 / mean-abs 2e-3; fp32 1e-4 relative
 BF16_MAX_ABS = 2e-2
 BF16_MEAN_ABS = 2e-3
 F32_REL = 1e-4

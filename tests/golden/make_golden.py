@@ -45,7 +45,7 @@ def flash_cases():
 
 
 def config1():
-    # BASELINE config 1: causal GQA fp32, B1, 8 q heads / 2 kv heads, D64, N256, scale 1/8:
+    # benchmark config 1: causal GQA fp32, B1, 8 q heads / 2 kv heads, D64, N256, scale 1/8:
     # repeat_kv -> flash_attention, and the same through scaled_dot_product_attention (N<512 => matmul branch).
     B, Hq, Hkv, N, D = 1, 8, 2, 256, 64
     q, k, v = I.qkv(1001, B, Hq, Hkv, N, N, D)

@@ -125,7 +125,7 @@ def test_decode_is_deterministic_and_ignores_stale_tail(va):
 
 
 def test_decode_config4_shape_properties(va):
-    # BASELINE config 4 at full size (B32, 32/8 heads, D128, S_max 32768, lengths U[1024, 32768]):
+    # benchmark config 4 at full size (B32, 32/8 heads, D128, S_max 32768, lengths U[1024, 32768]):
     # two sequences against the oracle, all of them against the prefill kernel's last row (an independent kernel).
     B, Hq, Hkv, S, D = 32, 32, 8, 32768, 128
     lens = I.seq_lens(4004, B, 1024, S)

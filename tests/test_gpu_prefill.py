@@ -34,7 +34,7 @@ def closed_form64(q, k, v, scale, causal):
 # ---- fp32 -----------------------------------------------------------------------------------------
 
 def test_f32_config1_against_reference_fixture(va):
-    # BASELINE config 1: B1, 8 q heads / 2 kv heads, D64, N256, scale 1/8, causal
+    # benchmark config 1: B1, 8 q heads / 2 kv heads, D64, N256, scale 1/8, causal
     z = np.load(os.path.join(GOLD, "config1.npz"), allow_pickle=False)
     B, Hq, Hkv, N, D, seed = [int(x) for x in z["meta"]]
     q, k, v = I.qkv(seed, B, Hq, Hkv, N, N, D)
@@ -172,7 +172,7 @@ def test_bf16_negative_scale_and_large_logits(va):
 
 
 def test_bf16_full_size_properties(va):
-    # BASELINE config 2 shape (B4, 32/8 heads, D128, N2048): properties that need no oracle at this size
+    # benchmark config 2 shape (B4, 32/8 heads, D128, N2048): properties that need no oracle at this size
     B, Hq, Hkv, N, D = 4, 32, 8, 2048, 128
     g = torch.Generator(device="cuda").manual_seed(7)
     q = (torch.randn(B, Hq, N, D, device=G.dev(), generator=g) * 0.5).to(torch.bfloat16)

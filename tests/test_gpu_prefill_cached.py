@@ -103,7 +103,7 @@ def test_f32_cache_planes(va):
 
 
 def test_chunked_equals_one_shot_at_config2_size(va):
-    # BASELINE config 2 shape, prefilled in two chunks of 1024 through the cache: same rows as the dense launch
+    # benchmark config 2 shape, prefilled in two chunks of 1024 through the cache: same rows as the dense launch
     B, Hq, Hkv, N, D = 4, 32, 8, 2048, 128
     g = torch.Generator(device="cuda").manual_seed(5)
     mk = lambda h: (torch.randn(B, h, N, D, device=G.dev(), generator=g) * 0.5).to(torch.bfloat16)
