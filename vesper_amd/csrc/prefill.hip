@@ -700,6 +700,9 @@ extern "C" int vsp_attn_prefill(const vsp_tensor* q, const vsp_tensor* k, const 
         return rc;
     if (lse && !lse->data) return VSP_ERR_NULL;
     if (T > INT32_MAX / 2 || L > INT32_MAX / 2) return VSP_ERR_ARG;
+    // the tile loads address one head's rows through a 32-bit buffer descriptor
+    if (k->stride[2] < 0 || v->stride[2] < 0) return VSP_ERR_STRIDE;
+    if (q->dtype == VSP_BF16 && (L * k->stride[2] * 2 > INT32_MAX || L * v->stride[2] * 2 > INT32_MAX)) return VSP_ERR_STRIDE;
 
     PrefillArgs a{};
     a.q = q->data;
