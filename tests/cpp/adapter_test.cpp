@@ -236,6 +236,23 @@ static void run_rope_generation(KVFormat fmt, DType qdt, double tol, const char*
     };
     step(0, T0);
     for (int64_t t = T0; t < N; ++t) step(t, t + 1);
+    // the same 12 tokens as a prompt processed in chunks of 8 + 4 (start_pos > 0 with T > 1)
+    {
+        CacheT cc(B, Hkv, S_max, D, Device::HIP, fmt);
+        int64_t bounds[3] = {0, 8, N};
+        for (int ci = 0; ci < 2; ++ci) {
+            const int64_t t0 = bounds[ci], t1 = bounds[ci + 1];
+            Tensor tq = to_dev(slice(q, Hq, t0, t1), {B, Hq, t1 - t0, D}, DType::Float32);
+            Tensor tk = to_dev(slice(k, Hkv, t0, t1), {B, Hkv, t1 - t0, D}, DType::Float32);
+            Tensor tv = to_dev(slice(v, Hkv, t0, t1), {B, Hkv, t1 - t0, D}, DType::Float32);
+            Tensor out = attn.forward_chunk(tq, tk, tv, &cc, t0, rope, qdt);
+            auto got = to_host(out), w = slice(want, Hq, t0, t1);
+            double err = max_abs_diff(got, w.data(), w.size());
+            if (!(err < tol)) std::printf("  chunk [%ld,%ld): max-abs %.3g\n", (long)t0, (long)t1, err);
+            CHECK(err < tol);
+        }
+        CHECK((int64_t)cc.current_seq_len() == N);
+    }
     // positions outside the table are refused, nothing is written
     nn::RopeTable small(4, D);
     Tensor tq = to_dev(slice(q, Hq, 0, 8), {B, Hq, 8, D}, DType::Float32);

@@ -266,6 +266,20 @@ public:
         q = q_out;
         return {view(false), view(true)};
     }
+    // Chunked prefill: attention of the LAST T tokens of the context (q [B,Hq,T,D], already appended to the cache)
+    // with K/V read in place from the planes.  The reference's scaled_dot_product_attention throws for a causal
+    // T != L (src/nn/functional.cpp:406-410); the rows returned are [len-T, len) of its full causal forward.
+    Tensor attend(const Tensor& q, bool is_causal = true) const {
+        Tensor out = empty(q.shape(), q.dtype());
+        vsp_tensor dq = q.desc(), dout = out.desc();
+        const size_t ws_bytes = vsp_attn_prefill_cached_workspace_bytes(&st_->c, 0);
+        std::shared_ptr<Storage> ws = ws_bytes ? std::make_shared<Storage>(ws_bytes) : nullptr;
+        const float scale = 1.0f / std::sqrt(static_cast<float>(q.shape()[3]));
+        throw_status(vsp_attn_prefill_cached(&dq, &st_->c, nullptr, nullptr, &dout, nullptr, scale, is_causal ? 1 : 0,
+                                             ws ? ws->data() : nullptr, ws_bytes, current_stream()));
+        hip_check(hipStreamSynchronize(current_stream()), "attend");  // the scratch buffer dies with this scope
+        return out;
+    }
     void reset() { throw_status(vsp_kv_cache_reset(&st_->c, current_stream())); }
     LenT current_seq_len() const { return (LenT)st_->c.len; }
     LenT get_max_seq_len() const { return (LenT)st_->c.S_max; }  // KVCache spelling
@@ -429,6 +443,16 @@ public:
         const int64_t T = q.shape()[2];
         auto kv = cache->rope_update(q, k, v, (decltype(cache->current_seq_len()))start_pos, rope, q_dtype);
         return functional::scaled_dot_product_attention(q, ops::repeat_kv(kv.first, num_rep_), ops::repeat_kv(kv.second, num_rep_), T > 1, 0.0);
+    }
+
+    // The same for a chunk that continues a longer context (start_pos > 0, T > 1), which the reference cannot
+    // run: RoPE + append, then the chunk attends over the cache planes in place.
+    template <typename CacheT>
+    Tensor forward_chunk(Tensor q, const Tensor& k, const Tensor& v, CacheT* cache, int64_t start_pos, const RopeTable& rope,
+                         DType q_dtype) const {
+        if (!cache) throw std::runtime_error("forward_chunk: a cache is required");
+        cache->rope_update(q, k, v, (decltype(cache->current_seq_len()))start_pos, rope, q_dtype);
+        return cache->attend(q, true);
     }
 
 private:
