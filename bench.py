@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on ONE MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|p4k|c3|c4|c5|r2] [--no-cpu] [--no-extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|p4k|c3|c4|c5|c4p|c2c|c3c|r2] [--no-cpu] [--no-extra]
 
 A "step" is one pass of the hot path over one batch of synthetic input that is already resident in
 HBM: one prefill launch (c2, p4k, c3) or one decode call = split-K kernel + combine kernel (c4, c5).
@@ -36,6 +36,8 @@ WORKLOADS = {
                name="BASELINE config 4: batched decode bf16 KV cache, B32, 32 q / 8 kv heads, D128, L~U[1024,32768]"),
     "c5": dict(kind="decode", fmt="q8_0", B=16, Hq=64, Hkv=8, D=128, S=65536, lens=None,
                name="BASELINE config 5: decode over Q8_0 KV cache, B16, 64 q / 8 kv heads, D128, L=65536"),
+    "c4p": dict(kind="decode", fmt="bf16", B=32, Hq=32, Hkv=8, D=128, S=32768, lens=(1024, 32768, 4004), page=256,
+                name="config 4 over a paged cache: pages of 256 tokens in a shuffled page table, otherwise as config 4"),
     "c2c": dict(kind="prefill_cached", fmt="bf16", B=4, Hq=32, Hkv=8, D=128, N=2048,
                 name="config 2 through the cache: causal GQA prefill bf16 reading K/V from the bf16 cache planes, "
                      "B4, 32 q / 8 kv heads, D128, N2048"),
@@ -108,12 +110,24 @@ class Runner:
             else:
                 lens = np.full(B, S, np.int32)
             self.lens = lens
-            self.cache = va.KVCache(B, Hkv, S, D, fmt=w["fmt"])
-            for b in range(B):  # fill through the append path, a batch row at a time (bounded fp32 temporaries)
-                kb = torch.randn(1, Hkv, S, D, device=dev, generator=g)
-                vb = torch.randn(1, Hkv, S, D, device=dev, generator=g)
-                self._append_row(b, kb, vb)
-                del kb, vb
+            if w.get("page"):
+                P = w["page"]
+                n_pages = B * (S // P)
+                self.cache = va.KVCache(B, Hkv, S, D, fmt=w["fmt"], paging=(P, n_pages))
+                perm = np.random.default_rng(7).permutation(n_pages).astype(np.int32).reshape(B, S // P)
+                self.cache.page_table.copy_(torch.from_numpy(perm))
+                for t0 in range(0, S, 2048):  # fill through the append path, 2048 tokens of every row at a time
+                    kb = torch.randn(B, Hkv, 2048, D, device=dev, generator=g).to(torch.bfloat16)
+                    vb = torch.randn(B, Hkv, 2048, D, device=dev, generator=g).to(torch.bfloat16)
+                    self.cache.update(kb, vb, t0, return_views=False)
+                    del kb, vb
+            else:
+                self.cache = va.KVCache(B, Hkv, S, D, fmt=w["fmt"])
+                for b in range(B):  # fill through the append path, a batch row at a time (bounded fp32 temporaries)
+                    kb = torch.randn(1, Hkv, S, D, device=dev, generator=g)
+                    vb = torch.randn(1, Hkv, S, D, device=dev, generator=g)
+                    self._append_row(b, kb, vb)
+                    del kb, vb
             self.cache.set_len(S)
             self.seq_lens = torch.from_numpy(lens).to(dev)
             self.q = torch.randn(B, Hq, 1, D, device=dev, generator=g).to(torch.bfloat16)
@@ -121,7 +135,7 @@ class Runner:
             self.scale = 1.0 / math.sqrt(D)
             self.work = decode_bytes(w, lens)
             self.unit, self.peak, self.bound = "GB/s", HBM_PEAK_GBS, "hbm"
-            self.kernel = "decode_bf16_kernel<128>" if w["fmt"] == "bf16" else "decode_q8_kernel<128>"
+            self.kernel = ("decode_bf16_kernel<128, %s>" if w["fmt"] == "bf16" else "decode_q8_kernel<128, %s>") % ("true" if w.get("page") else "false")
             self.max_len = int(lens.max())
 
     def _append_row(self, b, kb, vb):
@@ -319,7 +333,7 @@ def main():
 
     if not args.no_extra:
         others = {}
-        for key in ("c2", "p4k", "c3", "c4", "c5", "c2c", "c3c", "r2"):
+        for key in ("c2", "p4k", "c3", "c4", "c5", "c4p", "c2c", "c3c", "r2"):
             if key == args.workload:
                 continue
             r = Runner(key, torch, va)

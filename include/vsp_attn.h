@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define VSP_ATTN_ABI_VERSION 1
+#define VSP_ATTN_ABI_VERSION 2
 
 typedef enum {
     VSP_OK = 0,
@@ -98,6 +98,15 @@ typedef struct {
  *               v:       int8 [B][Hkv][S_pad/16][D][16]   (token-blocked by 16)
  *               v_scale: fp16 [B][Hkv][S_pad/16][D/32][16]
  * D must be 64 or 128 for BF16/Q8_0.  Plane sizes: vsp_kv_plane_bytes().
+ *
+ * Paged variant (page_table != NULL; no counterpart in the reference, whose caches are one allocation per
+ * batch): the planes hold n_pages pages of page_tokens tokens, each page laid out exactly like one batch
+ * row above with S_pad = page_tokens -- [n_pages][Hkv][page_tokens][D] and so on -- and sequence b's tokens
+ * [i*page_tokens, (i+1)*page_tokens) live in page page_table[b*pages_per_seq + i] (device int32, values in
+ * [0, n_pages), owned and kept consistent by the caller).  BF16 and Q8_0 only; page_tokens a multiple of 64;
+ * S_max == pages_per_seq * page_tokens; plane sizes: vsp_kv_plane_bytes(format, n_pages, Hkv, page_tokens, D, plane).
+ * Append, RoPE-append, read and decode accept paged caches; vsp_attn_prefill_cached does not yet
+ * (VSP_ERR_UNSUPPORTED).
  */
 typedef enum { VSP_KV_F32 = 0, VSP_KV_BF16 = 1, VSP_KV_Q8_0 = 2 } vsp_kv_format;
 typedef enum { VSP_KV_PLANE_K = 0, VSP_KV_PLANE_V = 1, VSP_KV_PLANE_K_SCALE = 2, VSP_KV_PLANE_V_SCALE = 3 } vsp_kv_plane;
@@ -110,6 +119,9 @@ typedef struct {
     void* k_scale; /* Q8_0 only, else NULL */
     void* v_scale; /* Q8_0 only, else NULL */
     int32_t len;   /* the reference's current_len_ (host side, maintained by vsp_kv_append) */
+    /* paged variant; all zero / NULL for a contiguous cache */
+    const int32_t* page_table; /* device int32 [B][pages_per_seq] */
+    int32_t page_tokens, pages_per_seq, n_pages;
 } vsp_kv_cache;
 
 /* Bytes the caller must allocate for one plane (0 for planes the format lacks). */

@@ -27,7 +27,7 @@ def test_library_exports_every_declared_symbol(ffi):
     assert declared == set(ffi.SYMBOLS), declared ^ set(ffi.SYMBOLS)
     for name in declared:
         assert hasattr(ffi.lib, name), name
-    assert ffi.lib.vsp_attn_abi_version() == 1
+    assert ffi.lib.vsp_attn_abi_version() == 2
 
 
 def test_status_strings_are_the_reference_messages(ffi):

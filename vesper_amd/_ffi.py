@@ -28,7 +28,9 @@ class VspTensor(C.Structure):
 class VspKVCache(C.Structure):
     _fields_ = [("format", C.c_int32), ("B", C.c_int32), ("Hkv", C.c_int32), ("S_max", C.c_int32), ("D", C.c_int32),
                 ("k", C.c_void_p), ("v", C.c_void_p), ("k_scale", C.c_void_p), ("v_scale", C.c_void_p),
-                ("len", C.c_int32)]
+                ("len", C.c_int32),
+                ("page_table", C.c_void_p), ("page_tokens", C.c_int32), ("pages_per_seq", C.c_int32),
+                ("n_pages", C.c_int32)]
 
 
 # every symbol include/vsp_attn.h declares: name -> (restype, argtypes)

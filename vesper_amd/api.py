@@ -77,15 +77,27 @@ class KVCache:
 
     _FMT = {"f32": _ffi.KV_F32, "bf16": _ffi.KV_BF16, "q8_0": _ffi.KV_Q8_0}
 
-    def __init__(self, batch_size, num_heads, max_seq_len, head_dim, device="cuda", fmt="f32"):
+    def __init__(self, batch_size, num_heads, max_seq_len, head_dim, device="cuda", fmt="f32", paging=None):
+        """paging=(page_tokens, n_pages): the planes hold n_pages pages of page_tokens tokens and `page_table`
+        (device int32 [batch, max_seq_len / page_tokens], set by the caller) says which page holds which tokens."""
         self.fmt = fmt
         self.device = torch.device(device)
         c = VspKVCache()
         c.format = self._FMT[fmt]
         c.B, c.Hkv, c.S_max, c.D = batch_size, num_heads, max_seq_len, head_dim
+        self.page_table = None
+        if paging is not None:
+            page_tokens, n_pages = paging
+            c.page_tokens, c.n_pages = int(page_tokens), int(n_pages)
+            c.pages_per_seq = max_seq_len // max(int(page_tokens), 1)
+            self.page_table = torch.zeros((batch_size, max(c.pages_per_seq, 1)), dtype=torch.int32, device=self.device)
+            c.page_table = self.page_table.data_ptr()
         self._planes = []
         for plane in range(4):
-            n = lib.vsp_kv_plane_bytes(c.format, c.B, c.Hkv, c.S_max, c.D, plane)
+            if paging is not None:
+                n = lib.vsp_kv_plane_bytes(c.format, c.n_pages, c.Hkv, c.page_tokens, c.D, plane)
+            else:
+                n = lib.vsp_kv_plane_bytes(c.format, c.B, c.Hkv, c.S_max, c.D, plane)
             self._planes.append(torch.empty(n, dtype=torch.uint8, device=self.device) if n else None)
         c.k, c.v, c.k_scale, c.v_scale = [p.data_ptr() if p is not None else None for p in self._planes]
         c.len = 0
@@ -185,8 +197,8 @@ class RaggedKVCache(KVCache):
     one host-side length for the batch).  Every step is asynchronous: nothing is read back to the host.
     `upper` is a host-side upper bound of the longest row, used only to size work (grids, workspaces)."""
 
-    def __init__(self, batch_size, num_heads, max_seq_len, head_dim, device="cuda", fmt="bf16"):
-        super().__init__(batch_size, num_heads, max_seq_len, head_dim, device=device, fmt=fmt)
+    def __init__(self, batch_size, num_heads, max_seq_len, head_dim, device="cuda", fmt="bf16", paging=None):
+        super().__init__(batch_size, num_heads, max_seq_len, head_dim, device=device, fmt=fmt, paging=paging)
         self.seq_lens = torch.zeros(batch_size, dtype=torch.int32, device=self.device)
         self.upper = 0
 

@@ -44,7 +44,26 @@ struct DecodeArgs {
     float scale_log2;  // scale * log2(e)
     float* ws_o;       // [B][Hq][max_splits][D]
     float* ws_ml;      // [B][Hq][max_splits][2]  (m in log2 domain, l)
+    // paged cache: sequence b's 64-key group starting at token t lives in page page_table[b * pages_per_seq +
+    // t / page_tokens] (page_tokens is a multiple of 64, so a group never straddles two pages); S is then the
+    // page size.  nullptr for a contiguous cache.
+    const int32_t* page_table;
+    int32_t page_tokens, pages_per_seq;
 };
+
+// Index of the [S][D] slab that holds the 64-key group at token `kbase` of (sequence b, kv head), and the
+// group's first token inside that slab.
+template <bool PAGED>
+__device__ inline int64_t group_slab(const DecodeArgs& a, int b, int kvh, int kbase, int& local) {
+    if constexpr (PAGED) {
+        const int pg = kbase / a.page_tokens;
+        local = kbase - pg * a.page_tokens;
+        return (int64_t)a.page_table[(int64_t)b * a.pages_per_seq + pg] * a.Hkv + kvh;
+    } else {
+        local = kbase;
+        return (int64_t)b * a.Hkv + kvh;
+    }
+}
 
 __device__ inline float wave_max_over_groups(float x) {
     x = fmaxf(x, __shfl_xor(x, 16));
@@ -112,7 +131,7 @@ __device__ inline bool locate_work(const DecodeArgs& a, int item, int lane, int&
 // ---------------------------------------------------------------------------------------------
 // bf16 cache
 // ---------------------------------------------------------------------------------------------
-template <int D>
+template <int D, bool PAGED>
 __global__ void __launch_bounds__(256, 2) decode_bf16_kernel(DecodeArgs a) {
     constexpr int KS = D / 32;   // MFMA k-steps over the head dim
     constexpr int DB = D / 16;   // 16-row tiles of O^T
@@ -136,8 +155,6 @@ __global__ void __launch_bounds__(256, 2) decode_bf16_kernel(DecodeArgs a) {
             qf[ks] = __builtin_bit_cast(bf16x8_t, w);
         }
     }
-    const uint16_t* Kp = (const uint16_t*)a.k + ((int64_t)b * a.Hkv + kvh) * a.S * D;
-    const uint16_t* Vp = (const uint16_t*)a.v + ((int64_t)b * a.Hkv + kvh) * a.S * D;
     const int krow = 16 * (c >> 2) + (c & 3);  // this lane's A-operand row: key offset before + 4*jj
 
     f32x4_t acc[DB];
@@ -152,15 +169,19 @@ __global__ void __launch_bounds__(256, 2) decode_bf16_kernel(DecodeArgs a) {
     uint4 kf[4][KS];
     uint4 vf[DB][2];
     auto load_k = [&](int kbase) {
+        int local;
+        const uint16_t* Kp = (const uint16_t*)a.k + group_slab<PAGED>(a, b, kvh, kbase, local) * a.S * D;
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj) {
-            const uint16_t* kr = Kp + (int64_t)(kbase + krow + 4 * jj) * D + 8 * g;
+            const uint16_t* kr = Kp + (int64_t)(local + krow + 4 * jj) * D + 8 * g;
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) kf[jj][ks] = *(const uint4*)(kr + 32 * ks);
         }
     };
     auto load_v = [&](int kbase) {
-        const uint16_t* vb = Vp + ((int64_t)(kbase / kVBlkBf16 + 2 * g) * D + c) * kVBlkBf16;
+        int local;
+        const uint16_t* Vp = (const uint16_t*)a.v + group_slab<PAGED>(a, b, kvh, kbase, local) * a.S * D;
+        const uint16_t* vb = Vp + ((int64_t)(local / kVBlkBf16 + 2 * g) * D + c) * kVBlkBf16;
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -279,7 +300,7 @@ __device__ inline void i8x4_to_f16x4(uint32_t w, f16x2_t& lo, f16x2_t& hi) {
 }
 __device__ inline uint32_t f16x2_bits(f16x2_t v) { return __builtin_bit_cast(uint32_t, v); }
 
-template <int D>
+template <int D, bool PAGED>
 __global__ void __launch_bounds__(256, 2) decode_q8_kernel(DecodeArgs a) {
     constexpr int KS = D / 32;
     constexpr int DB = D / 16;
@@ -314,11 +335,6 @@ __global__ void __launch_bounds__(256, 2) decode_q8_kernel(DecodeArgs a) {
             }
         }
     }
-    const int64_t head = (int64_t)b * a.Hkv + kvh;
-    const int8_t* Kp = (const int8_t*)a.k + head * a.S * D;
-    const int8_t* Vp = (const int8_t*)a.v + head * a.S * D;
-    const uint16_t* KSp = (const uint16_t*)a.k_scale + head * a.S * NQ;
-    const uint16_t* VSp = (const uint16_t*)a.v_scale + head * a.S * NQ;
     const int krow = 16 * (c >> 2) + (c & 3);
 
     f32x4_t acc[DB];
@@ -332,9 +348,13 @@ __global__ void __launch_bounds__(256, 2) decode_q8_kernel(DecodeArgs a) {
     uint4 vq[DB];
     uint4 vsc[NQ][2];
     auto load_k = [&](int kbase) {
+        int local;
+        const int64_t head = group_slab<PAGED>(a, b, kvh, kbase, local);
+        const int8_t* Kp = (const int8_t*)a.k + head * a.S * D;
+        const uint16_t* KSp = (const uint16_t*)a.k_scale + head * a.S * NQ;
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj) {
-            const int64_t key = kbase + krow + 4 * jj;
+            const int64_t key = local + krow + 4 * jj;
 #pragma unroll
             for (int h = 0; h < NH; ++h) {
                 kq[jj][h] = *(const uint4*)(Kp + key * D + 64 * h + 16 * g);
@@ -343,7 +363,11 @@ __global__ void __launch_bounds__(256, 2) decode_q8_kernel(DecodeArgs a) {
         }
     };
     auto load_v = [&](int kbase) {
-        const int64_t blk = kbase / kVBlkQ8 + g;
+        int local;
+        const int64_t head = group_slab<PAGED>(a, b, kvh, kbase, local);
+        const int8_t* Vp = (const int8_t*)a.v + head * a.S * D;
+        const uint16_t* VSp = (const uint16_t*)a.v_scale + head * a.S * NQ;
+        const int64_t blk = local / kVBlkQ8 + g;
 #pragma unroll
         for (int db = 0; db < DB; ++db) vq[db] = *(const uint4*)(Vp + (blk * D + 16 * db + c) * kVBlkQ8);
 #pragma unroll
@@ -695,8 +719,11 @@ int vsp_attn_decode(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_
     a.Hq = (int)Hq;
     a.Hkv = cache->Hkv;
     a.n_rep = n_rep;
-    a.S = kv_s_pad(cache->format, cache->S_max);
+    a.S = cache->page_table ? cache->page_tokens : kv_s_pad(cache->format, cache->S_max);
     a.S_max = cache->S_max;
+    a.page_table = cache->page_table;
+    a.page_tokens = cache->page_tokens;
+    a.pages_per_seq = cache->pages_per_seq;
     a.chunk = chunk;
     a.max_splits = max_splits;
     a.scale_log2 = scale * kLog2e;
@@ -706,12 +733,22 @@ int vsp_attn_decode(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_
     if (max_len > 0) {
         if (cache->format == VSP_KV_BF16) {
             dim3 grid((unsigned)(max_splits * B), cache->Hkv);
-            if (D == 128) hipLaunchKernelGGL(decode_bf16_kernel<128>, grid, dim3(256), 0, st, a);
-            else hipLaunchKernelGGL(decode_bf16_kernel<64>, grid, dim3(256), 0, st, a);
+            if (cache->page_table) {
+                if (D == 128) hipLaunchKernelGGL((decode_bf16_kernel<128, true>), grid, dim3(256), 0, st, a);
+                else hipLaunchKernelGGL((decode_bf16_kernel<64, true>), grid, dim3(256), 0, st, a);
+            } else {
+                if (D == 128) hipLaunchKernelGGL((decode_bf16_kernel<128, false>), grid, dim3(256), 0, st, a);
+                else hipLaunchKernelGGL((decode_bf16_kernel<64, false>), grid, dim3(256), 0, st, a);
+            }
         } else if (cache->format == VSP_KV_Q8_0) {
             dim3 grid((unsigned)(max_splits * B), cache->Hkv);
-            if (D == 128) hipLaunchKernelGGL(decode_q8_kernel<128>, grid, dim3(256), 0, st, a);
-            else hipLaunchKernelGGL(decode_q8_kernel<64>, grid, dim3(256), 0, st, a);
+            if (cache->page_table) {
+                if (D == 128) hipLaunchKernelGGL((decode_q8_kernel<128, true>), grid, dim3(256), 0, st, a);
+                else hipLaunchKernelGGL((decode_q8_kernel<64, true>), grid, dim3(256), 0, st, a);
+            } else {
+                if (D == 128) hipLaunchKernelGGL((decode_q8_kernel<128, false>), grid, dim3(256), 0, st, a);
+                else hipLaunchKernelGGL((decode_q8_kernel<64, false>), grid, dim3(256), 0, st, a);
+            }
         } else {
             dim3 grid((unsigned)(max_splits * B), (unsigned)Hq);
             const size_t smem = (256 + chunk + 256) * sizeof(float);

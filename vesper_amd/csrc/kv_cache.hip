@@ -55,6 +55,10 @@ struct AppendArgs {
     int64_t Hq, T;
     int64_t kv_items;      // threads of the K/V part; the Q part follows
     int32_t q_out_bf16;
+    // paged cache (kv_locate): table == nullptr for a contiguous one
+    const int32_t* page_table;
+    int32_t page_tokens, pages_per_seq;
+    int64_t S_logical;  // per-sequence token capacity (the bound for device-side positions)
 };
 
 template <typename SrcT>
@@ -112,7 +116,8 @@ __device__ inline void rope_q_item(const AppendArgs& a, int64_t i) {
 // index decomposed by the slot shape on the destination side and by the source shape on the
 // source side.
 struct RowMap {
-    int64_t b, h, s;     // destination coordinates
+    int64_t b, h, s;     // destination coordinates in the planes (page and token within it for a paged cache)
+    int64_t pos;         // the token's position in its sequence (what RoPE rotates by); < 0: drop the token
     int64_t src_off_k, src_off_v;
 };
 __device__ inline RowMap map_row(const AppendArgs& a, int64_t r) {
@@ -122,6 +127,8 @@ __device__ inline RowMap map_row(const AppendArgs& a, int64_t r) {
     m.b = bh / a.H;
     int64_t start = a.start_dev ? (int64_t)a.start_dev[m.b] : a.slot_start;
     m.s = start + t;
+    m.pos = (m.s >= 0 && m.s < a.S_logical) ? m.s : -1;  // a device-side position outside the cache
+    if (m.pos >= 0) kv_locate(a.page_table, a.page_tokens, a.pages_per_seq, m.b, m.s);
     int64_t st = r % a.nT, sbh = r / a.nT;
     int64_t sh = sbh % a.nH, sb = sbh / a.nH;
     m.src_off_k = sb * a.sk[0] + sh * a.sk[1] + st * a.sk[2];
@@ -144,7 +151,7 @@ __global__ void __launch_bounds__(256) append_f32_kernel(AppendArgs a) {
     if (i >= a.rows * per_row) return;
     const int64_t r = i / per_row, d0 = (i % per_row) * 4;
     const RowMap m = map_row(a, r);
-    if (m.s < 0 || m.s >= a.S) return;  // a device-side position outside the planes: drop the token, never write out of bounds
+    if (m.pos < 0) return;  // never write out of bounds
     const SrcT* pk = (const SrcT*)a.src_k + m.src_off_k + d0;
     const SrcT* pv = (const SrcT*)a.src_v + m.src_off_v + d0;
     float* dk = (float*)a.k + kv_off_rowmajor(a.H, a.S, a.D, m.b, m.h, m.s, d0);
@@ -152,7 +159,7 @@ __global__ void __launch_bounds__(256) append_f32_kernel(AppendArgs a) {
     float xk[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) xk[j] = load_src<SrcT>(pk + j);
-    if constexpr (ROPE) rope_rotate<4>(xk, d0, m.s, a);
+    if constexpr (ROPE) rope_rotate<4>(xk, d0, m.pos, a);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         dk[j] = xk[j];
@@ -175,7 +182,7 @@ __global__ void __launch_bounds__(256) append_bf16_kernel(AppendArgs a) {
     if (i >= a.rows * per_row) return;
     const int64_t r = i / per_row, d0 = (i % per_row) * 8;
     const RowMap m = map_row(a, r);
-    if (m.s < 0 || m.s >= a.S) return;  // a device-side position outside the planes: drop the token, never write out of bounds
+    if (m.pos < 0) return;  // never write out of bounds
     const SrcT* pk = (const SrcT*)a.src_k + m.src_off_k + d0;
     const SrcT* pv = (const SrcT*)a.src_v + m.src_off_v + d0;
     uint16_t kb[8], vb[8];
@@ -183,7 +190,7 @@ __global__ void __launch_bounds__(256) append_bf16_kernel(AppendArgs a) {
         float xk[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) xk[j] = load_src<SrcT>(pk + j);
-        rope_rotate<8>(xk, d0, m.s, a);
+        rope_rotate<8>(xk, d0, m.pos, a);
 #pragma unroll
         for (int j = 0; j < 8; ++j) kb[j] = f32_to_bf16_bits(xk[j]);
     }
@@ -242,7 +249,7 @@ __global__ void __launch_bounds__(128) append_q8_kernel(AppendArgs a) {
     if (i >= a.rows * per_row) return;
     const int64_t r = i / per_row, blk = i % per_row, d0 = blk * kQBlock;
     const RowMap m = map_row(a, r);
-    if (m.s < 0 || m.s >= a.S) return;  // a device-side position outside the planes: drop the token, never write out of bounds
+    if (m.pos < 0) return;  // never write out of bounds
     const SrcT* pk = (const SrcT*)a.src_k + m.src_off_k + d0;
     const SrcT* pv = (const SrcT*)a.src_v + m.src_off_v + d0;
     float x[kQBlock];
@@ -251,7 +258,7 @@ __global__ void __launch_bounds__(128) append_q8_kernel(AppendArgs a) {
     // K: row-major int8, scales [s][blk]
 #pragma unroll
     for (int j = 0; j < kQBlock; ++j) x[j] = load_src<SrcT>(pk + j);
-    if constexpr (ROPE) rope_rotate<kQBlock>(x, d0, m.s, a);
+    if constexpr (ROPE) rope_rotate<kQBlock>(x, d0, m.pos, a);
     quantize_block(x, q, &sc);
     {
         uint32_t w[8];
@@ -288,6 +295,8 @@ struct ReadArgs {
     void* out_v;
     int64_t ok[3], ov[3];  // output strides of dims 0..2 (elements)
     int format;
+    const int32_t* page_table;
+    int32_t page_tokens, pages_per_seq;
 };
 
 template <typename DstT>
@@ -311,25 +320,27 @@ __global__ void __launch_bounds__(256) read_kernel(ReadArgs a) {
     const int64_t t = r % a.count;
     r /= a.count;
     const int64_t h = r % a.H, b = r / a.H;
-    const int64_t s = a.start + t;
+    const int64_t s_seq = a.start + t;
+    int64_t pb = b, s = s_seq;  // plane coordinates
+    kv_locate(a.page_table, a.page_tokens, a.pages_per_seq, pb, s);
     float fk, fv;
     uint16_t bk = 0, bv = 0;
     bool bits = false;
     if (a.format == VSP_KV_F32) {
-        fk = ((const float*)a.k)[kv_off_rowmajor(a.H, a.S, a.D, b, h, s, d)];
-        fv = ((const float*)a.v)[kv_off_rowmajor(a.H, a.S, a.D, b, h, s, d)];
+        fk = ((const float*)a.k)[kv_off_rowmajor(a.H, a.S, a.D, pb, h, s, d)];
+        fv = ((const float*)a.v)[kv_off_rowmajor(a.H, a.S, a.D, pb, h, s, d)];
     } else if (a.format == VSP_KV_BF16) {
-        bk = ((const uint16_t*)a.k)[kv_off_rowmajor(a.H, a.S, a.D, b, h, s, d)];
-        bv = ((const uint16_t*)a.v)[kv_off_vblocked(a.H, a.S, a.D, kVBlkBf16, b, h, s, d)];
+        bk = ((const uint16_t*)a.k)[kv_off_rowmajor(a.H, a.S, a.D, pb, h, s, d)];
+        bv = ((const uint16_t*)a.v)[kv_off_vblocked(a.H, a.S, a.D, kVBlkBf16, pb, h, s, d)];
         fk = bf16_bits_to_f32(bk);
         fv = bf16_bits_to_f32(bv);
         bits = true;
     } else {
         const int64_t blk = d / kQBlock;
-        const float dk = f16_bits_to_f32_dev(((const uint16_t*)a.k_scale)[kv_off_kscale(a.H, a.S, a.D, b, h, s, blk)]);
-        const float dv = f16_bits_to_f32_dev(((const uint16_t*)a.v_scale)[kv_off_vscale(a.H, a.S, a.D, b, h, s, blk)]);
-        fk = __fmul_rn((float)((const int8_t*)a.k)[kv_off_rowmajor(a.H, a.S, a.D, b, h, s, d)], dk);
-        fv = __fmul_rn((float)((const int8_t*)a.v)[kv_off_vblocked(a.H, a.S, a.D, kVBlkQ8, b, h, s, d)], dv);
+        const float dk = f16_bits_to_f32_dev(((const uint16_t*)a.k_scale)[kv_off_kscale(a.H, a.S, a.D, pb, h, s, blk)]);
+        const float dv = f16_bits_to_f32_dev(((const uint16_t*)a.v_scale)[kv_off_vscale(a.H, a.S, a.D, pb, h, s, blk)]);
+        fk = __fmul_rn((float)((const int8_t*)a.k)[kv_off_rowmajor(a.H, a.S, a.D, pb, h, s, d)], dk);
+        fv = __fmul_rn((float)((const int8_t*)a.v)[kv_off_vblocked(a.H, a.S, a.D, kVBlkQ8, pb, h, s, d)], dv);
     }
     if (a.out_k) store_dst<DstT>((DstT*)a.out_k + b * a.ok[0] + h * a.ok[1] + t * a.ok[2] + d, fk, bk, bits);
     if (a.out_v) store_dst<DstT>((DstT*)a.out_v + b * a.ov[0] + h * a.ov[1] + t * a.ov[2] + d, fv, bv, bits);
@@ -338,14 +349,17 @@ __global__ void __launch_bounds__(256) read_kernel(ReadArgs a) {
 __global__ void __launch_bounds__(256) read_q8_raw_kernel(const int8_t* __restrict__ qs, const uint16_t* __restrict__ sc,
                                                           int plane, int64_t B, int64_t H, int64_t S, int64_t D,
                                                           int64_t start, int64_t count, int8_t* __restrict__ qs_out,
-                                                          uint16_t* __restrict__ sc_out) {
+                                                          uint16_t* __restrict__ sc_out, const int32_t* __restrict__ page_table,
+                                                          int32_t page_tokens, int32_t pages_per_seq) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= B * H * count * D) return;
     const int64_t d = i % D;
     int64_t r = i / D;
     const int64_t t = r % count;
     r /= count;
-    const int64_t h = r % H, b = r / H, s = start + t;
+    const int64_t h = r % H;
+    int64_t b = r / H, s = start + t;
+    kv_locate(page_table, page_tokens, pages_per_seq, b, s);
     if (plane == VSP_KV_PLANE_K) {
         qs_out[i] = qs[kv_off_rowmajor(H, S, D, b, h, s, d)];
         if (d % kQBlock == 0) sc_out[i / kQBlock] = sc[kv_off_kscale(H, S, D, b, h, s, d / kQBlock)];
@@ -380,12 +394,22 @@ int check_cache(const vsp_kv_cache* c) {
     } else if (c->D != 64 && c->D != 128) {
         return VSP_ERR_UNSUPPORTED;
     }
+    if (c->page_table) {
+        if (c->format == VSP_KV_F32) return VSP_ERR_UNSUPPORTED;
+        if (c->page_tokens <= 0 || c->page_tokens % kTokPad != 0 || c->pages_per_seq <= 0 || c->n_pages <= 0) return VSP_ERR_ARG;
+        if ((int64_t)c->pages_per_seq * c->page_tokens != c->S_max) return VSP_ERR_ARG;
+    } else if (c->page_tokens != 0 || c->pages_per_seq != 0 || c->n_pages != 0) {
+        return VSP_ERR_ARG;  // paging fields without a table
+    }
     return VSP_OK;
 }
 
 }  // namespace
 
 int check_kv_cache(const vsp_kv_cache* c) { return check_cache(c); }
+// Physical batch and token capacity of the planes: pages for a paged cache.
+int64_t kv_phys_batch(const vsp_kv_cache* c) { return c->page_table ? c->n_pages : c->B; }
+int64_t kv_phys_tokens(const vsp_kv_cache* c) { return c->page_table ? c->page_tokens : kv_s_pad(c->format, c->S_max); }
 
 }  // namespace vsp
 
@@ -398,7 +422,9 @@ int vsp_kv_cache_reset(vsp_kv_cache* cache, void* stream) {
     if (rc != VSP_OK) return rc;
     hipStream_t st = (hipStream_t)stream;
     for (int plane = 0; plane < 4; ++plane) {
-        size_t bytes = kv_plane_bytes(cache->format, cache->B, cache->Hkv, cache->S_max, cache->D, plane);
+        size_t bytes = cache->page_table
+                           ? kv_plane_bytes(cache->format, cache->n_pages, cache->Hkv, cache->page_tokens, cache->D, plane)
+                           : kv_plane_bytes(cache->format, cache->B, cache->Hkv, cache->S_max, cache->D, plane);
         void* p = plane == 0 ? cache->k : plane == 1 ? cache->v : plane == 2 ? cache->k_scale : cache->v_scale;
         rc = zero_plane(p, bytes, st);
         if (rc != VSP_OK) return rc;
@@ -481,8 +507,12 @@ static int append_impl(vsp_kv_cache* cache, const vsp_tensor* new_k, const vsp_t
         a.v_scale = cache->v_scale;
         a.B = cache->B;
         a.H = cache->Hkv;
-        a.S = kv_s_pad(cache->format, cache->S_max);
+        a.S = kv_phys_tokens(cache);
         a.D = cache->D;
+        a.page_table = cache->page_table;
+        a.page_tokens = cache->page_tokens;
+        a.pages_per_seq = cache->pages_per_seq;
+        a.S_logical = cache->S_max;
         a.slot_start = slot_start;
         a.slot_len = slot_len;
         a.start_dev = start_pos_dev;
@@ -585,8 +615,11 @@ int vsp_kv_read(const vsp_kv_cache* cache, int64_t start, int64_t count, vsp_ten
     a.v_scale = cache->v_scale;
     a.B = cache->B;
     a.H = cache->Hkv;
-    a.S = kv_s_pad(cache->format, cache->S_max);
+    a.S = kv_phys_tokens(cache);
     a.D = cache->D;
+    a.page_table = cache->page_table;
+    a.page_tokens = cache->page_tokens;
+    a.pages_per_seq = cache->pages_per_seq;
     a.start = start;
     a.count = count;
     a.out_k = k_out ? k_out->data : nullptr;
@@ -616,8 +649,8 @@ int vsp_kv_read_q8_0(const vsp_kv_cache* cache, int32_t plane, int64_t start, in
     hipLaunchKernelGGL(read_q8_raw_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, (hipStream_t)stream,
                        (const int8_t*)(isk ? cache->k : cache->v),
                        (const uint16_t*)(isk ? cache->k_scale : cache->v_scale), plane, (int64_t)cache->B,
-                       (int64_t)cache->Hkv, kv_s_pad(cache->format, cache->S_max), (int64_t)cache->D, start, count,
-                       qs_out, scale_out);
+                       (int64_t)cache->Hkv, kv_phys_tokens(cache), (int64_t)cache->D, start, count, qs_out, scale_out,
+                       cache->page_table, cache->page_tokens, cache->pages_per_seq);
     return check_launch();
 }
 

@@ -21,6 +21,17 @@ __host__ __device__ inline int64_t kv_s_pad(int format, int64_t S_max) {
     return format == VSP_KV_F32 ? S_max : (S_max + kTokPad - 1) / kTokPad * kTokPad;
 }
 
+// Paged caches: logical (sequence b, token s) -> (page, token within the page).  The planes of a paged cache are
+// laid out like a contiguous cache with batch = n_pages and token capacity = page_tokens, so after this
+// translation every offset function below applies unchanged.  table == nullptr: contiguous, identity.
+__host__ __device__ inline void kv_locate(const int32_t* table, int32_t page_tokens, int32_t pages_per_seq, int64_t& b, int64_t& s) {
+    if (table) {
+        const int64_t pg = s / page_tokens;
+        s -= pg * page_tokens;
+        b = table[b * pages_per_seq + pg];
+    }
+}
+
 // ---- element offsets (in elements of the plane's type) ----
 // row-major [B][H][S][D]: the reference layout (K of every format, V of F32)
 __host__ __device__ inline int64_t kv_off_rowmajor(int64_t H, int64_t S, int64_t D, int64_t b, int64_t h, int64_t s,

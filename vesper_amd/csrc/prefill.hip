@@ -586,6 +586,7 @@ extern "C" int vsp_attn_prefill_cached(const vsp_tensor* q, const vsp_kv_cache* 
     if (!q || !out) return VSP_ERR_NULL;
     int rc = check_kv_cache(cache);
     if (rc != VSP_OK) return rc;
+    if (cache->page_table) return VSP_ERR_UNSUPPORTED;  // paged caches: append, read and decode only
     if (q->ndim != 4 || out->ndim != 4) return VSP_ERR_NDIM;
     const int64_t B = q->shape[0], Hq = q->shape[1], T = q->shape[2], D = q->shape[3];
     const int64_t Hkv = cache->Hkv;
