@@ -105,8 +105,7 @@ typedef struct {
  * [i*page_tokens, (i+1)*page_tokens) live in page page_table[b*pages_per_seq + i] (device int32, values in
  * [0, n_pages), owned and kept consistent by the caller).  BF16 and Q8_0 only; page_tokens a multiple of 64;
  * S_max == pages_per_seq * page_tokens; plane sizes: vsp_kv_plane_bytes(format, n_pages, Hkv, page_tokens, D, plane).
- * Append, RoPE-append, read and decode accept paged caches; vsp_attn_prefill_cached does not yet
- * (VSP_ERR_UNSUPPORTED).
+ * Every entry point that takes a cache accepts a paged one.
  */
 typedef enum { VSP_KV_F32 = 0, VSP_KV_BF16 = 1, VSP_KV_Q8_0 = 2 } vsp_kv_format;
 typedef enum { VSP_KV_PLANE_K = 0, VSP_KV_PLANE_V = 1, VSP_KV_PLANE_K_SCALE = 2, VSP_KV_PLANE_V_SCALE = 3 } vsp_kv_plane;

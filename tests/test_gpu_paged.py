@@ -88,7 +88,31 @@ def test_validation(va):
         va.KVCache(1, 2, 100, 64, fmt="bf16", paging=(64, 4))
     c = va.RaggedKVCache(1, 2, 128, 64, fmt="bf16", paging=(64, 4))
     c.page_table.copy_(torch.tensor([[1, 3]], dtype=torch.int32))
-    z = torch.zeros(1, 2, 70, 64, device=G.dev(), dtype=torch.bfloat16)
-    c.append(z, z)
-    with pytest.raises(va.VspError):   # chunked prefill over pages is not implemented
-        c.prefill(torch.zeros(1, 4, 8, 64, device=G.dev(), dtype=torch.bfloat16), seq_lens=c.seq_lens)
+
+
+@pytest.mark.parametrize("fmt", ["bf16", "q8_0"])
+def test_chunked_prefill_over_pages_matches_the_contiguous_cache(va, fmt):
+    B, Hq, Hkv, D, S_max, P = 3, 8, 2, 128, 640, 128
+    flat, paged = _pair(va, fmt, B, Hkv, S_max, D, P, seed=11)
+    lens = [500, 130, 333]
+    T = 100
+    q, k, v = [O.bf16_round(x) for x in I.qkv(6300, B, Hq, Hkv, 500, 500, D, scale=0.5)]
+    n0 = torch.tensor([l - T for l in lens], dtype=torch.int32, device=G.dev())
+    outs = []
+    for c in (flat, paged):
+        c.append(G.to_bf16_dev(k[:, :, :400]), G.to_bf16_dev(v[:, :, :400]), n_new=n0)      # the context
+        chunk_k = np.stack([k[b, :, lens[b] - T:lens[b]] for b in range(B)])
+        chunk_v = np.stack([v[b, :, lens[b] - T:lens[b]] for b in range(B)])
+        c.append(G.to_bf16_dev(chunk_k), G.to_bf16_dev(chunk_v))                            # the chunk, crossing pages
+        chunk_q = np.stack([q[b, :, lens[b] - T:lens[b]] for b in range(B)])
+        outs.append(c.prefill_chunk(G.to_bf16_dev(chunk_q)))
+    assert paged.seq_lens.cpu().tolist() == lens
+    assert torch.equal(outs[0], outs[1])
+    # and against the oracle, on what the cache holds
+    kk, vv = (k, v) if fmt == "bf16" else (O.q8_0_dequantize(*O.q8_0_quantize(k)), O.q8_0_dequantize(*O.q8_0_quantize(v)))
+    got = G.bf16_to_np(outs[1])
+    for b in range(B):
+        L = lens[b]
+        want = O.flash_attention(q[b:b + 1, :, :L], O.repeat_kv(kk[b:b + 1, :, :L], 4), O.repeat_kv(vv[b:b + 1, :, :L], 4),
+                                 float(np.float32(1.0 / np.sqrt(D))), True)[:, :, L - T:]
+        G.assert_bf16_close(got[b:b + 1], want, f"row {b}")

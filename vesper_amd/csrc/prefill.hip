@@ -48,6 +48,8 @@ struct PrefillArgs {
     int32_t s_pad;     // cache-plane mode: padded token capacity of the planes
     const int32_t* seq_lens;  // cache-plane mode: per-batch context lengths (device) or nullptr
     const int32_t* chunk_lens;  // cache-plane mode: per-batch number of valid query rows (device) or nullptr
+    const int32_t* page_table;  // cache-plane mode, paged cache: [B][pages_per_seq] page indices (device) or nullptr
+    int32_t page_tokens, pages_per_seq;
     float scale_log2;  // |scale| * log2(e) for bf16; scale * log2(e) for fp32
 };
 
@@ -228,12 +230,26 @@ __global__ void __launch_bounds__(256, 3) prefill_bf16_kernel(PrefillArgs a) {
     const int64_t rowK = a.sk[2] * 2, rowV = a.sv[2] * 2;  // bytes per key row
     auto load_tile = [&](int t, int slot) {
         const int key0 = t * kUnit;
-        const int rows = L - key0;  // > 0
-        __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)Kp + (int64_t)key0 * rowK), 0, (int)((int64_t)rows * rowK), 0x00020000);
-        // VBLK: 32 tokens = 4 token blocks = kUnit * D contiguous elements; bound = the rest of this head's plane
-        const int64_t v_base = VBLK ? (int64_t)key0 * D * 2 : (int64_t)key0 * rowV;
-        const int64_t v_bytes = VBLK ? ((int64_t)a.s_pad - key0) * D * 2 : (int64_t)rows * rowV;
-        __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)Vp + v_base), 0, (int)v_bytes, 0x00020000);
+        int rows = L - key0;  // > 0
+        const char* kb = (const char*)Kp;
+        const char* vb = (const char*)Vp;
+        int local = key0, cap = a.s_pad;  // first token of the tile inside its [cap][D] slab
+        if constexpr (VBLK) {
+            if (a.page_table) {  // paged cache: a tile (32 tokens) never straddles a page (a multiple of 64 tokens)
+                const int pg = key0 / a.page_tokens;
+                local = key0 - pg * a.page_tokens;
+                cap = a.page_tokens;
+                const int64_t slab = (int64_t)a.page_table[(int64_t)b * a.pages_per_seq + pg] * a.Hkv + kvh;
+                kb = (const char*)a.k + slab * cap * D * 2;
+                vb = (const char*)a.v + slab * cap * D * 2;
+                rows = min(rows, cap - local);
+            }
+        }
+        __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc((void*)(kb + (int64_t)local * rowK), 0, (int)((int64_t)rows * rowK), 0x00020000);
+        // VBLK: 32 tokens = 4 token blocks = kUnit * D contiguous elements; bound = the rest of this head's slab
+        const int64_t v_base = VBLK ? (int64_t)local * D * 2 : (int64_t)key0 * rowV;
+        const int64_t v_bytes = VBLK ? ((int64_t)cap - local) * D * 2 : (int64_t)rows * rowV;
+        __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc((void*)(vb + v_base), 0, (int)v_bytes, 0x00020000);
         uint16_t* dstK = smem + slot * SLOT;
         uint16_t* dstV = smem + (2 + slot) * SLOT;
 #pragma unroll
@@ -586,7 +602,6 @@ extern "C" int vsp_attn_prefill_cached(const vsp_tensor* q, const vsp_kv_cache* 
     if (!q || !out) return VSP_ERR_NULL;
     int rc = check_kv_cache(cache);
     if (rc != VSP_OK) return rc;
-    if (cache->page_table) return VSP_ERR_UNSUPPORTED;  // paged caches: append, read and decode only
     if (q->ndim != 4 || out->ndim != 4) return VSP_ERR_NDIM;
     const int64_t B = q->shape[0], Hq = q->shape[1], T = q->shape[2], D = q->shape[3];
     const int64_t Hkv = cache->Hkv;
@@ -657,6 +672,12 @@ extern "C" int vsp_attn_prefill_cached(const vsp_tensor* q, const vsp_kv_cache* 
     a.s_pad = (int)s_phys;
     a.seq_lens = seq_lens;
     a.chunk_lens = chunk_lens;
+    if (cache->page_table && cache->format == VSP_KV_BF16) {
+        a.page_table = cache->page_table;
+        a.page_tokens = cache->page_tokens;
+        a.pages_per_seq = cache->pages_per_seq;
+        a.s_pad = cache->page_tokens;
+    }
     a.causal = is_causal ? 1 : 0;
     a.n_qtiles = (int)ceil_div(T, kBM);
     a.negate_q = (q->dtype == VSP_BF16 && scale < 0.0f) ? 1 : 0;
