@@ -149,6 +149,34 @@ def test_decode_config4_shape_properties(va):
         assert (ref.float() - out[b:b + 1].float()).abs().max().item() <= 1e-2
 
 
+def test_decode_config5_shape_properties(va):
+    # benchmark config 5 at full size (B16, 64/8 heads, D128, Q8_0 cache, L = 65536)
+    B, Hq, Hkv, S, D = 16, 64, 8, 65536, 128
+    c = va.KVCache(B, Hkv, S, D, fmt="q8_0")
+    g = torch.Generator(device="cuda").manual_seed(13)
+    for t0 in range(0, S, 8192):  # fill through the append path in slices (bounded temporaries)
+        kb = torch.randn(B, Hkv, 8192, D, device=G.dev(), generator=g).to(torch.bfloat16)
+        vb = torch.randn(B, Hkv, 8192, D, device=G.dev(), generator=g).to(torch.bfloat16)
+        c.update(kb, vb, t0, return_views=False)
+        del kb, vb
+    assert c.current_seq_len() == S
+    q = torch.randn(B, Hq, 1, D, device=G.dev(), generator=g).to(torch.bfloat16)
+    out = va.decode_attention(q, c)
+    assert torch.isfinite(out.float()).all()
+    assert torch.equal(out, va.decode_attention(q, c))  # fixed split order: run-to-run deterministic
+    # two (sequence, kv head) slices against a float64 closed form over the dequantised rows the cache holds
+    for b, kvh in ((0, 0), (11, 5)):
+        import ctypes as C
+        kq, vq = c.read(0, S, torch.float32)
+        ks, vs = kq[b, kvh].cpu().numpy().astype(np.float64), vq[b, kvh].cpu().numpy().astype(np.float64)
+        del kq, vq
+        qs = G.bf16_to_np(q[b, kvh * 8:(kvh + 1) * 8, 0]).astype(np.float64)
+        s = qs @ ks.T / math.sqrt(D)
+        p = np.exp(s - s.max(axis=1, keepdims=True))
+        want = (p / p.sum(axis=1, keepdims=True)) @ vs
+        G.assert_bf16_close(G.bf16_to_np(out[b, kvh * 8:(kvh + 1) * 8, 0]), want.astype(np.float32), f"config-5 ({b},{kvh})")
+
+
 def test_decode_argument_errors(va):
     c = va.KVCache(2, 2, 64, 128, fmt="bf16")
     q = torch.zeros(2, 4, 1, 128, dtype=torch.bfloat16, device=G.dev())

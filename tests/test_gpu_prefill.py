@@ -196,6 +196,33 @@ def test_bf16_full_size_properties(va):
     G.assert_bf16_close(G.bf16_to_np(out[b:b + 1, h:h + 1]), want, "config-2 slice")
 
 
+def test_bf16_config3_size_properties(va):
+    # benchmark config 3 shape (B1, 32/8 heads, D128, N8192)
+    B, Hq, Hkv, N, D = 1, 32, 8, 8192, 128
+    g = torch.Generator(device="cuda").manual_seed(9)
+    q = (torch.randn(B, Hq, N, D, device=G.dev(), generator=g) * 0.5).to(torch.bfloat16)
+    k = (torch.randn(B, Hkv, N, D, device=G.dev(), generator=g) * 0.5).to(torch.bfloat16)
+    v = (torch.randn(B, Hkv, N, D, device=G.dev(), generator=g) * 0.5).to(torch.bfloat16)
+    scale = 1.0 / math.sqrt(D)
+    out, lse = va.flash_attention(q, k, v, scale, True, return_lse=True)
+    assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
+    assert torch.equal(out, va.flash_attention(q, k, v, scale, True))
+    # causal prefix: rows < 4096 see exactly the tiles a 4096-token launch sees, in the same order -> bit-identical
+    half = va.flash_attention(q[:, :, :4096].contiguous(), k[:, :, :4096].contiguous(), v[:, :, :4096].contiguous(), scale, True)
+    assert torch.equal(out[:, :, :4096], half)
+    # the last 128 rows of two heads against a float64 closed form over all 8192 keys
+    for h in (0, 29):
+        qs = G.bf16_to_np(q[0, h, N - 128:]).astype(np.float64)
+        ks, vs = G.bf16_to_np(k[0, h // 4]).astype(np.float64), G.bf16_to_np(v[0, h // 4]).astype(np.float64)
+        s = qs @ ks.T * scale
+        s[np.arange(N)[None, :] > (N - 128 + np.arange(128))[:, None]] = -np.inf
+        p = np.exp(s - s.max(axis=1, keepdims=True))
+        want = (p / p.sum(axis=1, keepdims=True)) @ vs
+        G.assert_bf16_close(G.bf16_to_np(out[0, h, N - 128:]), want.astype(np.float32), f"config-3 head {h}")
+        want_lse = s.max(axis=1) + np.log(p.sum(axis=1))
+        assert np.abs(lse[0, h, N - 128:].cpu().numpy() - want_lse).max() < 2e-2
+
+
 def test_validation_errors_follow_the_reference(va):
     d = G.dev()
     f = lambda *s, dt=torch.bfloat16: torch.zeros(*s, dtype=dt, device=d)
