@@ -80,6 +80,22 @@ int vref_flash_attention(const float* q, const float* k, const float* v,
     });
 }
 
+// ops::flash_attention_backward (src/ops/flash_attention.cpp:165-216 -> :366-482), no dropout.  out and lse are
+// the forward's own results for the same inputs.
+int vref_flash_attention_backward(const float* dout, const float* q, const float* k, const float* v,
+                                  const float* out, const float* lse, float* dq, float* dk, float* dv,
+                                  int64_t B, int64_t H, int64_t N, int64_t D, float scale, int is_causal) {
+    return guarded([&] {
+        Tensor tdo = from_host(dout, {B, H, N, D}), tq = from_host(q, {B, H, N, D});
+        Tensor tk = from_host(k, {B, H, N, D}), tv = from_host(v, {B, H, N, D});
+        Tensor to = from_host(out, {B, H, N, D}), tl = from_host(lse, {B, H, N});
+        auto g = vesper::ops::flash_attention_backward(tdo, tq, tk, tv, to, tl, scale, is_causal != 0, 0.0f, Tensor());
+        to_host(std::get<0>(g), dq);
+        to_host(std::get<1>(g), dk);
+        to_host(std::get<2>(g), dv);
+    });
+}
+
 // Same, but with arbitrary (possibly mismatching) shapes so that the
 // validation errors of the front-end can be observed.
 int vref_flash_attention_shapes(const int64_t* qs, const int64_t* ks, const int64_t* vs,

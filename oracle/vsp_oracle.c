@@ -490,3 +490,46 @@ void orc_rope_apply_f32(const float* x, int64_t B, int64_t H, int64_t S, int64_t
                 out[o + 1] = t3 + t4;
             }
 }
+
+/* ---- attention backward -------------------------------------------------- */
+
+/* src/ops/flash_attention.cpp:366-482, dropout off. */
+void orc_flash_attention_backward_f32(const float* dO, const float* Q, const float* K, const float* V,
+                                      const float* O, const float* Lse, float* dQ, float* dK, float* dV,
+                                      int64_t B, int64_t H, int64_t N, int64_t D, float scale, int is_causal) {
+    const int64_t total = B * H * N * D;
+    for (int64_t i = 0; i < total; ++i) dQ[i] = dK[i] = dV[i] = 0.0f;
+    float* Di = (float*)malloc(sizeof(float) * (size_t)(N > 0 ? N : 1));
+    for (int64_t b = 0; b < B; ++b) {
+        for (int64_t h = 0; h < H; ++h) {
+            const int64_t off = (b * H + h) * N * D;
+            const float *q_ptr = Q + off, *k_ptr = K + off, *v_ptr = V + off, *o_ptr = O + off, *do_ptr = dO + off;
+            const float* l_ptr = Lse + (b * H + h) * N;
+            float *dq_ptr = dQ + off, *dk_ptr = dK + off, *dv_ptr = dV + off;
+            for (int64_t i = 0; i < N; ++i) {
+                float sum = 0.0f;
+                for (int64_t d = 0; d < D; ++d) sum += do_ptr[i * D + d] * o_ptr[i * D + d];
+                Di[i] = sum;
+            }
+            for (int64_t qi = 0; qi < N; ++qi) {
+                const float li = l_ptr[qi];
+                const int64_t k_end = is_causal ? qi + 1 : N;
+                for (int64_t ki = 0; ki < k_end; ++ki) {
+                    float score = 0.0f;
+                    for (int64_t d = 0; d < D; ++d) score += q_ptr[qi * D + d] * k_ptr[ki * D + d];
+                    score *= scale;
+                    const float p = expf(score - li);
+                    for (int64_t d = 0; d < D; ++d) dv_ptr[ki * D + d] += p * do_ptr[qi * D + d];
+                    float dp = 0.0f;
+                    for (int64_t d = 0; d < D; ++d) dp += do_ptr[qi * D + d] * v_ptr[ki * D + d];
+                    const float ds = p * (dp - Di[qi]);
+                    for (int64_t d = 0; d < D; ++d) {
+                        dq_ptr[qi * D + d] += scale * ds * k_ptr[ki * D + d];
+                        dk_ptr[ki * D + d] += scale * ds * q_ptr[qi * D + d];
+                    }
+                }
+            }
+        }
+    }
+    free(Di);
+}

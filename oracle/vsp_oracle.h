@@ -17,6 +17,9 @@
  *                             float64 closed form; the reference tests' known
  *                             answers (identity/causal-prefix/constant-V/...).
  *   orc_sdpa_f32 / _matmul    same.
+ *   orc_flash_attention_backward_f32  bit-exact vs oracle/_ref (flash_attention_backward) and a fixture
+ *                             written from it; float64 closed-form gradients; central finite
+ *                             differences of the forward (the reference's own gradient check).
  *   orc_repeat_kv_f32         bit-exact vs _ref; iota head-map known answer.
  *   orc_gqa_attention_f32     bit-identical to repeat_kv -> sdpa by test.
  *   orc_slice_bounds,
@@ -69,6 +72,15 @@ int orc_flash_attention_check(int q_ndim, const int64_t* q_shape, int k_ndim, co
  * use_dropout == false).  Contiguous [B,H,N,D]; lse [B,H,N] may be NULL. */
 void orc_flash_attention_f32(const float* q, const float* k, const float* v, float* out, float* lse,
                              int64_t B, int64_t H, int64_t N, int64_t D, float scale, int is_causal);
+
+/* flash_attention_backward_cpu_dispatch, src/ops/flash_attention.cpp:366-482 (no dropout): contiguous
+ * [B,H,N,D] operands, lse [B,H,N]; dq, dk, dv are OVERWRITTEN (the reference allocates them as zeros,
+ * :178-181, and accumulates).  Di = rowsum(dO*O); for every (qi, ki <= qi if causal): p = expf(q.k*scale - lse),
+ * dV[ki] += p*dO[qi], dP = dO[qi].V[ki], dS = p*(dP - Di), dQ[qi] += scale*dS*K[ki], dK[ki] += scale*dS*Q[qi],
+ * all in the reference's loop order. */
+void orc_flash_attention_backward_f32(const float* dout, const float* q, const float* k, const float* v,
+                                      const float* out, const float* lse, float* dq, float* dk, float* dv,
+                                      int64_t B, int64_t H, int64_t N, int64_t D, float scale, int is_causal);
 
 /* ops::repeat_kv, src/ops/attention_ops.cpp:30-57 (CPU dispatch) and :92-155. */
 void orc_repeat_kv_f32(const float* in, float* out, int64_t B, int64_t Hkv, int64_t S, int64_t D,

@@ -74,6 +74,8 @@ def _load_oracle():
     L.orc_q8_0_quantize_row.restype = None
     L.orc_q8_0_dequantize_row.argtypes = [u16p, i8p, i64, f32p]
     L.orc_q8_0_dequantize_row.restype = None
+    L.orc_flash_attention_backward_f32.argtypes = [f32p] * 9 + [i64] * 4 + [C.c_float, C.c_int]
+    L.orc_flash_attention_backward_f32.restype = None
     L.orc_rope_angles.argtypes = [C.c_int, C.c_int, C.c_int, C.c_float, f32p]
     L.orc_rope_angles.restype = None
     L.orc_rope_apply_f32.argtypes = [f32p] + [i64] * 4 + [f32p, f32p]
@@ -262,6 +264,16 @@ def q8_0_dequantize(d, qs):
     return out
 
 
+def flash_attention_backward(dout, q, k, v, out, lse, scale, causal=True):
+    """Gradients (dq, dk, dv) of the reference's flash attention, all heads equal (no GQA: repeat first)."""
+    dout, q, k, v, out, lse = [_f32(x) for x in (dout, q, k, v, out, lse)]
+    B, H, N, D = q.shape
+    dq, dk, dv = np.empty_like(q), np.empty_like(q), np.empty_like(q)
+    orc.orc_flash_attention_backward_f32(_p(dout), _p(q), _p(k), _p(v), _p(out), _p(lse), _p(dq), _p(dk), _p(dv),
+                                         B, H, N, D, scale, int(causal))
+    return dq, dk, dv
+
+
 def rope_angles(seq_len, head_dim, start_pos=0, theta=10000.0):
     out = np.empty((seq_len, head_dim // 2), np.float32)
     orc.orc_rope_angles(seq_len, head_dim, start_pos, theta, _p(out))
@@ -306,6 +318,8 @@ def _load_ref():
     L.vref_gqacache_update.argtypes = [C.c_void_p, f32p, f32p] + [i64] * 5 + [f32p, f32p]
     L.vref_gqa_core.argtypes = [C.c_void_p, f32p, f32p, f32p] + [i64] * 5 + [C.c_int, C.c_int, f32p]
     L.vref_gqa_ctor.argtypes = [i64, i64, i64, i64p, i64p]
+    if hasattr(L, "vref_flash_attention_backward"):
+        L.vref_flash_attention_backward.argtypes = [f32p] * 9 + [i64] * 4 + [C.c_float, C.c_int]
     if hasattr(L, "vref_rope_frequencies"):
         L.vref_rope_frequencies.argtypes = [C.c_int, C.c_int, C.c_int, C.c_float, f32p]
         L.vref_apply_rotary_emb.argtypes = [f32p] + [i64] * 4 + [f32p, f32p]
@@ -421,6 +435,15 @@ class RefKVCache:
         _rchk(ref.vref_gqa_rope_core(self._h, _p(q), _p(new_k), _p(new_v), B, Hq, Hkv, T, D, start_pos,
                                      theta, _p(q_rot), _p(out)))
         return q_rot, out
+
+
+def ref_flash_attention_backward(dout, q, k, v, out, lse, scale, causal=True):
+    dout, q, k, v, out, lse = [_f32(x) for x in (dout, q, k, v, out, lse)]
+    B, H, N, D = q.shape
+    dq, dk, dv = np.empty_like(q), np.empty_like(q), np.empty_like(q)
+    _rchk(ref.vref_flash_attention_backward(_p(dout), _p(q), _p(k), _p(v), _p(out), _p(lse), _p(dq), _p(dk), _p(dv),
+                                            B, H, N, D, scale, int(causal)))
+    return dq, dk, dv
 
 
 def ref_rope_angles(seq_len, head_dim, start_pos=0, theta=10000.0):

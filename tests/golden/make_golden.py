@@ -157,6 +157,23 @@ def rope_cases():
     save("rope", **out)
 
 
+def backward_cases():
+    # ops::flash_attention_backward (src/ops/flash_attention.cpp:165-216, :366-482) on the forward's own out/lse:
+    # the shape of the reference's own test (tests/test_flash_attention.cpp:292-340), a ragged causal one, a
+    # non-causal one and D=128.
+    out = {}
+    for tag, (B, H, N, D, causal, seed) in {"t16": (1, 2, 16, 32, 1, 9000), "r70": (2, 3, 70, 64, 1, 9010),
+                                            "nc33": (1, 2, 33, 64, 0, 9020), "d128": (1, 2, 130, 128, 1, 9030)}.items():
+        q, k, v = I.qkv(seed, B, H, H, N, N, D)
+        dout = I.normal(seed + 5, (B, H, N, D))
+        scale = float(np.float32(1.0 / np.sqrt(D)))
+        o, lse = O.ref_flash_attention(q, k, v, scale, bool(causal))
+        dq, dk, dv = O.ref_flash_attention_backward(dout, q, k, v, o, lse, scale, bool(causal))
+        out[tag + "_meta"] = np.array([B, H, N, D, causal, seed], np.int64)
+        out[tag + "_dq"], out[tag + "_dk"], out[tag + "_dv"] = dq, dk, dv
+    save("flash_backward", **out)
+
+
 def bf16_vectors():
     rng = np.random.default_rng(42)
     bits = np.concatenate([
@@ -179,4 +196,5 @@ if __name__ == "__main__":
     kv_cache_cases()
     gqa_core_cases()
     rope_cases()
+    backward_cases()
     bf16_vectors()
