@@ -198,6 +198,21 @@ int vsp_kv_view_f32(const vsp_kv_cache* cache, vsp_tensor* k_view, vsp_tensor* v
 int vsp_attn_prefill(const vsp_tensor* q, const vsp_tensor* k, const vsp_tensor* v, vsp_tensor* out, vsp_tensor* lse,
                      float scale, int is_causal, float dropout_p, int training, void* stream);
 
+/* ops::flash_attention_backward (include/vesper/ops/flash_attention.h:61-66, src/ops/flash_attention.cpp:165-216)
+ * = flash_attention_backward_hip_dispatch (header :80-92, src/ops/hip/flash_attention.hip:183-299), the
+ * training-side companion of vsp_attn_prefill; mathematics of the CPU backward, src/ops/flash_attention.cpp:366-482,
+ * without dropout: Di = rowsum(dO*O), P = exp(scale q.k - lse), dV = P^T dO, dS = P*(dO V^T - Di), dQ = scale dS K,
+ * dK = scale dS^T Q.  dout/q/out/dq [B,Hq,N,D], k/v/dk/dv [B,Hkv,N,D] (Hq % Hkv == 0: dk/dv of a kv head sum over
+ * its query heads, the gradient of ops::repeat_kv), lse [B,Hq,N] fp32 as written by vsp_attn_prefill; fp32 or bf16
+ * (one dtype; fp32 arithmetic on matrix cores, bf16 gradients rounded to nearest even), D in {64,128}, any strides
+ * with stride[3]==1.  dq/dk/dv are overwritten.  No atomics: results are bitwise reproducible (the reference's
+ * HIP kernel accumulates dQ with atomicAdd).  workspace: vsp_attn_backward_workspace_bytes(B, Hq, N) bytes. */
+size_t vsp_attn_backward_workspace_bytes(int32_t B, int32_t Hq, int32_t N);
+int vsp_attn_prefill_backward(const vsp_tensor* dout, const vsp_tensor* q, const vsp_tensor* k, const vsp_tensor* v,
+                              const vsp_tensor* out, const vsp_tensor* lse, vsp_tensor* dq, vsp_tensor* dk,
+                              vsp_tensor* dv, float scale, int is_causal, void* workspace, size_t workspace_bytes,
+                              void* stream);
+
 /* Chunked / offset prefill straight over the cache planes (no counterpart in the reference, whose causal mask is
  * [T,T] and cannot be added to [T,L] scores, src/nn/functional.cpp:406-410; the semantics are the rows
  * [L-T, L) of the reference's full causal forward over L tokens, src/ops/flash_attention.cpp:218-364):

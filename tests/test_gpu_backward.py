@@ -1,0 +1,114 @@
+"""Attention backward on the GPU through the C ABI (vsp_attn_prefill_backward) against the oracle (bit-exact to the
+compiled reference), the reference-written fixture and a float64 closed form.  fp32: 1e-4 relative.  bf16 inputs:
+the arithmetic is fp32 on exactly widened operands, so the only extra error is the final rounding of the gradients."""
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import _gpu as G
+import _inputs as I
+import _oracle as O
+from test_oracle_backward import closed_form_grads
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+@pytest.fixture(scope="module")
+def va():
+    import vesper_amd
+    return vesper_amd
+
+
+def _forward_then_backward(va, q, k, v, dout, scale, causal, bf16=False):
+    cv = G.to_bf16_dev if bf16 else G.f32_dev
+    dq_, dk_, dv_, dd_ = cv(q), cv(k), cv(v), cv(dout)
+    out, lse = va.flash_attention(dq_, dk_, dv_, scale, causal, return_lse=True)
+    return va.flash_attention_backward(dd_, dq_, dk_, dv_, out, lse, scale, causal)
+
+
+def test_fixture_written_from_the_reference(va):
+    z = np.load(os.path.join(GOLD, "flash_backward.npz"), allow_pickle=False)
+    for tag in ("r70", "nc33", "d128"):   # t16 has D = 32, which the kernels do not implement
+        B, H, N, D, causal, seed = [int(x) for x in z[tag + "_meta"]]
+        q, k, v = I.qkv(seed, B, H, H, N, N, D)
+        dout = I.normal(seed + 5, (B, H, N, D))
+        scale = float(np.float32(1.0 / np.sqrt(D)))
+        dq, dk, dv = _forward_then_backward(va, q, k, v, dout, scale, bool(causal))
+        G.assert_f32_close(dq.cpu().numpy(), z[tag + "_dq"], tag + " dq")
+        G.assert_f32_close(dk.cpu().numpy(), z[tag + "_dk"], tag + " dk")
+        G.assert_f32_close(dv.cpu().numpy(), z[tag + "_dv"], tag + " dv")
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,N,D,causal", [(1, 4, 2, 100, 64, True), (2, 8, 2, 257, 128, True), (1, 4, 4, 64, 128, False),
+                                                 (1, 6, 1, 33, 64, True)])
+def test_f32_gqa_against_oracle_through_repeat_kv(va, B, Hq, Hkv, N, D, causal):
+    # GroupedQueryAttention trains through repeat_kv -> flash_attention: dk / dv of a kv head are the sums of the
+    # repeated heads' gradients (the backward of ops::repeat_kv, src/ops/attention_ops.cpp:120-150)
+    q, k, v = I.qkv(700 + N, B, Hq, Hkv, N, N, D)
+    dout = I.normal(705 + N, (B, Hq, N, D))
+    scale = float(np.float32(1.0 / np.sqrt(D)))
+    n = Hq // Hkv
+    kr, vr = O.repeat_kv(k, n), O.repeat_kv(v, n)
+    out, lse = O.flash_attention(q, kr, vr, scale, causal, return_lse=True)
+    wq, wk, wv = O.flash_attention_backward(dout, q, kr, vr, out, lse, scale, causal)
+    wk = wk.reshape(B, Hkv, n, N, D).sum(2)
+    wv = wv.reshape(B, Hkv, n, N, D).sum(2)
+    dq, dk, dv = _forward_then_backward(va, q, k, v, dout, scale, causal)
+    G.assert_f32_close(dq.cpu().numpy(), wq, "dq")
+    G.assert_f32_close(dk.cpu().numpy(), wk, "dk")
+    G.assert_f32_close(dv.cpu().numpy(), wv, "dv")
+    # and the float64 closed form (independent algebra)
+    cq, ck, cv = closed_form_grads(dout, q, kr, vr, scale, causal)
+    G.assert_f32_close(dq.cpu().numpy(), cq.astype(np.float32), "dq closed form")
+    G.assert_f32_close(dk.cpu().numpy(), ck.reshape(B, Hkv, n, N, D).sum(2).astype(np.float32), "dk closed form")
+
+
+def test_single_token(va):
+    # N = 1: P = 1, so dS = dP - Di = 0 and dq = dk = 0 exactly in exact arithmetic, dv = dout
+    q, k, v = I.qkv(750, 1, 2, 2, 1, 1, 64)
+    dout = I.normal(755, (1, 2, 1, 64))
+    dq, dk, dv = _forward_then_backward(va, q, k, v, dout, 0.125, True)
+    assert np.abs(dq.cpu().numpy()).max() < 1e-5 and np.abs(dk.cpu().numpy()).max() < 1e-5
+    G.assert_f32_close(dv.cpu().numpy(), dout, "dv")
+
+
+def test_bf16_inputs_and_determinism(va):
+    B, Hq, Hkv, N, D = 2, 8, 2, 300, 128
+    q, k, v = [O.bf16_round(x * np.float32(0.5)) for x in I.qkv(800, B, Hq, Hkv, N, N, D)]
+    dout = O.bf16_round(I.normal(805, (B, Hq, N, D)))
+    scale = 1.0 / math.sqrt(D)
+    dq, dk, dv = _forward_then_backward(va, q, k, v, dout, scale, True, bf16=True)
+    again = _forward_then_backward(va, q, k, v, dout, scale, True, bf16=True)
+    for a, b in zip((dq, dk, dv), again):
+        assert torch.equal(a, b)          # no atomics: bitwise reproducible
+    kr, vr = O.repeat_kv(k, 4), O.repeat_kv(v, 4)
+    cq, ck, cv = closed_form_grads(dout, q, kr, vr, float(np.float32(scale)), True)
+    ck = ck.reshape(B, Hkv, 4, N, D).sum(2)
+    cv = cv.reshape(B, Hkv, 4, N, D).sum(2)
+    # the forward's bf16 output and fp32 lse feed the backward: tolerance of the bf16 path
+    for got, want, name in ((dq, cq, "dq"), (dk, ck, "dk"), (dv, cv, "dv")):
+        g = G.bf16_to_np(got)
+        err = np.abs(g - want)
+        assert np.isfinite(g).all() and err.max() <= 3e-2 * max(1.0, np.abs(want).max()), (name, err.max())
+        assert err.mean() <= 2e-3 * max(1.0, np.abs(want).mean() * 10), (name, err.mean())
+
+
+def test_argument_errors(va):
+    d = G.dev()
+    q = torch.zeros(1, 4, 8, 64, device=d)
+    k = torch.zeros(1, 2, 8, 64, device=d)
+    lse = torch.zeros(1, 4, 8, device=d)
+    with pytest.raises(va.VspError):   # head dim 32 is not implemented
+        z = torch.zeros(1, 2, 8, 32, device=d)
+        va.flash_attention_backward(z, z, z, z, z, torch.zeros(1, 2, 8, device=d), 0.1)
+    with pytest.raises(va.VspError):   # 3 query heads over 2 kv heads
+        q3 = torch.zeros(1, 3, 8, 64, device=d)
+        va.flash_attention_backward(q3, q3, k, k, q3, torch.zeros(1, 3, 8, device=d), 0.1)
+    with pytest.raises(va.VspError):   # mixed dtypes
+        va.flash_attention_backward(q.to(torch.bfloat16), q, k, k, q, lse, 0.1)
+    dq, dk, dv = va.flash_attention_backward(q, q, k, k, q, lse, 0.1)
+    assert dq.shape == q.shape and dk.shape == k.shape and not dq.any() and not dv.any()

@@ -60,6 +60,18 @@ def flash_attention(q, k, v, scale, is_causal=True, dropout_p=0.0, training=Fals
     return (out, lse) if return_lse else out
 
 
+def flash_attention_backward(grad_output, q, k, v, output, lse, scale, is_causal=True):
+    """ops::flash_attention_backward: (dq, dk, dv); k, v may have fewer heads than q (their gradients then sum over
+    the query heads of each group)."""
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    descs = [_desc(t) for t in (grad_output, q, k, v, output, lse, dq, dk, dv)]
+    nws = lib.vsp_attn_backward_workspace_bytes(q.shape[0], q.shape[1], q.shape[2])
+    ws = torch.empty(max(nws, 4), dtype=torch.uint8, device=q.device)
+    check(lib.vsp_attn_prefill_backward(*[C.byref(d) for d in descs], float(scale), int(bool(is_causal)),
+                                        C.c_void_p(ws.data_ptr()), nws, _stream(q)))
+    return dq, dk, dv
+
+
 class RopeTable:
     """{cos, sin} of the angles of functional::compute_rope_frequencies (src/nn/functional.cpp:424-443) for
     absolute positions [0, length): computed once on the host by the library, kept on the device."""

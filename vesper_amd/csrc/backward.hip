@@ -1,0 +1,364 @@
+// Flash-attention backward for gfx950.
+//
+// Replaces flash_attention_backward_hip_dispatch (include/vesper/ops/flash_attention.h:80-92,
+// src/ops/hip/flash_attention.hip:183-299) with the mathematics of the reference's CPU backward
+// (src/ops/flash_attention.cpp:366-482): with P = exp(scale q.k - lse) recomputed from the forward's
+// log-sum-exp,  Di = rowsum(dO * O),  dV = P^T dO,  dP = dO V^T,  dS = P * (dP - Di),
+// dQ = scale dS K,  dK = scale dS^T Q.  Differences from the reference's HIP kernel: matrix cores
+// (fp32 MFMA 32x32x2) instead of scalar FMAs, any D in {64, 128}, grouped-query heads folded in
+// (dK / dV of a kv head sum over its query heads, the gradient of ops::repeat_kv), and no atomics:
+// dQ is produced by one pass that owns query rows, dK / dV by a second pass that owns key rows, so the
+// result is bitwise reproducible (the reference accumulates dQ with atomicAdd).
+//
+// Arithmetic is fp32 throughout; bf16 operands are widened exactly on load and gradients are rounded
+// to bf16 (round-to-nearest-even) on store.  This is the training-side companion of the inference
+// path and is written for clarity first: plain LDS tiles, no direct-to-LDS loads, one wavefront per
+// SIMD.
+#include <math.h>
+
+#include "vsp_common.hpp"
+
+namespace vsp {
+namespace {
+
+struct BwdArgs {
+    const void *dout, *q, *k, *v, *out;
+    const float* lse;
+    void *dq, *dk, *dv;
+    float* delta;                          // workspace: Di [B][Hq][N]
+    int64_t s_do[3], s_q[3], s_k[3], s_v[3], s_o[3], s_l[3], s_dq[3], s_dk[3], s_dv[3];
+    int32_t B, Hq, Hkv, n_rep, N;
+    int32_t causal;
+    float scale;
+};
+
+template <typename T>
+__device__ inline float ld(const T* p);
+template <>
+__device__ inline float ld<float>(const float* p) { return *p; }
+template <>
+__device__ inline float ld<uint16_t>(const uint16_t* p) { return bf16_bits_to_f32(*p); }
+template <typename T>
+__device__ inline void st(T* p, float f);
+template <>
+__device__ inline void st<float>(float* p, float f) { *p = f; }
+template <>
+__device__ inline void st<uint16_t>(uint16_t* p, float f) { *p = f32_to_bf16_bits(f); }
+
+// Di[b][h][i] = sum_d dO[i][d] * O[i][d]   (src/ops/flash_attention.cpp:416-423); one wavefront per row.
+template <typename T>
+__global__ void __launch_bounds__(256) bwd_delta_kernel(BwdArgs a, int D) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t rows = (int64_t)a.B * a.Hq * a.N;
+    if (row >= rows) return;
+    const int i = (int)(row % a.N);
+    const int64_t bh = row / a.N;
+    const int h = (int)(bh % a.Hq), b = (int)(bh / a.Hq);
+    const T* po = (const T*)a.out + (int64_t)b * a.s_o[0] + (int64_t)h * a.s_o[1] + (int64_t)i * a.s_o[2];
+    const T* pd = (const T*)a.dout + (int64_t)b * a.s_do[0] + (int64_t)h * a.s_do[1] + (int64_t)i * a.s_do[2];
+    float s = 0.f;
+    for (int d = lane; d < D; d += 64) s += ld<T>(pd + d) * ld<T>(po + d);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+    if (lane == 0) a.delta[row] = s;
+}
+
+constexpr int kBQ = 128;  // rows (queries or keys) per workgroup, 32 per wavefront
+constexpr int kBT = 32;   // rows of the streamed tile
+
+// ---- dQ: a wavefront owns 32 query rows and walks the key tiles (the forward's structure) ----
+//   S^T[key][q]  = K . Q^T      A = K tile (LDS), B = Q^T (registers)
+//   dP^T[key][q] = V . dO^T     A = V tile (LDS), B = dO^T (registers)
+//   dS^T = exp(scale S^T - lse[q]) * (dP^T - Di[q])        a lane owns one query column: lse, Di are per lane
+//   dQ^T[d][q]  += K^T . dS^T   A = K^T (the same tile read column-wise), B = dS^T straight from registers
+template <int D, typename T>
+__global__ void __launch_bounds__(256) bwd_dq_kernel(BwdArgs a) {
+    constexpr int PITCH = D + 1;
+    constexpr int DB = D / 32;
+    __shared__ float sK[kBT * PITCH];
+    __shared__ float sV[kBT * PITCH];
+    const int n_qtiles = (a.N + kBQ - 1) / kBQ;
+    const int bid = blockIdx.x;
+    const int qt = n_qtiles - 1 - bid / (a.B * a.Hq);
+    const int bh = bid % (a.B * a.Hq);
+    const int b = bh / a.Hq, hq = bh % a.Hq, kvh = hq / a.n_rep;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int ql = lane & 31, h = lane >> 5;
+    const int q0 = qt * kBQ + wave * 32;
+    const int qi = q0 + ql;
+    const int qrow = min(qi, a.N - 1);
+
+    const T* Qp = (const T*)a.q + (int64_t)b * a.s_q[0] + (int64_t)hq * a.s_q[1] + (int64_t)qrow * a.s_q[2];
+    const T* Op = (const T*)a.dout + (int64_t)b * a.s_do[0] + (int64_t)hq * a.s_do[1] + (int64_t)qrow * a.s_do[2];
+    const T* Kp = (const T*)a.k + (int64_t)b * a.s_k[0] + (int64_t)kvh * a.s_k[1];
+    const T* Vp = (const T*)a.v + (int64_t)b * a.s_v[0] + (int64_t)kvh * a.s_v[1];
+    float qf[D / 2], dof[D / 2];
+#pragma unroll
+    for (int ks = 0; ks < D / 2; ++ks) {
+        qf[ks] = ld<T>(Qp + 2 * ks + h);
+        dof[ks] = ld<T>(Op + 2 * ks + h);
+    }
+    const float lse_q = a.lse[(int64_t)b * a.s_l[0] + (int64_t)hq * a.s_l[1] + (int64_t)qrow * a.s_l[2]];
+    const float di_q = a.delta[((int64_t)b * a.Hq + hq) * a.N + qrow];
+
+    const int wg_qmax = min(qt * kBQ + kBQ - 1, a.N - 1);
+    const int kv_end_wg = a.causal ? min(a.N, wg_qmax + 1) : a.N;
+    const int n_tiles = (kv_end_wg + kBT - 1) / kBT;
+    const int kv_end_wave = (q0 < a.N) ? (a.causal ? min(a.N, min(q0 + 31, a.N - 1) + 1) : a.N) : 0;
+
+    f32x16_t acc[DB];
+#pragma unroll
+    for (int i = 0; i < DB; ++i)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) acc[i][j] = 0.f;
+
+    for (int kt = 0; kt < n_tiles; ++kt) {
+        __syncthreads();
+        for (int id = tid; id < kBT * D; id += 256) {
+            const int row = id / D, col = id % D, key = kt * kBT + row;
+            sK[row * PITCH + col] = key < a.N ? ld<T>(Kp + (int64_t)key * a.s_k[2] + col) : 0.f;
+            sV[row * PITCH + col] = key < a.N ? ld<T>(Vp + (int64_t)key * a.s_v[2] + col) : 0.f;
+        }
+        __syncthreads();
+        const int k0 = kt * kBT;
+        if (k0 >= kv_end_wave) continue;
+        f32x16_t s, dp;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) s[j] = dp[j] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < D / 2; ++ks) {
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(sK[ql * PITCH + 2 * ks + h], qf[ks], s, 0, 0, 0);
+            dp = __builtin_amdgcn_mfma_f32_32x32x2f32(sV[ql * PITCH + 2 * ks + h], dof[ks], dp, 0, 0, 0);
+        }
+        const int lim = a.causal ? min(qi, a.N - 1) : a.N - 1;
+        float ds[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int key = k0 + 8 * (v >> 2) + 4 * h + (v & 3);
+            const float p = key <= lim ? expf(s[v] * a.scale - lse_q) : 0.f;
+            ds[v] = p * (dp[v] - di_q);
+        }
+        // dQ^T += K^T . dS^T : contraction slot h of step v is key 8*(v/4) + 4*h + v%4, the key ds[v] belongs to
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int krow = 8 * (v >> 2) + 4 * h + (v & 3);
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+                acc[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(sK[krow * PITCH + 32 * db + ql], ds[v], acc[db], 0, 0, 0);
+        }
+    }
+    if (qi < a.N) {
+        T* op = (T*)a.dq + (int64_t)b * a.s_dq[0] + (int64_t)hq * a.s_dq[1] + (int64_t)qi * a.s_dq[2];
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) st<T>(op + 32 * db + 8 * (v >> 2) + 4 * h + (v & 3), a.scale * acc[db][v]);
+    }
+}
+
+// ---- dK, dV: a wavefront owns 32 key rows of one kv head and walks the query heads of the group and their
+// query tiles (the forward's structure with the roles of queries and keys exchanged) ----
+//   S[q][key]  = Q . K^T        A = Q tile (LDS), B = K^T (registers);  a lane owns one key column
+//   dP[q][key] = dO . V^T       A = dO tile (LDS), B = V^T (registers)
+//   P = exp(scale S - lse[q]),  dS = P * (dP - Di[q])      lse, Di per row: read from LDS
+//   dV^T[d][key] += dO^T . P    A = dO^T (tile read column-wise), B = P from registers
+//   dK^T[d][key] += Q^T . dS    A = Q^T, B = dS
+template <int D, typename T>
+__global__ void __launch_bounds__(256) bwd_dkdv_kernel(BwdArgs a) {
+    constexpr int PITCH = D + 1;
+    constexpr int DB = D / 32;
+    __shared__ float sQ[kBT * PITCH];
+    __shared__ float sO[kBT * PITCH];
+    __shared__ float sL[kBT], sD[kBT];
+    const int n_ktiles = (a.N + kBQ - 1) / kBQ;
+    const int bid = blockIdx.x;
+    const int kt = bid / (a.B * a.Hkv);  // causal: early key tiles see the most queries -> dispatched first
+    const int bh = bid % (a.B * a.Hkv);
+    const int b = bh / a.Hkv, kvh = bh % a.Hkv;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kl = lane & 31, h = lane >> 5;
+    const int key0 = kt * kBQ + wave * 32;
+    const int ki = key0 + kl;
+    const int krow = min(ki, a.N - 1);
+    (void)n_ktiles;
+
+    const T* Kp = (const T*)a.k + (int64_t)b * a.s_k[0] + (int64_t)kvh * a.s_k[1] + (int64_t)krow * a.s_k[2];
+    const T* Vp = (const T*)a.v + (int64_t)b * a.s_v[0] + (int64_t)kvh * a.s_v[1] + (int64_t)krow * a.s_v[2];
+    float kf[D / 2], vf[D / 2];
+#pragma unroll
+    for (int ks = 0; ks < D / 2; ++ks) {
+        kf[ks] = ld<T>(Kp + 2 * ks + h);
+        vf[ks] = ld<T>(Vp + 2 * ks + h);
+    }
+    f32x16_t acck[DB], accv[DB];
+#pragma unroll
+    for (int i = 0; i < DB; ++i)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) acck[i][j] = accv[i][j] = 0.f;
+
+    // query tiles that can see any key of this workgroup / of this wavefront
+    const int wg_kmin = kt * kBQ;
+    const int qt_begin_wg = a.causal ? wg_kmin / kBT : 0;
+    const int n_qt = (a.N + kBT - 1) / kBT;
+    const int q_begin_wave = a.causal ? key0 : 0;
+
+    for (int r = 0; r < a.n_rep; ++r) {
+        const int hq = kvh * a.n_rep + r;
+        const T* Qp = (const T*)a.q + (int64_t)b * a.s_q[0] + (int64_t)hq * a.s_q[1];
+        const T* Op = (const T*)a.dout + (int64_t)b * a.s_do[0] + (int64_t)hq * a.s_do[1];
+        const float* Lp = a.lse + (int64_t)b * a.s_l[0] + (int64_t)hq * a.s_l[1];
+        const float* Dp = a.delta + ((int64_t)b * a.Hq + hq) * a.N;
+        for (int qt = qt_begin_wg; qt < n_qt; ++qt) {
+            __syncthreads();
+            for (int id = tid; id < kBT * D; id += 256) {
+                const int row = id / D, col = id % D, qi = qt * kBT + row;
+                sQ[row * PITCH + col] = qi < a.N ? ld<T>(Qp + (int64_t)qi * a.s_q[2] + col) : 0.f;
+                sO[row * PITCH + col] = qi < a.N ? ld<T>(Op + (int64_t)qi * a.s_do[2] + col) : 0.f;
+            }
+            if (tid < kBT) {
+                const int qi = qt * kBT + tid;
+                sL[tid] = qi < a.N ? Lp[(int64_t)qi * a.s_l[2]] : 0.f;
+                sD[tid] = qi < a.N ? Dp[qi] : 0.f;
+            }
+            __syncthreads();
+            const int qb = qt * kBT;
+            if (key0 >= a.N || qb + kBT - 1 < q_begin_wave) continue;  // no query of this tile sees these keys
+            f32x16_t s, dp;
+#pragma unroll
+            for (int j = 0; j < 16; ++j) s[j] = dp[j] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < D / 2; ++ks) {
+                s = __builtin_amdgcn_mfma_f32_32x32x2f32(sQ[kl * PITCH + 2 * ks + h], kf[ks], s, 0, 0, 0);
+                dp = __builtin_amdgcn_mfma_f32_32x32x2f32(sO[kl * PITCH + 2 * ks + h], vf[ks], dp, 0, 0, 0);
+            }
+            float p[16], ds[16];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = 8 * (v >> 2) + 4 * h + (v & 3);
+                const int qi = qb + row;
+                const bool ok = qi < a.N && ki < a.N && (!a.causal || ki <= qi);
+                p[v] = ok ? expf(s[v] * a.scale - sL[row]) : 0.f;
+                ds[v] = p[v] * (dp[v] - sD[row]);
+            }
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = 8 * (v >> 2) + 4 * h + (v & 3);
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    accv[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(sO[row * PITCH + 32 * db + kl], p[v], accv[db], 0, 0, 0);
+                    acck[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(sQ[row * PITCH + 32 * db + kl], ds[v], acck[db], 0, 0, 0);
+                }
+            }
+        }
+    }
+    if (ki < a.N) {
+        T* pk = (T*)a.dk + (int64_t)b * a.s_dk[0] + (int64_t)kvh * a.s_dk[1] + (int64_t)ki * a.s_dk[2];
+        T* pv = (T*)a.dv + (int64_t)b * a.s_dv[0] + (int64_t)kvh * a.s_dv[1] + (int64_t)ki * a.s_dv[2];
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int d = 32 * db + 8 * (v >> 2) + 4 * h + (v & 3);
+                st<T>(pk + d, a.scale * acck[db][v]);
+                st<T>(pv + d, accv[db][v]);
+            }
+    }
+}
+
+int check4(const vsp_tensor* t, int64_t B, int64_t H, int64_t N, int64_t D, int dtype) {
+    if (!t) return VSP_ERR_NULL;
+    if (t->ndim != 4) return VSP_ERR_NDIM;
+    if (t->shape[0] != B || t->shape[1] != H || t->shape[2] != N || t->shape[3] != D) return VSP_ERR_SHAPE;
+    if (t->dtype != dtype) return VSP_ERR_DTYPE;
+    if (t->stride[3] != 1) return VSP_ERR_STRIDE;
+    if (B * H * N * D > 0 && !t->data) return VSP_ERR_NULL;
+    return VSP_OK;
+}
+
+template <typename T>
+int launch_backward(const BwdArgs& a, int64_t D, hipStream_t st) {
+    const int64_t rows = (int64_t)a.B * a.Hq * a.N;
+    hipLaunchKernelGGL(bwd_delta_kernel<T>, dim3((unsigned)ceil_div(rows, 4)), dim3(256), 0, st, a, (int)D);
+    int rc = check_launch();
+    if (rc != VSP_OK) return rc;
+    const int64_t tiles = ceil_div(a.N, kBQ);
+    const dim3 gq((unsigned)(tiles * a.B * a.Hq)), gk((unsigned)(tiles * a.B * a.Hkv));
+    if (D == 128) {
+        hipLaunchKernelGGL((bwd_dq_kernel<128, T>), gq, dim3(256), 0, st, a);
+        hipLaunchKernelGGL((bwd_dkdv_kernel<128, T>), gk, dim3(256), 0, st, a);
+    } else {
+        hipLaunchKernelGGL((bwd_dq_kernel<64, T>), gq, dim3(256), 0, st, a);
+        hipLaunchKernelGGL((bwd_dkdv_kernel<64, T>), gk, dim3(256), 0, st, a);
+    }
+    return check_launch();
+}
+
+}  // namespace
+}  // namespace vsp
+
+using namespace vsp;
+
+extern "C" size_t vsp_attn_backward_workspace_bytes(int32_t B, int32_t Hq, int32_t N) {
+    if (B <= 0 || Hq <= 0 || N <= 0) return 0;
+    return (size_t)B * (size_t)Hq * (size_t)N * sizeof(float);
+}
+
+extern "C" int vsp_attn_prefill_backward(const vsp_tensor* dout, const vsp_tensor* q, const vsp_tensor* k,
+                                         const vsp_tensor* v, const vsp_tensor* out, const vsp_tensor* lse,
+                                         vsp_tensor* dq, vsp_tensor* dk, vsp_tensor* dv, float scale, int is_causal,
+                                         void* workspace, size_t workspace_bytes, void* stream) {
+    if (!q || !k || !v) return VSP_ERR_NULL;
+    if (q->ndim != 4 || k->ndim != 4 || v->ndim != 4) return VSP_ERR_NDIM;
+    const int64_t B = q->shape[0], Hq = q->shape[1], N = q->shape[2], D = q->shape[3];
+    const int64_t Hkv = k->shape[1];
+    if (Hkv <= 0 ? Hq != 0 : (Hq % Hkv != 0)) return VSP_ERR_SHAPE;
+    const int dt = q->dtype;
+    if (dt != VSP_F32 && dt != VSP_BF16) return VSP_ERR_UNSUPPORTED;
+    int rc;
+    if ((rc = check4(q, B, Hq, N, D, dt)) || (rc = check4(dout, B, Hq, N, D, dt)) || (rc = check4(out, B, Hq, N, D, dt)) ||
+        (rc = check4(dq, B, Hq, N, D, dt)) || (rc = check4(k, B, Hkv, N, D, dt)) || (rc = check4(v, B, Hkv, N, D, dt)) ||
+        (rc = check4(dk, B, Hkv, N, D, dt)) || (rc = check4(dv, B, Hkv, N, D, dt)))
+        return rc;
+    if (!lse) return VSP_ERR_NULL;
+    if (lse->ndim != 3 || lse->shape[0] != B || lse->shape[1] != Hq || lse->shape[2] != N) return VSP_ERR_SHAPE;
+    if (lse->dtype != VSP_F32) return VSP_ERR_DTYPE;
+    if (B * Hq * N * D == 0) return VSP_OK;
+    if (!lse->data) return VSP_ERR_NULL;
+    if (D != 64 && D != 128) return VSP_ERR_UNSUPPORTED;
+    if (!(fabsf(scale) < INFINITY)) return VSP_ERR_ARG;
+    if (N > INT32_MAX / 2) return VSP_ERR_ARG;
+    if (!workspace || workspace_bytes < vsp_attn_backward_workspace_bytes((int32_t)B, (int32_t)Hq, (int32_t)N)) return VSP_ERR_WORKSPACE;
+    if (((uintptr_t)workspace & 3) != 0) return VSP_ERR_ALIGN;
+
+    BwdArgs a{};
+    a.dout = dout->data;
+    a.q = q->data;
+    a.k = k->data;
+    a.v = v->data;
+    a.out = out->data;
+    a.lse = (const float*)lse->data;
+    a.dq = dq->data;
+    a.dk = dk->data;
+    a.dv = dv->data;
+    a.delta = (float*)workspace;
+    for (int i = 0; i < 3; ++i) {
+        a.s_do[i] = dout->stride[i];
+        a.s_q[i] = q->stride[i];
+        a.s_k[i] = k->stride[i];
+        a.s_v[i] = v->stride[i];
+        a.s_o[i] = out->stride[i];
+        a.s_l[i] = lse->stride[i];
+        a.s_dq[i] = dq->stride[i];
+        a.s_dk[i] = dk->stride[i];
+        a.s_dv[i] = dv->stride[i];
+    }
+    a.B = (int)B;
+    a.Hq = (int)Hq;
+    a.Hkv = (int)Hkv;
+    a.n_rep = (int)(Hq / Hkv);
+    a.N = (int)N;
+    a.causal = is_causal ? 1 : 0;
+    a.scale = scale;
+    return dt == VSP_F32 ? launch_backward<float>(a, D, (hipStream_t)stream) : launch_backward<uint16_t>(a, D, (hipStream_t)stream);
+}
