@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on ONE MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|p4k|c3|c4|c5|c4p|c2c|c3c|r2] [--no-cpu] [--no-extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|p4k|c3|c4|c5|c4p|c2c|c3c|r2|b2] [--no-cpu] [--no-extra]
 
 A "step" is one pass of the hot path over one batch of synthetic input that is already resident in
 HBM: one prefill launch (c2, p4k, c3) or one decode call = split-K kernel + combine kernel (c4, c5).
@@ -44,6 +44,9 @@ WORKLOADS = {
     "c3c": dict(kind="prefill_cached", fmt="bf16", B=1, Hq=32, Hkv=8, D=128, N=8192,
                 name="config 3 through the cache: causal GQA prefill bf16 reading K/V from the bf16 cache planes, "
                      "B1, 32 q / 8 kv heads, D128, N8192"),
+    "b2": dict(kind="backward", B=4, Hq=32, Hkv=8, D=128, N=2048,
+               name="attention backward at config 2's shape: causal GQA bf16 in/out, fp32 MFMA arithmetic, "
+                    "B4, 32 q / 8 kv heads, D128, N2048 (dq, dk, dv; 2.5 x the forward's FLOPs)"),
     "r2": dict(kind="rope", fmt="bf16", B=4, Hq=32, Hkv=8, D=128, N=2048,
                name="RoPE + KV append for config 2: q/k/v bf16 views of one fused projection buffer [B,T,(Hq+2Hkv)D], "
                     "rotated q out bf16, bf16 cache, B4, 32 q / 8 kv heads, D128, T2048"),
@@ -89,6 +92,15 @@ class Runner:
             self.work = prefill_flops(w)
             self.unit, self.peak, self.bound = "TFLOP/s", MFMA_BF16_PEAK_TFLOPS, "mfma"
             self.kernel = "prefill_bf16_kernel<128, true>"
+        elif w["kind"] == "backward":
+            B, Hq, Hkv, D, N = w["B"], w["Hq"], w["Hkv"], w["D"], w["N"]
+            mk = lambda h: (torch.randn(B, h, N, D, device=dev, generator=g) * 0.5).to(torch.bfloat16)
+            self.q, self.k, self.v, self.dout = mk(Hq), mk(Hkv), mk(Hkv), mk(Hq)
+            self.scale = 1.0 / math.sqrt(D)
+            self.o, self.lse = va.flash_attention(self.q, self.k, self.v, self.scale, True, return_lse=True)
+            self.work = 2.5 * prefill_flops(w)
+            self.unit, self.peak, self.bound = "TFLOP/s", 157.3, "mfma"   # fp32 MFMA peak
+            self.kernel = "bwd_dkdv_kernel<128, unsigned short>"
         elif w["kind"] == "rope":
             B, Hq, Hkv, D, N = w["B"], w["Hq"], w["Hkv"], w["D"], w["N"]
             fused = (torch.randn(B, N, (Hq + 2 * Hkv) * D, device=dev, generator=g) * 0.5).to(torch.bfloat16)
@@ -159,6 +171,8 @@ class Runner:
     def step(self):
         if self.w["kind"] == "prefill":
             return self.va.flash_attention(self.q, self.k, self.v, self.scale, True)
+        if self.w["kind"] == "backward":
+            return self.va.flash_attention_backward(self.dout, self.q, self.k, self.v, self.o, self.lse, self.scale, True)
         if self.w["kind"] == "prefill_cached":
             return self.cache.prefill(self.q)
         if self.w["kind"] == "rope":
@@ -314,7 +328,8 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16" if primary.w.get("fmt", "bf16") == "bf16" else "q8_0 (int8 payload, fp16 MFMA)",
+        "dtype": ("f32 (bf16 operands widened exactly)" if primary.w["kind"] == "backward"
+                  else "bf16" if primary.w.get("fmt", "bf16") == "bf16" else "q8_0 (int8 payload, fp16 MFMA)"),
         "data": "synthetic",
         "config": {"workload": primary.w["name"], "key": args.workload,
                    "algorithmic_work_per_step": primary.work,
@@ -333,7 +348,7 @@ def main():
 
     if not args.no_extra:
         others = {}
-        for key in ("c2", "p4k", "c3", "c4", "c5", "c4p", "c2c", "c3c", "r2"):
+        for key in ("c2", "p4k", "c3", "c4", "c5", "c4p", "c2c", "c3c", "r2", "b2"):
             if key == args.workload:
                 continue
             r = Runner(key, torch, va)
