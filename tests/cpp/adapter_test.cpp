@@ -143,6 +143,22 @@ static void test_flash_attention_against_oracle() {
                                            to_dev(vb, {B, H, N, D}, DType::BFloat16), scale, causal != 0);
         CHECK(max_abs_diff(to_host(outb), want.data(), want.size()) < 2e-2);
     }
+    // backward on the forward's own output and log-sum-exp (reference tests/test_flash_attention.cpp:292-340)
+    {
+        auto dout = randn(B * H * N * D, 4);
+        orc_flash_attention_f32(q.data(), k.data(), v.data(), want.data(), lse.data(), B, H, N, D, scale, 1);
+        std::vector<float> wq(q.size()), wk(q.size()), wv(q.size());
+        orc_flash_attention_backward_f32(dout.data(), q.data(), k.data(), v.data(), want.data(), lse.data(), wq.data(), wk.data(),
+                                         wv.data(), B, H, N, D, scale, 1);
+        Tensor tq = to_dev(q, {B, H, N, D}, DType::Float32), tk = to_dev(k, {B, H, N, D}, DType::Float32);
+        Tensor tv = to_dev(v, {B, H, N, D}, DType::Float32), tdo = to_dev(dout, {B, H, N, D}, DType::Float32);
+        Tensor out = empty({B, H, N, D}, DType::Float32), l = empty({B, H, N}, DType::Float32);
+        ops::flash_attention_hip_dispatch(tq, tk, tv, out, l, scale, true, 0.0f, false, nullptr);
+        auto g = ops::flash_attention_backward(tdo, tq, tk, tv, out, l, scale, true);
+        CHECK(max_abs_diff(to_host(std::get<0>(g)), wq.data(), wq.size()) < 2e-4);
+        CHECK(max_abs_diff(to_host(std::get<1>(g)), wk.data(), wk.size()) < 2e-4);
+        CHECK(max_abs_diff(to_host(std::get<2>(g)), wv.data(), wv.size()) < 2e-4);
+    }
     // the reference's validation messages (src/ops/flash_attention.cpp:45-59)
     Tensor a = empty({1, 2, 4, 64}, DType::Float32), b = empty({1, 2, 5, 64}, DType::Float32), c3 = empty({2, 4, 64}, DType::Float32);
     CHECK(thrown<std::runtime_error>([&] { ops::flash_attention(c3, c3, c3, 1.f); }) == "flash_attention: inputs must be 4D [B, H, N, D]");

@@ -361,6 +361,25 @@ inline Tensor flash_attention(const Tensor& q, const Tensor& k, const Tensor& v,
     return output;
 }
 
+// include/vesper/ops/flash_attention.h:61-66, src/ops/flash_attention.cpp:165-216: (grad_q, grad_k, grad_v).
+// `output` and `lse` are the forward's results (flash_attention_hip_dispatch writes both).  k and v may carry
+// fewer heads than q: their gradients are then already summed over each group's query heads.
+inline std::tuple<Tensor, Tensor, Tensor> flash_attention_backward(const Tensor& grad_output, const Tensor& q, const Tensor& k,
+                                                                   const Tensor& v, const Tensor& output, const Tensor& lse, float scale,
+                                                                   bool is_causal, float dropout_p = 0.0f) {
+    if (dropout_p > 0.0f) throw_status(VSP_ERR_UNSUPPORTED);
+    if (q.ndim() != 4 || k.ndim() != 4 || v.ndim() != 4) throw_status(VSP_ERR_NDIM);
+    Tensor gq = empty(q.shape(), q.dtype()), gk = empty(k.shape(), k.dtype()), gv = empty(v.shape(), v.dtype());
+    vsp_tensor d0 = grad_output.desc(), d1 = q.desc(), d2 = k.desc(), d3 = v.desc(), d4 = output.desc(), d5 = lse.desc();
+    vsp_tensor o0 = gq.desc(), o1 = gk.desc(), o2 = gv.desc();
+    const size_t ws_bytes = vsp_attn_backward_workspace_bytes((int32_t)q.shape()[0], (int32_t)q.shape()[1], (int32_t)q.shape()[2]);
+    Storage ws(ws_bytes ? ws_bytes : 4);
+    throw_status(vsp_attn_prefill_backward(&d0, &d1, &d2, &d3, &d4, &d5, &o0, &o1, &o2, scale, is_causal ? 1 : 0, ws.data(), ws_bytes,
+                                           current_stream()));
+    hip_check(hipStreamSynchronize(current_stream()), "flash_attention_backward");  // the scratch buffer dies with this scope
+    return {gq, gk, gv};
+}
+
 }  // namespace ops
 
 namespace nn {
