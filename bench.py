@@ -45,7 +45,7 @@ WORKLOADS = {
                 name="config 3 through the cache: causal GQA prefill bf16 reading K/V from the bf16 cache planes, "
                      "B1, 32 q / 8 kv heads, D128, N8192"),
     "b2": dict(kind="backward", B=4, Hq=32, Hkv=8, D=128, N=2048,
-               name="attention backward at config 2's shape: causal GQA bf16 in/out, fp32 MFMA arithmetic, "
+               name="attention backward at config 2's shape: causal GQA bf16 in/out, bf16 MFMA with fp32 accumulation, "
                     "B4, 32 q / 8 kv heads, D128, N2048 (dq, dk, dv; 2.5 x the forward's FLOPs)"),
     "r2": dict(kind="rope", fmt="bf16", B=4, Hq=32, Hkv=8, D=128, N=2048,
                name="RoPE + KV append for config 2: q/k/v bf16 views of one fused projection buffer [B,T,(Hq+2Hkv)D], "
@@ -99,8 +99,8 @@ class Runner:
             self.scale = 1.0 / math.sqrt(D)
             self.o, self.lse = va.flash_attention(self.q, self.k, self.v, self.scale, True, return_lse=True)
             self.work = 2.5 * prefill_flops(w)
-            self.unit, self.peak, self.bound = "TFLOP/s", 157.3, "mfma"   # fp32 MFMA peak
-            self.kernel = "bwd_dkdv_kernel<128, unsigned short>"
+            self.unit, self.peak, self.bound = "TFLOP/s", MFMA_BF16_PEAK_TFLOPS, "mfma"
+            self.kernel = "bwd_delta + bwd_dq_bf16_kernel<128> + bwd_dkdv_bf16_kernel<128> (the three launches of one step)"
         elif w["kind"] == "rope":
             B, Hq, Hkv, D, N = w["B"], w["Hq"], w["Hkv"], w["D"], w["N"]
             fused = (torch.randn(B, N, (Hq + 2 * Hkv) * D, device=dev, generator=g) * 0.5).to(torch.bfloat16)
@@ -328,8 +328,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": ("f32 (bf16 operands widened exactly)" if primary.w["kind"] == "backward"
-                  else "bf16" if primary.w.get("fmt", "bf16") == "bf16" else "q8_0 (int8 payload, fp16 MFMA)"),
+        "dtype": ("bf16" if primary.w.get("fmt", "bf16") == "bf16" else "q8_0 (int8 payload, fp16 MFMA)"),
         "data": "synthetic",
         "config": {"workload": primary.w["name"], "key": args.workload,
                    "algorithmic_work_per_step": primary.work,

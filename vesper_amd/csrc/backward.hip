@@ -10,10 +10,10 @@
 // dQ is produced by one pass that owns query rows, dK / dV by a second pass that owns key rows, so the
 // result is bitwise reproducible (the reference accumulates dQ with atomicAdd).
 //
-// Arithmetic is fp32 throughout; bf16 operands are widened exactly on load and gradients are rounded
-// to bf16 (round-to-nearest-even) on store.  This is the training-side companion of the inference
-// path and is written for clarity first: plain LDS tiles, no direct-to-LDS loads, one wavefront per
-// SIMD.
+// fp32 operands: fp32 MFMA (32x32x2) throughout.  bf16 operands: bf16 MFMA (32x32x16) with fp32 accumulation
+// and fp32 softmax algebra; P and dS are rounded to bf16 (round-to-nearest-even) between the products, as P is
+// in the forward kernel, and the gradients are rounded to bf16 on store.  This is the training-side companion of
+// the inference path: plain LDS tiles filled by ordinary loads, no direct-to-LDS pipeline.
 #include <math.h>
 
 #include "vsp_common.hpp"
@@ -266,6 +266,237 @@ __global__ void __launch_bounds__(256) bwd_dkdv_kernel(BwdArgs a) {
     }
 }
 
+// =============================================================================================
+// bf16 operands: the same two passes on bf16 matrix cores (v_mfma_f32_32x32x16_bf16), fp32 accumulation and
+// fp32 softmax algebra.  Tiles are bf16 in LDS with a padded pitch; the operand that a product contracts
+// over rows (K^T, Q^T, dO^T) is fetched with the transposing LDS read, as V^T is in the forward kernel, and
+// P / dS go from the accumulator registers into the next MFMA without leaving the lane.
+// =============================================================================================
+typedef short s16x4b_t __attribute__((ext_vector_type(4)));
+
+__device__ inline uint2 lds_tr16(const uint16_t* p) {
+    s16x4b_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4b_t*)p);
+    return __builtin_bit_cast(uint2, v);
+}
+// A operand [32 rows d][16 contraction slots] of the transposed tile: contraction slot (h, e) of k-step j is tile
+// row 16 j + 8 (e / 4) + 4 h + e % 4, the row the accumulator register 8 j + e of this lane half belongs to.
+template <int P>
+__device__ inline bf16x8_t load_transposed(const uint16_t* tile, int j, int db, int lane) {
+    const int h = lane >> 5, i16 = lane & 15;
+    const uint16_t* p = tile + (16 * j + 4 * h + (i16 >> 2)) * P + 32 * db + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+    const uint2 lo = lds_tr16(p), hi = lds_tr16(p + 8 * P);
+    return __builtin_bit_cast(bf16x8_t, uint4{lo.x, lo.y, hi.x, hi.y});
+}
+template <int D, int P>
+__device__ inline void fill_tile(uint16_t* dst, const uint16_t* src, int64_t row_stride, int row0, int n_rows, int tid) {
+    constexpr int CPR = D / 8;
+    for (int c = tid; c < kBT * CPR; c += 256) {
+        const int row = c / CPR, col = c % CPR;
+        const uint4 w = row0 + row < n_rows ? *(const uint4*)(src + (int64_t)(row0 + row) * row_stride + 8 * col) : uint4{0, 0, 0, 0};
+        *(uint4*)(dst + row * P + 8 * col) = w;
+    }
+}
+
+template <int D>
+__global__ void __launch_bounds__(256) bwd_dq_bf16_kernel(BwdArgs a) {
+    constexpr int KS = D / 16, DB = D / 32, P = D + 8;
+    __shared__ __attribute__((aligned(16))) uint16_t sK[kBT * P];
+    __shared__ __attribute__((aligned(16))) uint16_t sV[kBT * P];
+    const int n_qtiles = (a.N + kBQ - 1) / kBQ;
+    const int bid = blockIdx.x;
+    const int qt = n_qtiles - 1 - bid / (a.B * a.Hq);
+    const int bh = bid % (a.B * a.Hq);
+    const int b = bh / a.Hq, hq = bh % a.Hq, kvh = hq / a.n_rep;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int ql = lane & 31, h = lane >> 5;
+    const int q0 = qt * kBQ + wave * 32;
+    const int qi = q0 + ql;
+    const int qrow = min(qi, a.N - 1);
+
+    const uint16_t* Qp = (const uint16_t*)a.q + (int64_t)b * a.s_q[0] + (int64_t)hq * a.s_q[1] + (int64_t)qrow * a.s_q[2];
+    const uint16_t* Op = (const uint16_t*)a.dout + (int64_t)b * a.s_do[0] + (int64_t)hq * a.s_do[1] + (int64_t)qrow * a.s_do[2];
+    const uint16_t* Kp = (const uint16_t*)a.k + (int64_t)b * a.s_k[0] + (int64_t)kvh * a.s_k[1];
+    const uint16_t* Vp = (const uint16_t*)a.v + (int64_t)b * a.s_v[0] + (int64_t)kvh * a.s_v[1];
+    bf16x8_t qf[KS], dof[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        qf[ks] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(Qp + 16 * ks + 8 * h));
+        dof[ks] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(Op + 16 * ks + 8 * h));
+    }
+    const float lse_q = a.lse[(int64_t)b * a.s_l[0] + (int64_t)hq * a.s_l[1] + (int64_t)qrow * a.s_l[2]];
+    const float di_q = a.delta[((int64_t)b * a.Hq + hq) * a.N + qrow];
+
+    const int wg_qmax = min(qt * kBQ + kBQ - 1, a.N - 1);
+    const int kv_end_wg = a.causal ? min(a.N, wg_qmax + 1) : a.N;
+    const int n_tiles = (kv_end_wg + kBT - 1) / kBT;
+    const int kv_end_wave = (q0 < a.N) ? (a.causal ? min(a.N, min(q0 + 31, a.N - 1) + 1) : a.N) : 0;
+
+    f32x16_t acc[DB];
+#pragma unroll
+    for (int i = 0; i < DB; ++i)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) acc[i][j] = 0.f;
+
+    for (int kt = 0; kt < n_tiles; ++kt) {
+        __syncthreads();
+        fill_tile<D, P>(sK, Kp, a.s_k[2], kt * kBT, a.N, tid);
+        fill_tile<D, P>(sV, Vp, a.s_v[2], kt * kBT, a.N, tid);
+        __syncthreads();
+        const int k0 = kt * kBT;
+        if (k0 >= kv_end_wave) continue;
+        f32x16_t s, dp;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) s[j] = dp[j] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const bf16x8_t kf = __builtin_bit_cast(bf16x8_t, *(const uint4*)(sK + ql * P + 16 * ks + 8 * h));
+            const bf16x8_t vf = __builtin_bit_cast(bf16x8_t, *(const uint4*)(sV + ql * P + 16 * ks + 8 * h));
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], s, 0, 0, 0);
+            dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, dof[ks], dp, 0, 0, 0);
+        }
+        const int lim = a.causal ? min(qi, a.N - 1) : a.N - 1;
+        uint32_t dsw[2][4];
+#pragma unroll
+        for (int v = 0; v < 16; v += 2) {
+            float d2[2];
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int key = k0 + 8 * ((v + u) >> 2) + 4 * h + ((v + u) & 3);
+                const float p = key <= lim ? expf(s[v + u] * a.scale - lse_q) : 0.f;
+                d2[u] = p * (dp[v + u] - di_q);
+            }
+            dsw[v >> 3][(v & 7) >> 1] = pack_bf16x2(d2[0], d2[1]);
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const bf16x8_t dsf = __builtin_bit_cast(bf16x8_t, uint4{dsw[j][0], dsw[j][1], dsw[j][2], dsw[j][3]});
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+                acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_transposed<P>(sK, j, db, lane), dsf, acc[db], 0, 0, 0);
+        }
+    }
+    if (qi < a.N) {
+        uint16_t* op = (uint16_t*)a.dq + (int64_t)b * a.s_dq[0] + (int64_t)hq * a.s_dq[1] + (int64_t)qi * a.s_dq[2];
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int vq = 0; vq < 4; ++vq) {
+                uint2 w;
+                w.x = pack_bf16x2(a.scale * acc[db][4 * vq], a.scale * acc[db][4 * vq + 1]);
+                w.y = pack_bf16x2(a.scale * acc[db][4 * vq + 2], a.scale * acc[db][4 * vq + 3]);
+                *(uint2*)(op + 32 * db + 8 * vq + 4 * h) = w;
+            }
+    }
+}
+
+template <int D>
+__global__ void __launch_bounds__(256) bwd_dkdv_bf16_kernel(BwdArgs a) {
+    constexpr int KS = D / 16, DB = D / 32, P = D + 8;
+    __shared__ __attribute__((aligned(16))) uint16_t sQ[kBT * P];
+    __shared__ __attribute__((aligned(16))) uint16_t sO[kBT * P];
+    __shared__ float sL[kBT], sD[kBT];
+    const int bid = blockIdx.x;
+    const int kt = bid / (a.B * a.Hkv);
+    const int bh = bid % (a.B * a.Hkv);
+    const int b = bh / a.Hkv, kvh = bh % a.Hkv;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kl = lane & 31, h = lane >> 5;
+    const int key0 = kt * kBQ + wave * 32;
+    const int ki = key0 + kl;
+    const int krow = min(ki, a.N - 1);
+
+    const uint16_t* Kp = (const uint16_t*)a.k + (int64_t)b * a.s_k[0] + (int64_t)kvh * a.s_k[1] + (int64_t)krow * a.s_k[2];
+    const uint16_t* Vp = (const uint16_t*)a.v + (int64_t)b * a.s_v[0] + (int64_t)kvh * a.s_v[1] + (int64_t)krow * a.s_v[2];
+    bf16x8_t kf[KS], vf[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        kf[ks] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(Kp + 16 * ks + 8 * h));
+        vf[ks] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(Vp + 16 * ks + 8 * h));
+    }
+    f32x16_t acck[DB], accv[DB];
+#pragma unroll
+    for (int i = 0; i < DB; ++i)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) acck[i][j] = accv[i][j] = 0.f;
+
+    const int qt_begin_wg = a.causal ? (kt * kBQ) / kBT : 0;
+    const int n_qt = (a.N + kBT - 1) / kBT;
+    const int q_begin_wave = a.causal ? key0 : 0;
+
+    for (int r = 0; r < a.n_rep; ++r) {
+        const int hq = kvh * a.n_rep + r;
+        const uint16_t* Qp = (const uint16_t*)a.q + (int64_t)b * a.s_q[0] + (int64_t)hq * a.s_q[1];
+        const uint16_t* Op = (const uint16_t*)a.dout + (int64_t)b * a.s_do[0] + (int64_t)hq * a.s_do[1];
+        const float* Lp = a.lse + (int64_t)b * a.s_l[0] + (int64_t)hq * a.s_l[1];
+        const float* Dp = a.delta + ((int64_t)b * a.Hq + hq) * a.N;
+        for (int qt = qt_begin_wg; qt < n_qt; ++qt) {
+            __syncthreads();
+            fill_tile<D, P>(sQ, Qp, a.s_q[2], qt * kBT, a.N, tid);
+            fill_tile<D, P>(sO, Op, a.s_do[2], qt * kBT, a.N, tid);
+            if (tid < kBT) {
+                const int qi = qt * kBT + tid;
+                sL[tid] = qi < a.N ? Lp[(int64_t)qi * a.s_l[2]] : 0.f;
+                sD[tid] = qi < a.N ? Dp[qi] : 0.f;
+            }
+            __syncthreads();
+            const int qb = qt * kBT;
+            if (key0 >= a.N || qb + kBT - 1 < q_begin_wave) continue;
+            f32x16_t s, dp;
+#pragma unroll
+            for (int j = 0; j < 16; ++j) s[j] = dp[j] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const bf16x8_t qa = __builtin_bit_cast(bf16x8_t, *(const uint4*)(sQ + kl * P + 16 * ks + 8 * h));
+                const bf16x8_t oa = __builtin_bit_cast(bf16x8_t, *(const uint4*)(sO + kl * P + 16 * ks + 8 * h));
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kf[ks], s, 0, 0, 0);
+                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(oa, vf[ks], dp, 0, 0, 0);
+            }
+            uint32_t pw[2][4], dsw[2][4];
+#pragma unroll
+            for (int v = 0; v < 16; v += 2) {
+                float p2[2], d2[2];
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const int row = 8 * ((v + u) >> 2) + 4 * h + ((v + u) & 3);
+                    const int qi = qb + row;
+                    const bool ok = qi < a.N && ki < a.N && (!a.causal || ki <= qi);
+                    p2[u] = ok ? expf(s[v + u] * a.scale - sL[row]) : 0.f;
+                    d2[u] = p2[u] * (dp[v + u] - sD[row]);
+                }
+                pw[v >> 3][(v & 7) >> 1] = pack_bf16x2(p2[0], p2[1]);
+                dsw[v >> 3][(v & 7) >> 1] = pack_bf16x2(d2[0], d2[1]);
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, uint4{pw[j][0], pw[j][1], pw[j][2], pw[j][3]});
+                const bf16x8_t dsf = __builtin_bit_cast(bf16x8_t, uint4{dsw[j][0], dsw[j][1], dsw[j][2], dsw[j][3]});
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    accv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_transposed<P>(sO, j, db, lane), pf, accv[db], 0, 0, 0);
+                    acck[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_transposed<P>(sQ, j, db, lane), dsf, acck[db], 0, 0, 0);
+                }
+            }
+        }
+    }
+    if (ki < a.N) {
+        uint16_t* pk = (uint16_t*)a.dk + (int64_t)b * a.s_dk[0] + (int64_t)kvh * a.s_dk[1] + (int64_t)ki * a.s_dk[2];
+        uint16_t* pv = (uint16_t*)a.dv + (int64_t)b * a.s_dv[0] + (int64_t)kvh * a.s_dv[1] + (int64_t)ki * a.s_dv[2];
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int vq = 0; vq < 4; ++vq) {
+                const int d = 32 * db + 8 * vq + 4 * h;
+                uint2 wk, wv;
+                wk.x = pack_bf16x2(a.scale * acck[db][4 * vq], a.scale * acck[db][4 * vq + 1]);
+                wk.y = pack_bf16x2(a.scale * acck[db][4 * vq + 2], a.scale * acck[db][4 * vq + 3]);
+                wv.x = pack_bf16x2(accv[db][4 * vq], accv[db][4 * vq + 1]);
+                wv.y = pack_bf16x2(accv[db][4 * vq + 2], accv[db][4 * vq + 3]);
+                *(uint2*)(pk + d) = wk;
+                *(uint2*)(pv + d) = wv;
+            }
+    }
+}
+
 int check4(const vsp_tensor* t, int64_t B, int64_t H, int64_t N, int64_t D, int dtype) {
     if (!t) return VSP_ERR_NULL;
     if (t->ndim != 4) return VSP_ERR_NDIM;
@@ -284,6 +515,16 @@ int launch_backward(const BwdArgs& a, int64_t D, hipStream_t st) {
     if (rc != VSP_OK) return rc;
     const int64_t tiles = ceil_div(a.N, kBQ);
     const dim3 gq((unsigned)(tiles * a.B * a.Hq)), gk((unsigned)(tiles * a.B * a.Hkv));
+    if constexpr (sizeof(T) == 2) {
+        if (D == 128) {
+            hipLaunchKernelGGL(bwd_dq_bf16_kernel<128>, gq, dim3(256), 0, st, a);
+            hipLaunchKernelGGL(bwd_dkdv_bf16_kernel<128>, gk, dim3(256), 0, st, a);
+        } else {
+            hipLaunchKernelGGL(bwd_dq_bf16_kernel<64>, gq, dim3(256), 0, st, a);
+            hipLaunchKernelGGL(bwd_dkdv_bf16_kernel<64>, gk, dim3(256), 0, st, a);
+        }
+        return check_launch();
+    }
     if (D == 128) {
         hipLaunchKernelGGL((bwd_dq_kernel<128, T>), gq, dim3(256), 0, st, a);
         hipLaunchKernelGGL((bwd_dkdv_kernel<128, T>), gk, dim3(256), 0, st, a);
@@ -330,6 +571,13 @@ extern "C" int vsp_attn_prefill_backward(const vsp_tensor* dout, const vsp_tenso
     if (N > INT32_MAX / 2) return VSP_ERR_ARG;
     if (!workspace || workspace_bytes < vsp_attn_backward_workspace_bytes((int32_t)B, (int32_t)Hq, (int32_t)N)) return VSP_ERR_WORKSPACE;
     if (((uintptr_t)workspace & 3) != 0) return VSP_ERR_ALIGN;
+    if (dt == VSP_BF16) {  // 16-byte row segments are moved whole
+        for (const vsp_tensor* t : {dout, q, k, v, (const vsp_tensor*)dq, (const vsp_tensor*)dk, (const vsp_tensor*)dv}) {
+            if (!is_aligned16(t->data)) return VSP_ERR_ALIGN;
+            for (int i = 0; i < 3; ++i)
+                if ((t->stride[i] * 2) % 16 != 0) return VSP_ERR_ALIGN;
+        }
+    }
 
     BwdArgs a{};
     a.dout = dout->data;
