@@ -274,34 +274,70 @@ __global__ void __launch_bounds__(256) bwd_dkdv_kernel(BwdArgs a) {
 // =============================================================================================
 typedef short s16x4b_t __attribute__((ext_vector_type(4)));
 
-__device__ inline uint2 lds_tr16(const uint16_t* p) {
+// ---- a [32][D] bf16 tile in LDS ----
+// Rows are dense (2 D bytes); the 16-byte chunks of a row are permuted by an XOR that depends on the row, chosen
+// so that both access patterns the kernels use are free of bank conflicts: 16 lanes reading the same chunk of
+// 16 consecutive rows (the row-major MFMA operand), and a 4-row x 64-byte block (the transposing read).
+template <int D>
+__device__ inline int tile_off(int row, int chunk) {
+    const int f = D == 128 ? (((row & 3) << 2) | ((row >> 2) & 3)) : ((((row >> 1) & 1) << 2) | ((row >> 2) & 3));
+    return row * (2 * D) + ((chunk ^ f) << 4);
+}
+// MFMA operand, contraction over the row's elements: lane (row r = lane % 32, half h) takes elements 16 ks + 8 h ..
+template <int D>
+__device__ inline bf16x8_t load_row(const uint16_t* tile, int ks, int lane) {
+    return __builtin_bit_cast(bf16x8_t, *(const uint4*)((const char*)tile + tile_off<D>(lane & 31, 2 * ks + (lane >> 5))));
+}
+__device__ inline uint2 lds_tr16(const char* p) {
     s16x4b_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4b_t*)p);
     return __builtin_bit_cast(uint2, v);
 }
-// A operand [32 rows d][16 contraction slots] of the transposed tile: contraction slot (h, e) of k-step j is tile
-// row 16 j + 8 (e / 4) + 4 h + e % 4, the row the accumulator register 8 j + e of this lane half belongs to.
-template <int P>
+// MFMA operand, contraction over the tile's rows: lane (column 32 db + lane % 32, half h) takes, as slot e of
+// k-step j, row 16 j + 8 (e / 4) + 4 h + e % 4 - the row that accumulator register 8 j + e of this lane half
+// belongs to, so a product's result feeds the next product without leaving the lane.
+template <int D>
 __device__ inline bf16x8_t load_transposed(const uint16_t* tile, int j, int db, int lane) {
-    const int h = lane >> 5, i16 = lane & 15;
-    const uint16_t* p = tile + (16 * j + 4 * h + (i16 >> 2)) * P + 32 * db + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-    const uint2 lo = lds_tr16(p), hi = lds_tr16(p + 8 * P);
+    const int h = lane >> 5, row = 16 * j + 4 * h + ((lane & 15) >> 2);
+    const int chunk = 4 * db + 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1), o8 = (lane & 1) * 8;
+    const uint2 lo = lds_tr16((const char*)tile + tile_off<D>(row, chunk) + o8);
+    const uint2 hi = lds_tr16((const char*)tile + tile_off<D>(row + 8, chunk) + o8);
     return __builtin_bit_cast(bf16x8_t, uint4{lo.x, lo.y, hi.x, hi.y});
 }
-template <int D, int P>
-__device__ inline void fill_tile(uint16_t* dst, const uint16_t* src, int64_t row_stride, int row0, int n_rows, int tid) {
+// A tile in flight between global memory and LDS: fetched into registers one iteration ahead, committed to the
+// idle LDS buffer after the barrier, so the global latency is covered by the MFMAs of the current tile.
+template <int D>
+struct TileRegs {
+    static constexpr int N = (kBT * D / 8 + 255) / 256;
+    uint4 w[N];
+};
+template <int D>
+__device__ inline void tile_fetch(TileRegs<D>& r, const uint16_t* src, int64_t row_stride, int row0, int n_rows, int tid) {
     constexpr int CPR = D / 8;
-    for (int c = tid; c < kBT * CPR; c += 256) {
-        const int row = c / CPR, col = c % CPR;
-        const uint4 w = row0 + row < n_rows ? *(const uint4*)(src + (int64_t)(row0 + row) * row_stride + 8 * col) : uint4{0, 0, 0, 0};
-        *(uint4*)(dst + row * P + 8 * col) = w;
+#pragma unroll
+    for (int i = 0; i < TileRegs<D>::N; ++i) {
+        const int c = tid + 256 * i, row = c / CPR, col = c % CPR;
+        r.w[i] = (c < kBT * CPR && row0 + row < n_rows) ? *(const uint4*)(src + (int64_t)(row0 + row) * row_stride + 8 * col)
+                                                        : uint4{0, 0, 0, 0};
+    }
+}
+template <int D>
+__device__ inline void tile_commit(uint16_t* dst, const TileRegs<D>& r, int tid) {
+    constexpr int CPR = D / 8;
+#pragma unroll
+    for (int i = 0; i < TileRegs<D>::N; ++i) {
+        const int c = tid + 256 * i;
+        if (c < kBT * CPR) *(uint4*)((char*)dst + tile_off<D>(c / CPR, c % CPR)) = r.w[i];
     }
 }
 
+constexpr float kLog2e = 1.4426950408889634f;
+
+// ---- dQ (bf16): the structure of bwd_dq_kernel; K serves both as rows (S^T) and transposed (dQ^T) ----
 template <int D>
-__global__ void __launch_bounds__(256) bwd_dq_bf16_kernel(BwdArgs a) {
-    constexpr int KS = D / 16, DB = D / 32, P = D + 8;
-    __shared__ __attribute__((aligned(16))) uint16_t sK[kBT * P];
-    __shared__ __attribute__((aligned(16))) uint16_t sV[kBT * P];
+__global__ void __launch_bounds__(256, 2) bwd_dq_bf16_kernel(BwdArgs a) {
+    constexpr int KS = D / 16, DB = D / 32;
+    __shared__ __attribute__((aligned(16))) uint16_t sK[2][kBT * D];
+    __shared__ __attribute__((aligned(16))) uint16_t sV[2][kBT * D];
     const int n_qtiles = (a.N + kBQ - 1) / kBQ;
     const int bid = blockIdx.x;
     const int qt = n_qtiles - 1 - bid / (a.B * a.Hq);
@@ -323,13 +359,15 @@ __global__ void __launch_bounds__(256) bwd_dq_bf16_kernel(BwdArgs a) {
         qf[ks] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(Qp + 16 * ks + 8 * h));
         dof[ks] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(Op + 16 * ks + 8 * h));
     }
-    const float lse_q = a.lse[(int64_t)b * a.s_l[0] + (int64_t)hq * a.s_l[1] + (int64_t)qrow * a.s_l[2]];
+    const float lse_q = kLog2e * a.lse[(int64_t)b * a.s_l[0] + (int64_t)hq * a.s_l[1] + (int64_t)qrow * a.s_l[2]];
     const float di_q = a.delta[((int64_t)b * a.Hq + hq) * a.N + qrow];
+    const float scale_log2 = a.scale * kLog2e;
 
     const int wg_qmax = min(qt * kBQ + kBQ - 1, a.N - 1);
     const int kv_end_wg = a.causal ? min(a.N, wg_qmax + 1) : a.N;
     const int n_tiles = (kv_end_wg + kBT - 1) / kBT;
     const int kv_end_wave = (q0 < a.N) ? (a.causal ? min(a.N, min(q0 + 31, a.N - 1) + 1) : a.N) : 0;
+    const int lim = a.causal ? min(qi, a.N - 1) : a.N - 1;
 
     f32x16_t acc[DB];
 #pragma unroll
@@ -337,24 +375,37 @@ __global__ void __launch_bounds__(256) bwd_dq_bf16_kernel(BwdArgs a) {
 #pragma unroll
         for (int j = 0; j < 16; ++j) acc[i][j] = 0.f;
 
+    TileRegs<D> rk, rv;
+    tile_fetch<D>(rk, Kp, a.s_k[2], 0, a.N, tid);
+    tile_fetch<D>(rv, Vp, a.s_v[2], 0, a.N, tid);
+    tile_commit<D>(sK[0], rk, tid);
+    tile_commit<D>(sV[0], rv, tid);
+    if (n_tiles > 1) {
+        tile_fetch<D>(rk, Kp, a.s_k[2], kBT, a.N, tid);
+        tile_fetch<D>(rv, Vp, a.s_v[2], kBT, a.N, tid);
+    }
     for (int kt = 0; kt < n_tiles; ++kt) {
-        __syncthreads();
-        fill_tile<D, P>(sK, Kp, a.s_k[2], kt * kBT, a.N, tid);
-        fill_tile<D, P>(sV, Vp, a.s_v[2], kt * kBT, a.N, tid);
-        __syncthreads();
+        __syncthreads();   // tile kt is visible; every wavefront has left tile kt - 1, whose buffer is refilled now
+        if (kt + 1 < n_tiles) {
+            tile_commit<D>(sK[(kt + 1) & 1], rk, tid);
+            tile_commit<D>(sV[(kt + 1) & 1], rv, tid);
+            if (kt + 2 < n_tiles) {
+                tile_fetch<D>(rk, Kp, a.s_k[2], (kt + 2) * kBT, a.N, tid);
+                tile_fetch<D>(rv, Vp, a.s_v[2], (kt + 2) * kBT, a.N, tid);
+            }
+        }
         const int k0 = kt * kBT;
         if (k0 >= kv_end_wave) continue;
+        const uint16_t* tK = sK[kt & 1];
+        const uint16_t* tV = sV[kt & 1];
         f32x16_t s, dp;
 #pragma unroll
         for (int j = 0; j < 16; ++j) s[j] = dp[j] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            const bf16x8_t kf = __builtin_bit_cast(bf16x8_t, *(const uint4*)(sK + ql * P + 16 * ks + 8 * h));
-            const bf16x8_t vf = __builtin_bit_cast(bf16x8_t, *(const uint4*)(sV + ql * P + 16 * ks + 8 * h));
-            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], s, 0, 0, 0);
-            dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, dof[ks], dp, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_row<D>(tK, ks, lane), qf[ks], s, 0, 0, 0);
+            dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_row<D>(tV, ks, lane), dof[ks], dp, 0, 0, 0);
         }
-        const int lim = a.causal ? min(qi, a.N - 1) : a.N - 1;
         uint32_t dsw[2][4];
 #pragma unroll
         for (int v = 0; v < 16; v += 2) {
@@ -362,8 +413,8 @@ __global__ void __launch_bounds__(256) bwd_dq_bf16_kernel(BwdArgs a) {
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
                 const int key = k0 + 8 * ((v + u) >> 2) + 4 * h + ((v + u) & 3);
-                const float p = key <= lim ? expf(s[v + u] * a.scale - lse_q) : 0.f;
-                d2[u] = p * (dp[v + u] - di_q);
+                const float p = __builtin_amdgcn_exp2f(s[v + u] * scale_log2 - lse_q);
+                d2[u] = key <= lim ? p * (dp[v + u] - di_q) : 0.f;
             }
             dsw[v >> 3][(v & 7) >> 1] = pack_bf16x2(d2[0], d2[1]);
         }
@@ -372,7 +423,7 @@ __global__ void __launch_bounds__(256) bwd_dq_bf16_kernel(BwdArgs a) {
             const bf16x8_t dsf = __builtin_bit_cast(bf16x8_t, uint4{dsw[j][0], dsw[j][1], dsw[j][2], dsw[j][3]});
 #pragma unroll
             for (int db = 0; db < DB; ++db)
-                acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_transposed<P>(sK, j, db, lane), dsf, acc[db], 0, 0, 0);
+                acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_transposed<D>(tK, j, db, lane), dsf, acc[db], 0, 0, 0);
         }
     }
     if (qi < a.N) {
@@ -389,110 +440,150 @@ __global__ void __launch_bounds__(256) bwd_dq_bf16_kernel(BwdArgs a) {
     }
 }
 
+// ---- dK, dV (bf16) ----
+// A workgroup owns 64 key rows of one kv head: two blocks of 32, each worked by a pair of wavefronts that share
+// the arithmetic of a (query tile, key block) step by product instead of by rows, which halves what each has to
+// keep in registers (one of K / V, one of dK / dV):
+//   wavefront P:  S = Q K^T  ->  P = exp2(..)  -> hands P (bf16) to its partner through LDS  ->  dV^T += dO^T P
+//   wavefront D:  dP = dO V^T                  ->  takes P  ->  dS = P (dP - Di)              ->  dK^T += Q^T dS
+// Both see the same accumulator layout, so lane l of one reads exactly the words lane l of the other wrote.
+constexpr int kBK = 64;   // key rows per workgroup in the bf16 dK / dV pass
+
 template <int D>
-__global__ void __launch_bounds__(256) bwd_dkdv_bf16_kernel(BwdArgs a) {
-    constexpr int KS = D / 16, DB = D / 32, P = D + 8;
-    __shared__ __attribute__((aligned(16))) uint16_t sQ[kBT * P];
-    __shared__ __attribute__((aligned(16))) uint16_t sO[kBT * P];
-    __shared__ float sL[kBT], sD[kBT];
+__global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
+    constexpr int KS = D / 16, DB = D / 32;
+    __shared__ __attribute__((aligned(16))) uint16_t sQ[2][kBT * D];
+    __shared__ __attribute__((aligned(16))) uint16_t sO[2][kBT * D];
+    __shared__ __attribute__((aligned(16))) float sL[2][kBT];
+    __shared__ __attribute__((aligned(16))) float sD[2][kBT];
+    __shared__ __attribute__((aligned(16))) uint32_t sP[2][8][64];   // [key block][word][lane]
     const int bid = blockIdx.x;
-    const int kt = bid / (a.B * a.Hkv);
+    const int kt = bid / (a.B * a.Hkv);          // causal work falls with the key tile: heaviest first
     const int bh = bid % (a.B * a.Hkv);
     const int b = bh / a.Hkv, kvh = bh % a.Hkv;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kb = wave >> 1;
+    const bool role_d = wave & 1;
     const int kl = lane & 31, h = lane >> 5;
-    const int key0 = kt * kBQ + wave * 32;
+    const int key0 = kt * kBK + kb * 32;
     const int ki = key0 + kl;
     const int krow = min(ki, a.N - 1);
 
-    const uint16_t* Kp = (const uint16_t*)a.k + (int64_t)b * a.s_k[0] + (int64_t)kvh * a.s_k[1] + (int64_t)krow * a.s_k[2];
-    const uint16_t* Vp = (const uint16_t*)a.v + (int64_t)b * a.s_v[0] + (int64_t)kvh * a.s_v[1] + (int64_t)krow * a.s_v[2];
-    bf16x8_t kf[KS], vf[KS];
+    // the stationary operand: K rows for the P wavefront, V rows for the D wavefront
+    const uint16_t* Xp = role_d ? (const uint16_t*)a.v + (int64_t)b * a.s_v[0] + (int64_t)kvh * a.s_v[1] + (int64_t)krow * a.s_v[2]
+                                : (const uint16_t*)a.k + (int64_t)b * a.s_k[0] + (int64_t)kvh * a.s_k[1] + (int64_t)krow * a.s_k[2];
+    bf16x8_t xf[KS];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-        kf[ks] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(Kp + 16 * ks + 8 * h));
-        vf[ks] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(Vp + 16 * ks + 8 * h));
-    }
-    f32x16_t acck[DB], accv[DB];
+    for (int ks = 0; ks < KS; ++ks) xf[ks] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(Xp + 16 * ks + 8 * h));
+    f32x16_t acc[DB];
 #pragma unroll
     for (int i = 0; i < DB; ++i)
 #pragma unroll
-        for (int j = 0; j < 16; ++j) acck[i][j] = accv[i][j] = 0.f;
+        for (int j = 0; j < 16; ++j) acc[i][j] = 0.f;
 
-    const int qt_begin_wg = a.causal ? (kt * kBQ) / kBT : 0;
-    const int n_qt = (a.N + kBT - 1) / kBT;
-    const int q_begin_wave = a.causal ? key0 : 0;
+    const int qt_begin = a.causal ? (kt * kBK) / kBT : 0;
+    const int n_qt = (a.N + kBT - 1) / kBT - qt_begin;   // query tiles per head
+    const int n_it = a.n_rep * n_qt;                     // the loop runs over (head of the group, query tile)
+    const float scale_log2 = a.scale * kLog2e;
 
-    for (int r = 0; r < a.n_rep; ++r) {
-        const int hq = kvh * a.n_rep + r;
-        const uint16_t* Qp = (const uint16_t*)a.q + (int64_t)b * a.s_q[0] + (int64_t)hq * a.s_q[1];
-        const uint16_t* Op = (const uint16_t*)a.dout + (int64_t)b * a.s_do[0] + (int64_t)hq * a.s_do[1];
-        const float* Lp = a.lse + (int64_t)b * a.s_l[0] + (int64_t)hq * a.s_l[1];
-        const float* Dp = a.delta + ((int64_t)b * a.Hq + hq) * a.N;
-        for (int qt = qt_begin_wg; qt < n_qt; ++qt) {
-            __syncthreads();
-            fill_tile<D, P>(sQ, Qp, a.s_q[2], qt * kBT, a.N, tid);
-            fill_tile<D, P>(sO, Op, a.s_do[2], qt * kBT, a.N, tid);
-            if (tid < kBT) {
-                const int qi = qt * kBT + tid;
-                sL[tid] = qi < a.N ? Lp[(int64_t)qi * a.s_l[2]] : 0.f;
-                sD[tid] = qi < a.N ? Dp[qi] : 0.f;
-            }
-            __syncthreads();
-            const int qb = qt * kBT;
-            if (key0 >= a.N || qb + kBT - 1 < q_begin_wave) continue;
-            f32x16_t s, dp;
+    TileRegs<D> rq, ro;
+    float rl = 0.f, rd = 0.f;
+    auto fetch = [&](int it) {
+        const int hq = kvh * a.n_rep + it / n_qt, qb = (qt_begin + it % n_qt) * kBT;
+        tile_fetch<D>(rq, (const uint16_t*)a.q + (int64_t)b * a.s_q[0] + (int64_t)hq * a.s_q[1], a.s_q[2], qb, a.N, tid);
+        tile_fetch<D>(ro, (const uint16_t*)a.dout + (int64_t)b * a.s_do[0] + (int64_t)hq * a.s_do[1], a.s_do[2], qb, a.N, tid);
+        if (tid < kBT) {
+            const int qi = min(qb + tid, a.N - 1);
+            rl = kLog2e * a.lse[(int64_t)b * a.s_l[0] + (int64_t)hq * a.s_l[1] + (int64_t)qi * a.s_l[2]];
+            rd = a.delta[((int64_t)b * a.Hq + hq) * a.N + qi];
+        }
+    };
+    auto commit = [&](int buf) {
+        tile_commit<D>(sQ[buf], rq, tid);
+        tile_commit<D>(sO[buf], ro, tid);
+        if (tid < kBT) {
+            sL[buf][tid] = rl;
+            sD[buf][tid] = rd;
+        }
+    };
+    fetch(0);
+    commit(0);
+    if (n_it > 1) fetch(1);
+    for (int it = 0; it < n_it; ++it) {
+        __syncthreads();   // tile `it` is visible; every wavefront has left tile it - 1, whose buffer is refilled now
+        if (it + 1 < n_it) {
+            commit((it + 1) & 1);
+            if (it + 2 < n_it) fetch(it + 2);
+        }
+        const int qb = (qt_begin + it % n_qt) * kBT;
+        const bool live = key0 < a.N && !(a.causal && qb + kBT - 1 < key0);   // same for both wavefronts of a pair
+        const uint16_t* tQ = sQ[it & 1];
+        const uint16_t* tO = sO[it & 1];
+        f32x16_t s;
+        uint32_t pw[2][4];
+        if (live) {
+            const uint16_t* rows = role_d ? tO : tQ;
 #pragma unroll
-            for (int j = 0; j < 16; ++j) s[j] = dp[j] = 0.f;
+            for (int j = 0; j < 16; ++j) s[j] = 0.f;
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                const bf16x8_t qa = __builtin_bit_cast(bf16x8_t, *(const uint4*)(sQ + kl * P + 16 * ks + 8 * h));
-                const bf16x8_t oa = __builtin_bit_cast(bf16x8_t, *(const uint4*)(sO + kl * P + 16 * ks + 8 * h));
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kf[ks], s, 0, 0, 0);
-                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(oa, vf[ks], dp, 0, 0, 0);
-            }
-            uint32_t pw[2][4], dsw[2][4];
+            for (int ks = 0; ks < KS; ++ks)
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_row<D>(rows, ks, lane), xf[ks], s, 0, 0, 0);
+            if (!role_d) {
+                float lq[16];
 #pragma unroll
-            for (int v = 0; v < 16; v += 2) {
-                float p2[2], d2[2];
+                for (int g = 0; g < 4; ++g) *(float4*)&lq[4 * g] = *(const float4*)&sL[it & 1][8 * g + 4 * h];
 #pragma unroll
-                for (int u = 0; u < 2; ++u) {
-                    const int row = 8 * ((v + u) >> 2) + 4 * h + ((v + u) & 3);
-                    const int qi = qb + row;
-                    const bool ok = qi < a.N && ki < a.N && (!a.causal || ki <= qi);
-                    p2[u] = ok ? expf(s[v + u] * a.scale - sL[row]) : 0.f;
-                    d2[u] = p2[u] * (dp[v + u] - sD[row]);
+                for (int v = 0; v < 16; v += 2) {
+                    float p2[2];
+#pragma unroll
+                    for (int u = 0; u < 2; ++u) {
+                        const int qi = qb + 8 * ((v + u) >> 2) + 4 * h + ((v + u) & 3);
+                        const float e = __builtin_amdgcn_exp2f(s[v + u] * scale_log2 - lq[v + u]);
+                        p2[u] = (qi < a.N && ki < a.N && (!a.causal || ki <= qi)) ? e : 0.f;
+                    }
+                    pw[v >> 3][(v & 7) >> 1] = pack_bf16x2(p2[0], p2[1]);
                 }
-                pw[v >> 3][(v & 7) >> 1] = pack_bf16x2(p2[0], p2[1]);
-                dsw[v >> 3][(v & 7) >> 1] = pack_bf16x2(d2[0], d2[1]);
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) sP[kb][4 * j + w][lane] = pw[j][w];
             }
+        }
+        __syncthreads();   // P of this step is in LDS
+        if (live) {
+            if (role_d) {
+                float dq_[16];
+#pragma unroll
+                for (int g = 0; g < 4; ++g) *(float4*)&dq_[4 * g] = *(const float4*)&sD[it & 1][8 * g + 4 * h];
+#pragma unroll
+                for (int v = 0; v < 16; v += 2) {
+                    const uint32_t w = sP[kb][v >> 1][lane];
+                    const float p0 = __uint_as_float(w << 16), p1 = __uint_as_float(w & 0xffff0000u);
+                    pw[v >> 3][(v & 7) >> 1] = pack_bf16x2(p0 * (s[v] - dq_[v]), p1 * (s[v + 1] - dq_[v + 1]));
+                }
+            }
+            const uint16_t* cols = role_d ? tQ : tO;
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, uint4{pw[j][0], pw[j][1], pw[j][2], pw[j][3]});
-                const bf16x8_t dsf = __builtin_bit_cast(bf16x8_t, uint4{dsw[j][0], dsw[j][1], dsw[j][2], dsw[j][3]});
+                const bf16x8_t bf = __builtin_bit_cast(bf16x8_t, uint4{pw[j][0], pw[j][1], pw[j][2], pw[j][3]});
 #pragma unroll
-                for (int db = 0; db < DB; ++db) {
-                    accv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_transposed<P>(sO, j, db, lane), pf, accv[db], 0, 0, 0);
-                    acck[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_transposed<P>(sQ, j, db, lane), dsf, acck[db], 0, 0, 0);
-                }
+                for (int db = 0; db < DB; ++db)
+                    acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_transposed<D>(cols, j, db, lane), bf, acc[db], 0, 0, 0);
             }
         }
     }
     if (ki < a.N) {
-        uint16_t* pk = (uint16_t*)a.dk + (int64_t)b * a.s_dk[0] + (int64_t)kvh * a.s_dk[1] + (int64_t)ki * a.s_dk[2];
-        uint16_t* pv = (uint16_t*)a.dv + (int64_t)b * a.s_dv[0] + (int64_t)kvh * a.s_dv[1] + (int64_t)ki * a.s_dv[2];
+        const float f = role_d ? a.scale : 1.f;
+        uint16_t* po = role_d ? (uint16_t*)a.dk + (int64_t)b * a.s_dk[0] + (int64_t)kvh * a.s_dk[1] + (int64_t)ki * a.s_dk[2]
+                              : (uint16_t*)a.dv + (int64_t)b * a.s_dv[0] + (int64_t)kvh * a.s_dv[1] + (int64_t)ki * a.s_dv[2];
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll
             for (int vq = 0; vq < 4; ++vq) {
-                const int d = 32 * db + 8 * vq + 4 * h;
-                uint2 wk, wv;
-                wk.x = pack_bf16x2(a.scale * acck[db][4 * vq], a.scale * acck[db][4 * vq + 1]);
-                wk.y = pack_bf16x2(a.scale * acck[db][4 * vq + 2], a.scale * acck[db][4 * vq + 3]);
-                wv.x = pack_bf16x2(accv[db][4 * vq], accv[db][4 * vq + 1]);
-                wv.y = pack_bf16x2(accv[db][4 * vq + 2], accv[db][4 * vq + 3]);
-                *(uint2*)(pk + d) = wk;
-                *(uint2*)(pv + d) = wv;
+                uint2 w;
+                w.x = pack_bf16x2(f * acc[db][4 * vq], f * acc[db][4 * vq + 1]);
+                w.y = pack_bf16x2(f * acc[db][4 * vq + 2], f * acc[db][4 * vq + 3]);
+                *(uint2*)(po + 32 * db + 8 * vq + 4 * h) = w;
             }
     }
 }
@@ -516,6 +607,7 @@ int launch_backward(const BwdArgs& a, int64_t D, hipStream_t st) {
     const int64_t tiles = ceil_div(a.N, kBQ);
     const dim3 gq((unsigned)(tiles * a.B * a.Hq)), gk((unsigned)(tiles * a.B * a.Hkv));
     if constexpr (sizeof(T) == 2) {
+        const dim3 gk((unsigned)(ceil_div(a.N, kBK) * a.B * a.Hkv));
         if (D == 128) {
             hipLaunchKernelGGL(bwd_dq_bf16_kernel<128>, gq, dim3(256), 0, st, a);
             hipLaunchKernelGGL(bwd_dkdv_bf16_kernel<128>, gk, dim3(256), 0, st, a);
