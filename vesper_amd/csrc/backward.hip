@@ -273,16 +273,18 @@ __global__ void __launch_bounds__(256) bwd_dkdv_kernel(BwdArgs a) {
 // P / dS go from the accumulator registers into the next MFMA without leaving the lane.
 // =============================================================================================
 typedef short s16x4b_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
 // ---- a [32][D] bf16 tile in LDS ----
 // Rows are dense (2 D bytes); the 16-byte chunks of a row are permuted by an XOR that depends on the row, chosen
 // so that both access patterns the kernels use are free of bank conflicts: 16 lanes reading the same chunk of
 // 16 consecutive rows (the row-major MFMA operand), and a 4-row x 64-byte block (the transposing read).
 template <int D>
-__device__ inline int tile_off(int row, int chunk) {
-    const int f = D == 128 ? (((row & 3) << 2) | ((row >> 2) & 3)) : ((((row >> 1) & 1) << 2) | ((row >> 2) & 3));
-    return row * (2 * D) + ((chunk ^ f) << 4);
+__device__ inline int tile_swz(int row) {
+    return D == 128 ? (((row & 3) << 2) | ((row >> 2) & 3)) : ((((row >> 1) & 1) << 2) | ((row >> 2) & 3));
 }
+template <int D>
+__device__ inline int tile_off(int row, int chunk) { return row * (2 * D) + ((chunk ^ tile_swz<D>(row)) << 4); }
 // MFMA operand, contraction over the row's elements: lane (row r = lane % 32, half h) takes elements 16 ks + 8 h ..
 template <int D>
 __device__ inline bf16x8_t load_row(const uint16_t* tile, int ks, int lane) {
@@ -303,32 +305,33 @@ __device__ inline bf16x8_t load_transposed(const uint16_t* tile, int j, int db, 
     const uint2 hi = lds_tr16((const char*)tile + tile_off<D>(row + 8, chunk) + o8);
     return __builtin_bit_cast(bf16x8_t, uint4{lo.x, lo.y, hi.x, hi.y});
 }
-// A tile in flight between global memory and LDS: fetched into registers one iteration ahead, committed to the
-// idle LDS buffer after the barrier, so the global latency is covered by the MFMAs of the current tile.
+// Global -> LDS without passing through registers: a wavefront instruction moves 64 x 16 bytes to 1 KB of
+// consecutive LDS, so the lane that lands on (row, physical chunk) fetches the row's chunk `physical ^ swizzle`.
+// Rows at or past `valid_rows` fall outside the buffer descriptor's range and arrive as zeros.
 template <int D>
-struct TileRegs {
-    static constexpr int N = (kBT * D / 8 + 255) / 256;
-    uint4 w[N];
+struct TileDma {
+    static constexpr int CPR = D / 8, RPG = 64 / CPR, NLD = CPR / 8;   // chunks per row, rows per instruction, instructions per wavefront
+    uint32_t voff[NLD];
+    __device__ inline void init(int64_t row_stride, int wave, int lane) {
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int r = (wave + 4 * i) * RPG + lane / CPR;
+            voff[i] = (uint32_t)r * (uint32_t)row_stride * 2u + 16u * (uint32_t)((lane % CPR) ^ tile_swz<D>(r));
+        }
+    }
+    __device__ inline void load(uint16_t* dst, const uint16_t* row0, int valid_rows, int64_t row_stride, int wave) const {
+        __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)row0, 0, (int)((int64_t)max(valid_rows, 0) * row_stride * 2), 0x00020000);
+#pragma unroll
+        for (int i = 0; i < NLD; ++i)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)((char*)dst + (wave + 4 * i) * 1024), 16, voff[i], 0, 0, 0);
+    }
 };
-template <int D>
-__device__ inline void tile_fetch(TileRegs<D>& r, const uint16_t* src, int64_t row_stride, int row0, int n_rows, int tid) {
-    constexpr int CPR = D / 8;
-#pragma unroll
-    for (int i = 0; i < TileRegs<D>::N; ++i) {
-        const int c = tid + 256 * i, row = c / CPR, col = c % CPR;
-        r.w[i] = (c < kBT * CPR && row0 + row < n_rows) ? *(const uint4*)(src + (int64_t)(row0 + row) * row_stride + 8 * col)
-                                                        : uint4{0, 0, 0, 0};
-    }
+// One float per lane (element stride `stride`) to 64 consecutive LDS words; lanes at or past `valid` bring zeros.
+__device__ inline void row_dma(float* dst, const float* src, int valid, int64_t stride, int lane) {
+    __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)src, 0, (int)((int64_t)valid * stride * 4), 0x00020000);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)dst, 4, (uint32_t)lane * (uint32_t)stride * 4u, 0, 0, 0);
 }
-template <int D>
-__device__ inline void tile_commit(uint16_t* dst, const TileRegs<D>& r, int tid) {
-    constexpr int CPR = D / 8;
-#pragma unroll
-    for (int i = 0; i < TileRegs<D>::N; ++i) {
-        const int c = tid + 256 * i;
-        if (c < kBT * CPR) *(uint4*)((char*)dst + tile_off<D>(c / CPR, c % CPR)) = r.w[i];
-    }
-}
+__device__ inline void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 constexpr float kLog2e = 1.4426950408889634f;
 
@@ -336,8 +339,8 @@ constexpr float kLog2e = 1.4426950408889634f;
 template <int D>
 __global__ void __launch_bounds__(256, 2) bwd_dq_bf16_kernel(BwdArgs a) {
     constexpr int KS = D / 16, DB = D / 32;
-    __shared__ __attribute__((aligned(16))) uint16_t sK[2][kBT * D];
-    __shared__ __attribute__((aligned(16))) uint16_t sV[2][kBT * D];
+    __shared__ __attribute__((aligned(1024))) uint16_t sK[2][kBT * D];
+    __shared__ __attribute__((aligned(1024))) uint16_t sV[2][kBT * D];
     const int n_qtiles = (a.N + kBQ - 1) / kBQ;
     const int bid = blockIdx.x;
     const int qt = n_qtiles - 1 - bid / (a.B * a.Hq);
@@ -375,25 +378,18 @@ __global__ void __launch_bounds__(256, 2) bwd_dq_bf16_kernel(BwdArgs a) {
 #pragma unroll
         for (int j = 0; j < 16; ++j) acc[i][j] = 0.f;
 
-    TileRegs<D> rk, rv;
-    tile_fetch<D>(rk, Kp, a.s_k[2], 0, a.N, tid);
-    tile_fetch<D>(rv, Vp, a.s_v[2], 0, a.N, tid);
-    tile_commit<D>(sK[0], rk, tid);
-    tile_commit<D>(sV[0], rv, tid);
-    if (n_tiles > 1) {
-        tile_fetch<D>(rk, Kp, a.s_k[2], kBT, a.N, tid);
-        tile_fetch<D>(rv, Vp, a.s_v[2], kBT, a.N, tid);
-    }
+    TileDma<D> dk_, dv_;
+    dk_.init(a.s_k[2], wave, lane);
+    dv_.init(a.s_v[2], wave, lane);
+    auto load = [&](int kt) {
+        dk_.load(sK[kt & 1], Kp + (int64_t)kt * kBT * a.s_k[2], a.N - kt * kBT, a.s_k[2], wave);
+        dv_.load(sV[kt & 1], Vp + (int64_t)kt * kBT * a.s_v[2], a.N - kt * kBT, a.s_v[2], wave);
+    };
+    load(0);
     for (int kt = 0; kt < n_tiles; ++kt) {
-        __syncthreads();   // tile kt is visible; every wavefront has left tile kt - 1, whose buffer is refilled now
-        if (kt + 1 < n_tiles) {
-            tile_commit<D>(sK[(kt + 1) & 1], rk, tid);
-            tile_commit<D>(sV[(kt + 1) & 1], rv, tid);
-            if (kt + 2 < n_tiles) {
-                tile_fetch<D>(rk, Kp, a.s_k[2], (kt + 2) * kBT, a.N, tid);
-                tile_fetch<D>(rv, Vp, a.s_v[2], (kt + 2) * kBT, a.N, tid);
-            }
-        }
+        dma_wait_all();
+        __syncthreads();   // tile kt is in LDS; every wavefront has left tile kt - 1, whose buffer is refilled now
+        if (kt + 1 < n_tiles) load(kt + 1);
         const int k0 = kt * kBT;
         if (k0 >= kv_end_wave) continue;
         const uint16_t* tK = sK[kt & 1];
@@ -444,19 +440,22 @@ __global__ void __launch_bounds__(256, 2) bwd_dq_bf16_kernel(BwdArgs a) {
 // A workgroup owns 64 key rows of one kv head: two blocks of 32, each worked by a pair of wavefronts that share
 // the arithmetic of a (query tile, key block) step by product instead of by rows, which halves what each has to
 // keep in registers (one of K / V, one of dK / dV):
-//   wavefront P:  S = Q K^T  ->  P = exp2(..)  -> hands P (bf16) to its partner through LDS  ->  dV^T += dO^T P
-//   wavefront D:  dP = dO V^T                  ->  takes P  ->  dS = P (dP - Di)              ->  dK^T += Q^T dS
+//   wavefront P:  S = Q K^T  ->  P = exp2(..)  ->  hands P (bf16) to its partner through LDS  ->  dV^T += dO^T P
+//   wavefront D:  dP = dO V^T                  ->  takes P  ->  dS = P (dP - Di)               ->  dK^T += Q^T dS
 // Both see the same accumulator layout, so lane l of one reads exactly the words lane l of the other wrote.
+// The two halves of a step are one iteration apart: while the second products of tile t run, the first products
+// of tile t + 1 are issued, and P(t + 1) crosses to the partner over the iteration's only barrier.  A tile is
+// therefore live for two iterations and the ring holds three.
 constexpr int kBK = 64;   // key rows per workgroup in the bf16 dK / dV pass
 
 template <int D>
 __global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
     constexpr int KS = D / 16, DB = D / 32;
-    __shared__ __attribute__((aligned(16))) uint16_t sQ[2][kBT * D];
-    __shared__ __attribute__((aligned(16))) uint16_t sO[2][kBT * D];
-    __shared__ __attribute__((aligned(16))) float sL[2][kBT];
-    __shared__ __attribute__((aligned(16))) float sD[2][kBT];
-    __shared__ __attribute__((aligned(16))) uint32_t sP[2][8][64];   // [key block][word][lane]
+    __shared__ __attribute__((aligned(1024))) uint16_t sQ[3][kBT * D];
+    __shared__ __attribute__((aligned(1024))) uint16_t sO[3][kBT * D];
+    __shared__ __attribute__((aligned(256))) float sL[3][64];      // lse and Di of the tile's rows (32 used; a wavefront
+    __shared__ __attribute__((aligned(256))) float sD[3][64];      // instruction fills 64 words)
+    __shared__ __attribute__((aligned(16))) uint32_t sP[2][2][8][64];   // [parity of the tile][key block][word][lane]
     const int bid = blockIdx.x;
     const int kt = bid / (a.B * a.Hkv);          // causal work falls with the key tile: heaviest first
     const int bh = bid % (a.B * a.Hkv);
@@ -486,91 +485,103 @@ __global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
     const int n_it = a.n_rep * n_qt;                     // the loop runs over (head of the group, query tile)
     const float scale_log2 = a.scale * kLog2e;
 
-    TileRegs<D> rq, ro;
-    float rl = 0.f, rd = 0.f;
-    auto fetch = [&](int it) {
+    TileDma<D> dq_, do_;
+    dq_.init(a.s_q[2], wave, lane);
+    do_.init(a.s_do[2], wave, lane);
+    auto load = [&](int it, int buf) {
         const int hq = kvh * a.n_rep + it / n_qt, qb = (qt_begin + it % n_qt) * kBT;
-        tile_fetch<D>(rq, (const uint16_t*)a.q + (int64_t)b * a.s_q[0] + (int64_t)hq * a.s_q[1], a.s_q[2], qb, a.N, tid);
-        tile_fetch<D>(ro, (const uint16_t*)a.dout + (int64_t)b * a.s_do[0] + (int64_t)hq * a.s_do[1], a.s_do[2], qb, a.N, tid);
-        if (tid < kBT) {
-            const int qi = min(qb + tid, a.N - 1);
-            rl = kLog2e * a.lse[(int64_t)b * a.s_l[0] + (int64_t)hq * a.s_l[1] + (int64_t)qi * a.s_l[2]];
-            rd = a.delta[((int64_t)b * a.Hq + hq) * a.N + qi];
+        dq_.load(sQ[buf], (const uint16_t*)a.q + (int64_t)b * a.s_q[0] + (int64_t)hq * a.s_q[1] + (int64_t)qb * a.s_q[2], a.N - qb,
+                 a.s_q[2], wave);
+        do_.load(sO[buf], (const uint16_t*)a.dout + (int64_t)b * a.s_do[0] + (int64_t)hq * a.s_do[1] + (int64_t)qb * a.s_do[2],
+                 a.N - qb, a.s_do[2], wave);
+        if (wave == 0)
+            row_dma(sL[buf], a.lse + (int64_t)b * a.s_l[0] + (int64_t)hq * a.s_l[1] + (int64_t)qb * a.s_l[2], min(a.N - qb, kBT), a.s_l[2], lane);
+        else if (wave == 1)
+            row_dma(sD[buf], a.delta + ((int64_t)b * a.Hq + hq) * a.N + qb, min(a.N - qb, kBT), 1, lane);
+    };
+    // first products of tile t: S (P wavefront) or dP (D wavefront) into s; the P wavefront goes on to P(t),
+    // packed into pw and posted for its partner.  Masked or out-of-range positions get P = 0, so a tile that lies
+    // wholly above the diagonal or past the end costs its MFMAs and contributes nothing.
+    auto first = [&](int t, int buf, f32x16_t& s, uint32_t (&pw)[2][4]) {
+        const uint16_t* rows = role_d ? sO[buf] : sQ[buf];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) s[j] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_row<D>(rows, ks, lane), xf[ks], s, 0, 0, 0);
+        if (!role_d) {
+            const int qb = (qt_begin + t % n_qt) * kBT;
+            float lq[16];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) *(float4*)&lq[4 * g] = *(const float4*)&sL[buf][8 * g + 4 * h];
+#pragma unroll
+            for (int v = 0; v < 16; v += 2) {
+                float p2[2];
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const int qi = qb + 8 * ((v + u) >> 2) + 4 * h + ((v + u) & 3);
+                    const float e = __builtin_amdgcn_exp2f(s[v + u] * scale_log2 - lq[v + u] * kLog2e);
+                    p2[u] = (qi < a.N && ki < a.N && (!a.causal || ki <= qi)) ? e : 0.f;
+                }
+                pw[v >> 3][(v & 7) >> 1] = pack_bf16x2(p2[0], p2[1]);
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int w = 0; w < 4; ++w) sP[t & 1][kb][4 * j + w][lane] = pw[j][w];
         }
     };
-    auto commit = [&](int buf) {
-        tile_commit<D>(sQ[buf], rq, tid);
-        tile_commit<D>(sO[buf], ro, tid);
-        if (tid < kBT) {
-            sL[buf][tid] = rl;
-            sD[buf][tid] = rd;
+    // second products of tile t: dV^T += dO^T P (P wavefront, P from its own registers) or
+    // dS = P (dP - Di), dK^T += Q^T dS (D wavefront, P from its partner)
+    auto second = [&](int t, int buf, const f32x16_t& s, uint32_t (&pw)[2][4]) {
+        if (role_d) {
+            float di[16];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) *(float4*)&di[4 * g] = *(const float4*)&sD[buf][8 * g + 4 * h];
+#pragma unroll
+            for (int v = 0; v < 16; v += 2) {
+                const uint32_t w = sP[t & 1][kb][v >> 1][lane];
+                const float p0 = __uint_as_float(w << 16), p1 = __uint_as_float(w & 0xffff0000u);
+                pw[v >> 3][(v & 7) >> 1] = pack_bf16x2(p0 * (s[v] - di[v]), p1 * (s[v + 1] - di[v + 1]));
+            }
+        }
+        const uint16_t* cols = role_d ? sQ[buf] : sO[buf];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const bf16x8_t bf = __builtin_bit_cast(bf16x8_t, uint4{pw[j][0], pw[j][1], pw[j][2], pw[j][3]});
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+                acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_transposed<D>(cols, j, db, lane), bf, acc[db], 0, 0, 0);
         }
     };
-    fetch(0);
-    commit(0);
-    if (n_it > 1) fetch(1);
+
+    f32x16_t s_cur, s_next;
+    uint32_t pw_cur[2][4], pw_next[2][4];
+    load(0, 0);
+    if (n_it > 1) load(1, 1);
+    dma_wait_all();
+    __syncthreads();
+    first(0, 0, s_cur, pw_cur);
+    int buf = 0;   // ring slot of tile `it`
     for (int it = 0; it < n_it; ++it) {
-        __syncthreads();   // tile `it` is visible; every wavefront has left tile it - 1, whose buffer is refilled now
+        // tile it + 1 and P(it) are in LDS; every wavefront has left tile it - 1, whose slot takes tile it + 2
+        dma_wait_all();
+        __syncthreads();
+        const int buf1 = buf == 2 ? 0 : buf + 1, buf2 = buf1 == 2 ? 0 : buf1 + 1;
+        if (it + 2 < n_it) load(it + 2, buf2);
         if (it + 1 < n_it) {
-            commit((it + 1) & 1);
-            if (it + 2 < n_it) fetch(it + 2);
+            // independent streams in one block: first products of the next tile, second products of this one
+            first(it + 1, buf1, s_next, pw_next);
+            second(it, buf, s_cur, pw_cur);
+            s_cur = s_next;
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int w = 0; w < 4; ++w) pw_cur[j][w] = pw_next[j][w];
+        } else {
+            second(it, buf, s_cur, pw_cur);
         }
-        const int qb = (qt_begin + it % n_qt) * kBT;
-        const bool live = key0 < a.N && !(a.causal && qb + kBT - 1 < key0);   // same for both wavefronts of a pair
-        const uint16_t* tQ = sQ[it & 1];
-        const uint16_t* tO = sO[it & 1];
-        f32x16_t s;
-        uint32_t pw[2][4];
-        if (live) {
-            const uint16_t* rows = role_d ? tO : tQ;
-#pragma unroll
-            for (int j = 0; j < 16; ++j) s[j] = 0.f;
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks)
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_row<D>(rows, ks, lane), xf[ks], s, 0, 0, 0);
-            if (!role_d) {
-                float lq[16];
-#pragma unroll
-                for (int g = 0; g < 4; ++g) *(float4*)&lq[4 * g] = *(const float4*)&sL[it & 1][8 * g + 4 * h];
-#pragma unroll
-                for (int v = 0; v < 16; v += 2) {
-                    float p2[2];
-#pragma unroll
-                    for (int u = 0; u < 2; ++u) {
-                        const int qi = qb + 8 * ((v + u) >> 2) + 4 * h + ((v + u) & 3);
-                        const float e = __builtin_amdgcn_exp2f(s[v + u] * scale_log2 - lq[v + u]);
-                        p2[u] = (qi < a.N && ki < a.N && (!a.causal || ki <= qi)) ? e : 0.f;
-                    }
-                    pw[v >> 3][(v & 7) >> 1] = pack_bf16x2(p2[0], p2[1]);
-                }
-#pragma unroll
-                for (int j = 0; j < 2; ++j)
-#pragma unroll
-                    for (int w = 0; w < 4; ++w) sP[kb][4 * j + w][lane] = pw[j][w];
-            }
-        }
-        __syncthreads();   // P of this step is in LDS
-        if (live) {
-            if (role_d) {
-                float dq_[16];
-#pragma unroll
-                for (int g = 0; g < 4; ++g) *(float4*)&dq_[4 * g] = *(const float4*)&sD[it & 1][8 * g + 4 * h];
-#pragma unroll
-                for (int v = 0; v < 16; v += 2) {
-                    const uint32_t w = sP[kb][v >> 1][lane];
-                    const float p0 = __uint_as_float(w << 16), p1 = __uint_as_float(w & 0xffff0000u);
-                    pw[v >> 3][(v & 7) >> 1] = pack_bf16x2(p0 * (s[v] - dq_[v]), p1 * (s[v + 1] - dq_[v + 1]));
-                }
-            }
-            const uint16_t* cols = role_d ? tQ : tO;
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const bf16x8_t bf = __builtin_bit_cast(bf16x8_t, uint4{pw[j][0], pw[j][1], pw[j][2], pw[j][3]});
-#pragma unroll
-                for (int db = 0; db < DB; ++db)
-                    acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_transposed<D>(cols, j, db, lane), bf, acc[db], 0, 0, 0);
-            }
-        }
+        buf = buf1;
     }
     if (ki < a.N) {
         const float f = role_d ? a.scale : 1.f;
@@ -587,6 +598,12 @@ __global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
             }
     }
 }
+
+// Instantiated explicitly: the host pass of this compiler drops the implicit instantiation of the launch stubs.
+template __global__ void bwd_dkdv_bf16_kernel<128>(BwdArgs);
+template __global__ void bwd_dkdv_bf16_kernel<64>(BwdArgs);
+template __global__ void bwd_dq_bf16_kernel<128>(BwdArgs);
+template __global__ void bwd_dq_bf16_kernel<64>(BwdArgs);
 
 int check4(const vsp_tensor* t, int64_t B, int64_t H, int64_t N, int64_t D, int dtype) {
     if (!t) return VSP_ERR_NULL;
@@ -668,6 +685,8 @@ extern "C" int vsp_attn_prefill_backward(const vsp_tensor* dout, const vsp_tenso
             if (!is_aligned16(t->data)) return VSP_ERR_ALIGN;
             for (int i = 0; i < 3; ++i)
                 if ((t->stride[i] * 2) % 16 != 0) return VSP_ERR_ALIGN;
+            if (t->stride[2] < D) return VSP_ERR_STRIDE;   // whole rows are fetched under a byte-range check
+            if ((uint64_t)N * (uint64_t)t->stride[2] * 2u > 0x7fffffffull) return VSP_ERR_STRIDE;
         }
     }
 
