@@ -26,6 +26,7 @@ struct BwdArgs {
     const float* lse;
     void *dq, *dk, *dv;
     float* delta;                          // workspace: Di [B][Hq][N]
+    float* lse2;                           // workspace: lse * log2(e) [B][Hq][N] (bf16 kernels)
     int64_t s_do[3], s_q[3], s_k[3], s_v[3], s_o[3], s_l[3], s_dq[3], s_dk[3], s_dv[3];
     int32_t B, Hq, Hkv, n_rep, N;
     int32_t causal;
@@ -335,6 +336,42 @@ __device__ inline void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "m
 
 constexpr float kLog2e = 1.4426950408889634f;
 
+// two fp32 -> packed bf16x2 (lo = a, hi = b), round-to-nearest-even in one instruction
+__device__ inline uint32_t cvt_pk_bf16(float a, float b) {
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    f32x2_t v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+
+// Di = rowsum(dO * O) and lse * log2(e) (the softmax is recomputed with exp2); D / 8 lanes share a row, 16 bytes each.
+template <int D>
+__global__ void __launch_bounds__(256) bwd_delta_bf16_kernel(BwdArgs a) {
+    constexpr int LPR = D / 8, RPB = 256 / LPR;
+    const int sub = threadIdx.x % LPR;
+    const int64_t rows = (int64_t)a.B * a.Hq * a.N;
+    const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / LPR;
+    const int64_t rr = row < rows ? row : rows - 1;   // every lane takes part in the shuffles
+    const int i = (int)(rr % a.N);
+    const int64_t bh = rr / a.N;
+    const int h = (int)(bh % a.Hq), b = (int)(bh / a.Hq);
+    const uint4 wo = *(const uint4*)((const uint16_t*)a.out + (int64_t)b * a.s_o[0] + (int64_t)h * a.s_o[1] + (int64_t)i * a.s_o[2] + 8 * sub);
+    const uint4 wd = *(const uint4*)((const uint16_t*)a.dout + (int64_t)b * a.s_do[0] + (int64_t)h * a.s_do[1] + (int64_t)i * a.s_do[2] + 8 * sub);
+    const uint32_t o4[4] = {wo.x, wo.y, wo.z, wo.w}, d4[4] = {wd.x, wd.y, wd.z, wd.w};
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        s += __uint_as_float(o4[j] << 16) * __uint_as_float(d4[j] << 16);
+        s += __uint_as_float(o4[j] & 0xffff0000u) * __uint_as_float(d4[j] & 0xffff0000u);
+    }
+#pragma unroll
+    for (int o = LPR / 2; o > 0; o >>= 1) s += __shfl_xor(s, o);
+    if (sub == 0 && row < rows) {
+        a.delta[row] = s;
+        a.lse2[row] = kLog2e * a.lse[(int64_t)b * a.s_l[0] + (int64_t)h * a.s_l[1] + (int64_t)i * a.s_l[2]];
+    }
+}
+
 // ---- dQ (bf16): the structure of bwd_dq_kernel; K serves both as rows (S^T) and transposed (dQ^T) ----
 template <int D>
 __global__ void __launch_bounds__(256, 2) bwd_dq_bf16_kernel(BwdArgs a) {
@@ -362,7 +399,7 @@ __global__ void __launch_bounds__(256, 2) bwd_dq_bf16_kernel(BwdArgs a) {
         qf[ks] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(Qp + 16 * ks + 8 * h));
         dof[ks] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(Op + 16 * ks + 8 * h));
     }
-    const float lse_q = kLog2e * a.lse[(int64_t)b * a.s_l[0] + (int64_t)hq * a.s_l[1] + (int64_t)qrow * a.s_l[2]];
+    const float lse_q = a.lse2[((int64_t)b * a.Hq + hq) * a.N + qrow];
     const float di_q = a.delta[((int64_t)b * a.Hq + hq) * a.N + qrow];
     const float scale_log2 = a.scale * kLog2e;
 
@@ -403,16 +440,25 @@ __global__ void __launch_bounds__(256, 2) bwd_dq_bf16_kernel(BwdArgs a) {
             dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_row<D>(tV, ks, lane), dof[ks], dp, 0, 0, 0);
         }
         uint32_t dsw[2][4];
+        if (k0 + kBT - 1 <= min(q0, a.N - 1) || (!a.causal && k0 + kBT <= a.N)) {   // no position of the tile is masked
 #pragma unroll
-        for (int v = 0; v < 16; v += 2) {
-            float d2[2];
-#pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                const int key = k0 + 8 * ((v + u) >> 2) + 4 * h + ((v + u) & 3);
-                const float p = __builtin_amdgcn_exp2f(s[v + u] * scale_log2 - lse_q);
-                d2[u] = key <= lim ? p * (dp[v + u] - di_q) : 0.f;
+            for (int v = 0; v < 16; v += 2) {
+                const float p0 = __builtin_amdgcn_exp2f(fmaf(s[v], scale_log2, -lse_q));
+                const float p1 = __builtin_amdgcn_exp2f(fmaf(s[v + 1], scale_log2, -lse_q));
+                dsw[v >> 3][(v & 7) >> 1] = cvt_pk_bf16(p0 * (dp[v] - di_q), p1 * (dp[v + 1] - di_q));
             }
-            dsw[v >> 3][(v & 7) >> 1] = pack_bf16x2(d2[0], d2[1]);
+        } else {
+#pragma unroll
+            for (int v = 0; v < 16; v += 2) {
+                float d2[2];
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const int key = k0 + 8 * ((v + u) >> 2) + 4 * h + ((v + u) & 3);
+                    const float p = __builtin_amdgcn_exp2f(key <= lim ? fmaf(s[v + u], scale_log2, -lse_q) : -INFINITY);
+                    d2[u] = p * (dp[v + u] - di_q);
+                }
+                dsw[v >> 3][(v & 7) >> 1] = cvt_pk_bf16(d2[0], d2[1]);
+            }
         }
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
@@ -429,8 +475,8 @@ __global__ void __launch_bounds__(256, 2) bwd_dq_bf16_kernel(BwdArgs a) {
 #pragma unroll
             for (int vq = 0; vq < 4; ++vq) {
                 uint2 w;
-                w.x = pack_bf16x2(a.scale * acc[db][4 * vq], a.scale * acc[db][4 * vq + 1]);
-                w.y = pack_bf16x2(a.scale * acc[db][4 * vq + 2], a.scale * acc[db][4 * vq + 3]);
+                w.x = cvt_pk_bf16(a.scale * acc[db][4 * vq], a.scale * acc[db][4 * vq + 1]);
+                w.y = cvt_pk_bf16(a.scale * acc[db][4 * vq + 2], a.scale * acc[db][4 * vq + 3]);
                 *(uint2*)(op + 32 * db + 8 * vq + 4 * h) = w;
             }
     }
@@ -462,7 +508,9 @@ __global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
     const int b = bh / a.Hkv, kvh = bh % a.Hkv;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int kb = wave >> 1;
-    const bool role_d = wave & 1;
+    // which wavefront of a pair takes which role alternates between workgroups, so that the exp-heavy role of two
+    // co-resident workgroups does not always fall on the same SIMDs
+    const bool role_d = (wave ^ __builtin_popcount(bid >> 3)) & 1;
     const int kl = lane & 31, h = lane >> 5;
     const int key0 = kt * kBK + kb * 32;
     const int ki = key0 + kl;
@@ -495,7 +543,7 @@ __global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
         do_.load(sO[buf], (const uint16_t*)a.dout + (int64_t)b * a.s_do[0] + (int64_t)hq * a.s_do[1] + (int64_t)qb * a.s_do[2],
                  a.N - qb, a.s_do[2], wave);
         if (wave == 0)
-            row_dma(sL[buf], a.lse + (int64_t)b * a.s_l[0] + (int64_t)hq * a.s_l[1] + (int64_t)qb * a.s_l[2], min(a.N - qb, kBT), a.s_l[2], lane);
+            row_dma(sL[buf], a.lse2 + ((int64_t)b * a.Hq + hq) * a.N + qb, min(a.N - qb, kBT), 1, lane);
         else if (wave == 1)
             row_dma(sD[buf], a.delta + ((int64_t)b * a.Hq + hq) * a.N + qb, min(a.N - qb, kBT), 1, lane);
     };
@@ -514,16 +562,24 @@ __global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
             float lq[16];
 #pragma unroll
             for (int g = 0; g < 4; ++g) *(float4*)&lq[4 * g] = *(const float4*)&sL[buf][8 * g + 4 * h];
+            const bool edge = (a.causal && qb < key0 + 31) || qb + kBT > a.N || key0 + 32 > a.N;   // same for the wavefront
+            if (!edge) {
 #pragma unroll
-            for (int v = 0; v < 16; v += 2) {
-                float p2[2];
+                for (int v = 0; v < 16; v += 2)
+                    pw[v >> 3][(v & 7) >> 1] = cvt_pk_bf16(__builtin_amdgcn_exp2f(fmaf(s[v], scale_log2, -lq[v])),
+                                                           __builtin_amdgcn_exp2f(fmaf(s[v + 1], scale_log2, -lq[v + 1])));
+            } else {
 #pragma unroll
-                for (int u = 0; u < 2; ++u) {
-                    const int qi = qb + 8 * ((v + u) >> 2) + 4 * h + ((v + u) & 3);
-                    const float e = __builtin_amdgcn_exp2f(s[v + u] * scale_log2 - lq[v + u] * kLog2e);
-                    p2[u] = (qi < a.N && ki < a.N && (!a.causal || ki <= qi)) ? e : 0.f;
+                for (int v = 0; v < 16; v += 2) {
+                    float p2[2];
+#pragma unroll
+                    for (int u = 0; u < 2; ++u) {
+                        const int qi = qb + 8 * ((v + u) >> 2) + 4 * h + ((v + u) & 3);
+                        const bool ok = qi < a.N && ki < a.N && (!a.causal || ki <= qi);
+                        p2[u] = __builtin_amdgcn_exp2f(ok ? fmaf(s[v + u], scale_log2, -lq[v + u]) : -INFINITY);
+                    }
+                    pw[v >> 3][(v & 7) >> 1] = cvt_pk_bf16(p2[0], p2[1]);
                 }
-                pw[v >> 3][(v & 7) >> 1] = pack_bf16x2(p2[0], p2[1]);
             }
 #pragma unroll
             for (int j = 0; j < 2; ++j)
@@ -542,7 +598,7 @@ __global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
             for (int v = 0; v < 16; v += 2) {
                 const uint32_t w = sP[t & 1][kb][v >> 1][lane];
                 const float p0 = __uint_as_float(w << 16), p1 = __uint_as_float(w & 0xffff0000u);
-                pw[v >> 3][(v & 7) >> 1] = pack_bf16x2(p0 * (s[v] - di[v]), p1 * (s[v + 1] - di[v + 1]));
+                pw[v >> 3][(v & 7) >> 1] = cvt_pk_bf16(p0 * (s[v] - di[v]), p1 * (s[v + 1] - di[v + 1]));
             }
         }
         const uint16_t* cols = role_d ? sQ[buf] : sO[buf];
@@ -592,8 +648,8 @@ __global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
 #pragma unroll
             for (int vq = 0; vq < 4; ++vq) {
                 uint2 w;
-                w.x = pack_bf16x2(f * acc[db][4 * vq], f * acc[db][4 * vq + 1]);
-                w.y = pack_bf16x2(f * acc[db][4 * vq + 2], f * acc[db][4 * vq + 3]);
+                w.x = cvt_pk_bf16(f * acc[db][4 * vq], f * acc[db][4 * vq + 1]);
+                w.y = cvt_pk_bf16(f * acc[db][4 * vq + 2], f * acc[db][4 * vq + 3]);
                 *(uint2*)(po + 32 * db + 8 * vq + 4 * h) = w;
             }
     }
@@ -604,6 +660,8 @@ template __global__ void bwd_dkdv_bf16_kernel<128>(BwdArgs);
 template __global__ void bwd_dkdv_bf16_kernel<64>(BwdArgs);
 template __global__ void bwd_dq_bf16_kernel<128>(BwdArgs);
 template __global__ void bwd_dq_bf16_kernel<64>(BwdArgs);
+template __global__ void bwd_delta_bf16_kernel<128>(BwdArgs);
+template __global__ void bwd_delta_bf16_kernel<64>(BwdArgs);
 
 int check4(const vsp_tensor* t, int64_t B, int64_t H, int64_t N, int64_t D, int dtype) {
     if (!t) return VSP_ERR_NULL;
@@ -618,7 +676,12 @@ int check4(const vsp_tensor* t, int64_t B, int64_t H, int64_t N, int64_t D, int 
 template <typename T>
 int launch_backward(const BwdArgs& a, int64_t D, hipStream_t st) {
     const int64_t rows = (int64_t)a.B * a.Hq * a.N;
-    hipLaunchKernelGGL(bwd_delta_kernel<T>, dim3((unsigned)ceil_div(rows, 4)), dim3(256), 0, st, a, (int)D);
+    if constexpr (sizeof(T) == 2) {
+        if (D == 128) hipLaunchKernelGGL(bwd_delta_bf16_kernel<128>, dim3((unsigned)ceil_div(rows, 16)), dim3(256), 0, st, a);
+        else hipLaunchKernelGGL(bwd_delta_bf16_kernel<64>, dim3((unsigned)ceil_div(rows, 32)), dim3(256), 0, st, a);
+    } else {
+        hipLaunchKernelGGL(bwd_delta_kernel<T>, dim3((unsigned)ceil_div(rows, 4)), dim3(256), 0, st, a, (int)D);
+    }
     int rc = check_launch();
     if (rc != VSP_OK) return rc;
     const int64_t tiles = ceil_div(a.N, kBQ);
@@ -651,7 +714,7 @@ using namespace vsp;
 
 extern "C" size_t vsp_attn_backward_workspace_bytes(int32_t B, int32_t Hq, int32_t N) {
     if (B <= 0 || Hq <= 0 || N <= 0) return 0;
-    return (size_t)B * (size_t)Hq * (size_t)N * sizeof(float);
+    return 2 * (size_t)B * (size_t)Hq * (size_t)N * sizeof(float);   // Di and the rescaled log-sum-exp
 }
 
 extern "C" int vsp_attn_prefill_backward(const vsp_tensor* dout, const vsp_tensor* q, const vsp_tensor* k,
@@ -701,6 +764,7 @@ extern "C" int vsp_attn_prefill_backward(const vsp_tensor* dout, const vsp_tenso
     a.dk = dk->data;
     a.dv = dv->data;
     a.delta = (float*)workspace;
+    a.lse2 = a.delta + B * Hq * N;
     for (int i = 0; i < 3; ++i) {
         a.s_do[i] = dout->stride[i];
         a.s_q[i] = q->stride[i];
