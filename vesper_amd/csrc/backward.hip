@@ -16,6 +16,8 @@
 // the inference path: plain LDS tiles filled by ordinary loads, no direct-to-LDS pipeline.
 #include <math.h>
 
+#include <type_traits>
+
 #include "vsp_common.hpp"
 
 namespace vsp {
@@ -376,8 +378,10 @@ __global__ void __launch_bounds__(256) bwd_delta_bf16_kernel(BwdArgs a) {
 template <int D>
 __global__ void __launch_bounds__(256, 2) bwd_dq_bf16_kernel(BwdArgs a) {
     constexpr int KS = D / 16, DB = D / 32;
-    __shared__ __attribute__((aligned(1024))) uint16_t sK[2][kBT * D];
-    __shared__ __attribute__((aligned(1024))) uint16_t sV[2][kBT * D];
+    // One variable per ring slot: the compiler then knows that a read of one slot does not touch the slot a
+    // direct-to-LDS load in flight is filling, and does not wait for that load.
+    __shared__ __attribute__((aligned(1024))) uint16_t sK0[kBT * D], sK1[kBT * D];
+    __shared__ __attribute__((aligned(1024))) uint16_t sV0[kBT * D], sV1[kBT * D];
     const int n_qtiles = (a.N + kBQ - 1) / kBQ;
     const int bid = blockIdx.x;
     const int qt = n_qtiles - 1 - bid / (a.B * a.Hq);
@@ -418,19 +422,18 @@ __global__ void __launch_bounds__(256, 2) bwd_dq_bf16_kernel(BwdArgs a) {
     TileDma<D> dk_, dv_;
     dk_.init(a.s_k[2], wave, lane);
     dv_.init(a.s_v[2], wave, lane);
-    auto load = [&](int kt) {
-        dk_.load(sK[kt & 1], Kp + (int64_t)kt * kBT * a.s_k[2], a.N - kt * kBT, a.s_k[2], wave);
-        dv_.load(sV[kt & 1], Vp + (int64_t)kt * kBT * a.s_v[2], a.N - kt * kBT, a.s_v[2], wave);
+    auto load = [&](int kt, auto slot) {
+        dk_.load(slot.value ? sK1 : sK0, Kp + (int64_t)kt * kBT * a.s_k[2], a.N - kt * kBT, a.s_k[2], wave);
+        dv_.load(slot.value ? sV1 : sV0, Vp + (int64_t)kt * kBT * a.s_v[2], a.N - kt * kBT, a.s_v[2], wave);
     };
-    load(0);
-    for (int kt = 0; kt < n_tiles; ++kt) {
+    auto step = [&](int kt, auto slot) {
         dma_wait_all();
-        __syncthreads();   // tile kt is in LDS; every wavefront has left tile kt - 1, whose buffer is refilled now
-        if (kt + 1 < n_tiles) load(kt + 1);
+        __syncthreads();   // tile kt is in LDS; every wavefront has left tile kt - 1, whose slot is refilled now
+        if (kt + 1 < n_tiles) load(kt + 1, std::integral_constant<int, 1 - slot.value>{});
+        const uint16_t* tK = slot.value ? sK1 : sK0;
+        const uint16_t* tV = slot.value ? sV1 : sV0;
         const int k0 = kt * kBT;
-        if (k0 >= kv_end_wave) continue;
-        const uint16_t* tK = sK[kt & 1];
-        const uint16_t* tV = sV[kt & 1];
+        if (k0 >= kv_end_wave) return;
         f32x16_t s, dp;
 #pragma unroll
         for (int j = 0; j < 16; ++j) s[j] = dp[j] = 0.f;
@@ -467,6 +470,11 @@ __global__ void __launch_bounds__(256, 2) bwd_dq_bf16_kernel(BwdArgs a) {
             for (int db = 0; db < DB; ++db)
                 acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_transposed<D>(tK, j, db, lane), dsf, acc[db], 0, 0, 0);
         }
+    };
+    load(0, std::integral_constant<int, 0>{});
+    for (int kt = 0; kt < n_tiles; kt += 2) {
+        step(kt, std::integral_constant<int, 0>{});
+        if (kt + 1 < n_tiles) step(kt + 1, std::integral_constant<int, 1>{});
     }
     if (qi < a.N) {
         uint16_t* op = (uint16_t*)a.dq + (int64_t)b * a.s_dq[0] + (int64_t)hq * a.s_dq[1] + (int64_t)qi * a.s_dq[2];
