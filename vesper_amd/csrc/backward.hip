@@ -505,11 +505,17 @@ constexpr int kBK = 64;   // key rows per workgroup in the bf16 dK / dV pass
 template <int D>
 __global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
     constexpr int KS = D / 16, DB = D / 32;
-    __shared__ __attribute__((aligned(1024))) uint16_t sQ[3][kBT * D];
-    __shared__ __attribute__((aligned(1024))) uint16_t sO[3][kBT * D];
-    __shared__ __attribute__((aligned(256))) float sL[3][64];      // lse and Di of the tile's rows (32 used; a wavefront
-    __shared__ __attribute__((aligned(256))) float sD[3][64];      // instruction fills 64 words)
-    __shared__ __attribute__((aligned(16))) uint32_t sP[2][2][8][64];   // [parity of the tile][key block][word][lane]
+    // One variable per ring slot: the compiler then knows that a read of one slot does not touch the slot a
+    // direct-to-LDS load in flight is filling, and does not wait for that load.
+    __shared__ __attribute__((aligned(1024))) uint16_t sQ0[kBT * D], sQ1[kBT * D], sQ2[kBT * D];
+    __shared__ __attribute__((aligned(1024))) uint16_t sO0[kBT * D], sO1[kBT * D], sO2[kBT * D];
+    __shared__ __attribute__((aligned(256))) float sL0[64], sL1[64], sL2[64];   // lse and Di of the tile's rows (32 used; a
+    __shared__ __attribute__((aligned(256))) float sD0[64], sD1[64], sD2[64];   // wavefront instruction fills 64 words)
+    __shared__ __attribute__((aligned(16))) uint32_t sP[3][2][8][64];            // [ring slot][key block][word][lane]
+    auto tq = [&](auto s) -> uint16_t* { if constexpr (s.value == 0) return sQ0; else if constexpr (s.value == 1) return sQ1; else return sQ2; };
+    auto to = [&](auto s) -> uint16_t* { if constexpr (s.value == 0) return sO0; else if constexpr (s.value == 1) return sO1; else return sO2; };
+    auto tl = [&](auto s) -> float* { if constexpr (s.value == 0) return sL0; else if constexpr (s.value == 1) return sL1; else return sL2; };
+    auto td = [&](auto s) -> float* { if constexpr (s.value == 0) return sD0; else if constexpr (s.value == 1) return sD1; else return sD2; };
     const int bid = blockIdx.x;
     const int kt = bid / (a.B * a.Hkv);          // causal work falls with the key tile: heaviest first
     const int bh = bid % (a.B * a.Hkv);
@@ -518,7 +524,7 @@ __global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
     const int kb = wave >> 1;
     // which wavefront of a pair takes which role alternates between workgroups, so that the exp-heavy role of two
     // co-resident workgroups does not always fall on the same SIMDs
-    const bool role_d = (wave ^ __builtin_popcount(bid >> 3)) & 1;
+    const bool role_d = __builtin_amdgcn_readfirstlane((wave ^ __builtin_popcount(bid >> 3)) & 1);
     const int kl = lane & 31, h = lane >> 5;
     const int key0 = kt * kBK + kb * 32;
     const int ki = key0 + kl;
@@ -544,32 +550,37 @@ __global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
     TileDma<D> dq_, do_;
     dq_.init(a.s_q[2], wave, lane);
     do_.init(a.s_do[2], wave, lane);
-    auto load = [&](int it, int buf) {
+    auto load = [&](int it, auto buf) {
         const int hq = kvh * a.n_rep + it / n_qt, qb = (qt_begin + it % n_qt) * kBT;
-        dq_.load(sQ[buf], (const uint16_t*)a.q + (int64_t)b * a.s_q[0] + (int64_t)hq * a.s_q[1] + (int64_t)qb * a.s_q[2], a.N - qb,
+        dq_.load(tq(buf), (const uint16_t*)a.q + (int64_t)b * a.s_q[0] + (int64_t)hq * a.s_q[1] + (int64_t)qb * a.s_q[2], a.N - qb,
                  a.s_q[2], wave);
-        do_.load(sO[buf], (const uint16_t*)a.dout + (int64_t)b * a.s_do[0] + (int64_t)hq * a.s_do[1] + (int64_t)qb * a.s_do[2],
+        do_.load(to(buf), (const uint16_t*)a.dout + (int64_t)b * a.s_do[0] + (int64_t)hq * a.s_do[1] + (int64_t)qb * a.s_do[2],
                  a.N - qb, a.s_do[2], wave);
         if (wave == 0)
-            row_dma(sL[buf], a.lse2 + ((int64_t)b * a.Hq + hq) * a.N + qb, min(a.N - qb, kBT), 1, lane);
+            row_dma(tl(buf), a.lse2 + ((int64_t)b * a.Hq + hq) * a.N + qb, min(a.N - qb, kBT), 1, lane);
         else if (wave == 1)
-            row_dma(sD[buf], a.delta + ((int64_t)b * a.Hq + hq) * a.N + qb, min(a.N - qb, kBT), 1, lane);
+            row_dma(td(buf), a.delta + ((int64_t)b * a.Hq + hq) * a.N + qb, min(a.N - qb, kBT), 1, lane);
     };
+    // The loop exists once per role, so that each wavefront's code reads its tiles from named variables.
+    auto run = [&](auto role) {
+    constexpr bool RD = decltype(role)::value;
     // first products of tile t: S (P wavefront) or dP (D wavefront) into s; the P wavefront goes on to P(t),
     // packed into pw and posted for its partner.  Masked or out-of-range positions get P = 0, so a tile that lies
     // wholly above the diagonal or past the end costs its MFMAs and contributes nothing.
-    auto first = [&](int t, int buf, f32x16_t& s, uint32_t (&pw)[2][4]) {
-        const uint16_t* rows = role_d ? sO[buf] : sQ[buf];
+    auto first = [&](int t, auto buf, f32x16_t& s, uint32_t (&pw)[2][4]) {
+        const uint16_t* rows;
+        if constexpr (RD) rows = to(buf);
+        else rows = tq(buf);
 #pragma unroll
         for (int j = 0; j < 16; ++j) s[j] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks)
             s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_row<D>(rows, ks, lane), xf[ks], s, 0, 0, 0);
-        if (!role_d) {
+        if constexpr (!RD) {
             const int qb = (qt_begin + t % n_qt) * kBT;
             float lq[16];
 #pragma unroll
-            for (int g = 0; g < 4; ++g) *(float4*)&lq[4 * g] = *(const float4*)&sL[buf][8 * g + 4 * h];
+            for (int g = 0; g < 4; ++g) *(float4*)&lq[4 * g] = *(const float4*)&tl(buf)[8 * g + 4 * h];
             const bool edge = (a.causal && qb < key0 + 31) || qb + kBT > a.N || key0 + 32 > a.N;   // same for the wavefront
             if (!edge) {
 #pragma unroll
@@ -592,24 +603,26 @@ __global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
 #pragma unroll
             for (int j = 0; j < 2; ++j)
 #pragma unroll
-                for (int w = 0; w < 4; ++w) sP[t & 1][kb][4 * j + w][lane] = pw[j][w];
+                for (int w = 0; w < 4; ++w) sP[buf.value][kb][4 * j + w][lane] = pw[j][w];
         }
     };
     // second products of tile t: dV^T += dO^T P (P wavefront, P from its own registers) or
     // dS = P (dP - Di), dK^T += Q^T dS (D wavefront, P from its partner)
-    auto second = [&](int t, int buf, const f32x16_t& s, uint32_t (&pw)[2][4]) {
-        if (role_d) {
+    auto second = [&](int t, auto buf, const f32x16_t& s, uint32_t (&pw)[2][4]) {
+        if constexpr (RD) {
             float di[16];
 #pragma unroll
-            for (int g = 0; g < 4; ++g) *(float4*)&di[4 * g] = *(const float4*)&sD[buf][8 * g + 4 * h];
+            for (int g = 0; g < 4; ++g) *(float4*)&di[4 * g] = *(const float4*)&td(buf)[8 * g + 4 * h];
 #pragma unroll
             for (int v = 0; v < 16; v += 2) {
-                const uint32_t w = sP[t & 1][kb][v >> 1][lane];
+                const uint32_t w = sP[buf.value][kb][v >> 1][lane];
                 const float p0 = __uint_as_float(w << 16), p1 = __uint_as_float(w & 0xffff0000u);
                 pw[v >> 3][(v & 7) >> 1] = cvt_pk_bf16(p0 * (s[v] - di[v]), p1 * (s[v + 1] - di[v + 1]));
             }
         }
-        const uint16_t* cols = role_d ? sQ[buf] : sO[buf];
+        const uint16_t* cols;
+        if constexpr (RD) cols = tq(buf);
+        else cols = to(buf);
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const bf16x8_t bf = __builtin_bit_cast(bf16x8_t, uint4{pw[j][0], pw[j][1], pw[j][2], pw[j][3]});
@@ -619,34 +632,36 @@ __global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
         }
     };
 
-    f32x16_t s_cur, s_next;
-    uint32_t pw_cur[2][4], pw_next[2][4];
-    load(0, 0);
-    if (n_it > 1) load(1, 1);
+    f32x16_t s_cur;
+    uint32_t pw_cur[2][4];
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
+    using S2 = std::integral_constant<int, 2>;
+    load(0, S0{});
+    if (n_it > 1) load(1, S1{});
     dma_wait_all();
     __syncthreads();
-    first(0, 0, s_cur, pw_cur);
-    int buf = 0;   // ring slot of tile `it`
-    for (int it = 0; it < n_it; ++it) {
+    first(0, S0{}, s_cur, pw_cur);
+    // one iteration, for tile `it` in ring slot `buf`
+    auto step = [&](int it, auto buf) {
+        using B1 = std::integral_constant<int, (buf.value + 1) % 3>;
+        using B2 = std::integral_constant<int, (buf.value + 2) % 3>;
         // tile it + 1 and P(it) are in LDS; every wavefront has left tile it - 1, whose slot takes tile it + 2
         dma_wait_all();
         __syncthreads();
-        const int buf1 = buf == 2 ? 0 : buf + 1, buf2 = buf1 == 2 ? 0 : buf1 + 1;
-        if (it + 2 < n_it) load(it + 2, buf2);
-        if (it + 1 < n_it) {
-            // independent streams in one block: first products of the next tile, second products of this one
-            first(it + 1, buf1, s_next, pw_next);
-            second(it, buf, s_cur, pw_cur);
-            s_cur = s_next;
-#pragma unroll
-            for (int j = 0; j < 2; ++j)
-#pragma unroll
-                for (int w = 0; w < 4; ++w) pw_cur[j][w] = pw_next[j][w];
-        } else {
-            second(it, buf, s_cur, pw_cur);
-        }
-        buf = buf1;
+        if (it + 2 < n_it) load(it + 2, B2{});
+        // the second products consume s / pw of this tile, then the first products of the next tile refill them
+        second(it, buf, s_cur, pw_cur);
+        if (it + 1 < n_it) first(it + 1, B1{}, s_cur, pw_cur);
+    };
+    for (int it = 0; it < n_it; it += 3) {
+        step(it, S0{});
+        if (it + 1 < n_it) step(it + 1, S1{});
+        if (it + 2 < n_it) step(it + 2, S2{});
     }
+    };
+    if (role_d) run(std::true_type{});
+    else run(std::false_type{});
     if (ki < a.N) {
         const float f = role_d ? a.scale : 1.f;
         uint16_t* po = role_d ? (uint16_t*)a.dk + (int64_t)b * a.s_dk[0] + (int64_t)kvh * a.s_dk[1] + (int64_t)ki * a.s_dk[2]
