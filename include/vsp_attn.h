@@ -204,8 +204,10 @@ int vsp_attn_prefill(const vsp_tensor* q, const vsp_tensor* k, const vsp_tensor*
  * without dropout: Di = rowsum(dO*O), P = exp(scale q.k - lse), dV = P^T dO, dS = P*(dO V^T - Di), dQ = scale dS K,
  * dK = scale dS^T Q.  dout/q/out/dq [B,Hq,N,D], k/v/dk/dv [B,Hkv,N,D] (Hq % Hkv == 0: dk/dv of a kv head sum over
  * its query heads, the gradient of ops::repeat_kv), lse [B,Hq,N] fp32 as written by vsp_attn_prefill; fp32 or bf16
- * (one dtype; fp32 arithmetic on matrix cores, bf16 gradients rounded to nearest even), D in {64,128}, any strides
- * with stride[3]==1.  dq/dk/dv are overwritten.  No atomics: results are bitwise reproducible (the reference's
+ * (one dtype).  fp32: fp32 matrix-core arithmetic, any strides with stride[3]==1.  bf16: bf16 matrix cores with fp32
+ * accumulation, P and dS rounded to bf16 between the products, gradients rounded to nearest even; base pointers and
+ * strides multiples of 16 bytes (VSP_ERR_ALIGN), stride[2] >= D (VSP_ERR_STRIDE).  D in {64,128}.  dq/dk/dv are
+ * overwritten.  No atomics: results are bitwise reproducible (the reference's
  * HIP kernel accumulates dQ with atomicAdd).  workspace: vsp_attn_backward_workspace_bytes(B, Hq, N) bytes. */
 size_t vsp_attn_backward_workspace_bytes(int32_t B, int32_t Hq, int32_t N);
 int vsp_attn_prefill_backward(const vsp_tensor* dout, const vsp_tensor* q, const vsp_tensor* k, const vsp_tensor* v,
