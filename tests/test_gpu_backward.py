@@ -147,6 +147,36 @@ def test_bf16_rows_must_be_16_byte_aligned(va):
         va.flash_attention_backward(ok, off, ok, ok, ok, torch.zeros(1, 2, 8, device=d), 0.1)
 
 
+def test_bf16_config3_shape_causal_truncation(va):
+    # benchmark config 3's shape (B1, 32/8 heads, D128, N8192).  With dO = 0 from row n on, causal attention makes the
+    # first n rows of dq / dk / dv those of the n-token problem - bit for bit, because the later query tiles add exact
+    # zeros (dP = 0, Di = 0, so dS = 0, and P * 0 = 0) in between the same partial sums - and the rest exactly zero.
+    B, Hq, Hkv, N, D, n = 1, 32, 8, 8192, 128, 2048
+    g = torch.Generator(device="cuda").manual_seed(19)
+    mk = lambda h: (torch.randn(B, h, N, D, device=G.dev(), generator=g) * 0.5).to(torch.bfloat16)
+    q, k, v, dout = mk(Hq), mk(Hkv), mk(Hkv), mk(Hq)
+    dout[:, :, n:] = 0
+    scale = 1.0 / math.sqrt(D)
+    out, lse = va.flash_attention(q, k, v, scale, True, return_lse=True)
+    dq, dk, dv = va.flash_attention_backward(dout, q, k, v, out, lse, scale, True)
+    cut = lambda t: t[:, :, :n].contiguous()
+    sq, sk, sv = va.flash_attention_backward(cut(dout), cut(q), cut(k), cut(v), cut(out), lse[:, :, :n].contiguous(), scale, True)
+    for big, small, name in ((dq, sq, "dq"), (dk, sk, "dk"), (dv, sv, "dv")):
+        assert torch.isfinite(big.float()).all(), name
+        assert torch.equal(big[:, :, :n], small), name
+        assert not big[:, :, n:].any(), name
+        assert small.float().abs().max() > 1e-3, name      # the comparison is not between zeros
+    # dv of the last key of the sub-problem: only query n - 1 sees it, P = exp(s - lse) -> dv = P * dO[n - 1], summed
+    # over the 4 query heads of the group (float64, from the kernel's own lse)
+    qf, kf = G.bf16_to_np(q[0, :, n - 1]).astype(np.float64), G.bf16_to_np(k[0, :, n - 1]).astype(np.float64)
+    dof = G.bf16_to_np(dout[0, :, n - 1]).astype(np.float64)
+    l = lse[0, :, n - 1].cpu().numpy().astype(np.float64)
+    for kvh in (0, 5):
+        want = sum(np.exp(qf[h] @ kf[kvh] * scale - l[h]) * dof[h] for h in range(4 * kvh, 4 * kvh + 4))
+        got = G.bf16_to_np(dv[0, kvh, n - 1]).astype(np.float64)
+        assert np.abs(got - want).max() <= 2e-2 * max(1.0, np.abs(want).max())
+
+
 def test_argument_errors(va):
     d = G.dev()
     q = torch.zeros(1, 4, 8, 64, device=d)
