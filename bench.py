@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on ONE MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|p4k|c3|c4|c5|c4p|c2c|c3c|r2|b2] [--no-cpu] [--no-extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|p4k|c3|c4|c5|c4p|c2c|c3c|r2|b2|b3] [--no-cpu] [--no-extra]
 
 A "step" is one pass of the hot path over one batch of synthetic input that is already resident in
 HBM: one prefill launch (c2, p4k, c3) or one decode call = split-K kernel + combine kernel (c4, c5).
@@ -47,6 +47,9 @@ WORKLOADS = {
     "b2": dict(kind="backward", B=4, Hq=32, Hkv=8, D=128, N=2048,
                name="attention backward at config 2's shape: causal GQA bf16 in/out, bf16 MFMA with fp32 accumulation, "
                     "B4, 32 q / 8 kv heads, D128, N2048 (dq, dk, dv; 2.5 x the forward's FLOPs)"),
+    "b3": dict(kind="backward", B=1, Hq=32, Hkv=8, D=128, N=8192,
+               name="attention backward at config 3's shape: causal GQA bf16 in/out, bf16 MFMA with fp32 accumulation, "
+                    "B1, 32 q / 8 kv heads, D128, N8192 (dq, dk, dv; 2.5 x the forward's FLOPs)"),
     "r2": dict(kind="rope", fmt="bf16", B=4, Hq=32, Hkv=8, D=128, N=2048,
                name="RoPE + KV append for config 2: q/k/v bf16 views of one fused projection buffer [B,T,(Hq+2Hkv)D], "
                     "rotated q out bf16, bf16 cache, B4, 32 q / 8 kv heads, D128, T2048"),
@@ -347,7 +350,7 @@ def main():
 
     if not args.no_extra:
         others = {}
-        for key in ("c2", "p4k", "c3", "c4", "c5", "c4p", "c2c", "c3c", "r2", "b2"):
+        for key in ("c2", "p4k", "c3", "c4", "c5", "c4p", "c2c", "c3c", "r2", "b2", "b3"):
             if key == args.workload:
                 continue
             r = Runner(key, torch, va)
