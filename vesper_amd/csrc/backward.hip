@@ -387,7 +387,7 @@ __global__ void __launch_bounds__(256, 2) bwd_dq_bf16_kernel(BwdArgs a) {
     const int qt = n_qtiles - 1 - bid / (a.B * a.Hq);
     const int bh = bid % (a.B * a.Hq);
     const int b = bh / a.Hq, hq = bh % a.Hq, kvh = hq / a.n_rep;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int ql = lane & 31, h = lane >> 5;
     const int q0 = qt * kBQ + wave * 32;
     const int qi = q0 + ql;
@@ -520,7 +520,7 @@ __global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
     const int kt = bid / (a.B * a.Hkv);          // causal work falls with the key tile: heaviest first
     const int bh = bid % (a.B * a.Hkv);
     const int b = bh / a.Hkv, kvh = bh % a.Hkv;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int kb = wave >> 1;
     // which wavefront of a pair takes which role alternates between workgroups, so that the exp-heavy role of two
     // co-resident workgroups does not always fall on the same SIMDs
@@ -550,8 +550,18 @@ __global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
     TileDma<D> dq_, do_;
     dq_.init(a.s_q[2], wave, lane);
     do_.init(a.s_do[2], wave, lane);
+    // (head of the group, query tile) of the tile being fetched and of the tile whose first products are due:
+    // the loop index split without a division per step
+    int ld_r = 0, ld_t = 0, fi_r = 0, fi_t = 0;
+    auto advance = [&](int& r, int& t) {
+        if (++t == n_qt) {
+            t = 0;
+            ++r;
+        }
+    };
     auto load = [&](int it, auto buf) {
-        const int hq = kvh * a.n_rep + it / n_qt, qb = (qt_begin + it % n_qt) * kBT;
+        const int hq = kvh * a.n_rep + ld_r, qb = (qt_begin + ld_t) * kBT;
+        advance(ld_r, ld_t);
         dq_.load(tq(buf), (const uint16_t*)a.q + (int64_t)b * a.s_q[0] + (int64_t)hq * a.s_q[1] + (int64_t)qb * a.s_q[2], a.N - qb,
                  a.s_q[2], wave);
         do_.load(to(buf), (const uint16_t*)a.dout + (int64_t)b * a.s_do[0] + (int64_t)hq * a.s_do[1] + (int64_t)qb * a.s_do[2],
@@ -577,7 +587,7 @@ __global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
         for (int ks = 0; ks < KS; ++ks)
             s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_row<D>(rows, ks, lane), xf[ks], s, 0, 0, 0);
         if constexpr (!RD) {
-            const int qb = (qt_begin + t % n_qt) * kBT;
+            const int qb = (qt_begin + fi_t) * kBT;
             float lq[16];
 #pragma unroll
             for (int g = 0; g < 4; ++g) *(float4*)&lq[4 * g] = *(const float4*)&tl(buf)[8 * g + 4 * h];
@@ -604,6 +614,7 @@ __global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
             for (int j = 0; j < 2; ++j)
 #pragma unroll
                 for (int w = 0; w < 4; ++w) sP[buf.value][kb][4 * j + w][lane] = pw[j][w];
+            advance(fi_r, fi_t);
         }
     };
     // second products of tile t: dV^T += dO^T P (P wavefront, P from its own registers) or

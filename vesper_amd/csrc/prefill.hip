@@ -54,7 +54,7 @@ struct PrefillArgs {
 };
 
 constexpr int kBM = 128;       // queries per workgroup
-constexpr float kRescaleThreshold = 8.0f;
+[[maybe_unused]] constexpr float kRescaleThreshold = 8.0f;
 
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
@@ -126,7 +126,7 @@ __device__ inline uint32_t lds_addr(const void* p) {
     return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
 }
 
-constexpr int kUnit = 32;  // keys per tile (one LDS ring slot)
+[[maybe_unused]] constexpr int kUnit = 32;  // keys per tile (one LDS ring slot)
 
 // VBLK: K and V are the planes of a bf16 KV cache (K row-major, V token-blocked by 8) instead of dense
 // tensors, and the context length may come per batch row from a device array.  With 8 tokens of one d
