@@ -1,7 +1,8 @@
 """The decode step (RoPE + append at device-side positions, length advance, split-K decode, combine) recorded
 into a HIP graph and replayed: every entry point is asynchronous, allocates nothing and records no memset node, so a
 serving loop can replay one graph per token.  Each replay is checked against the same step run eagerly, with the
-program's own eager work and synchronisations between replays."""
+program's own eager work and synchronisations between replays.  The same for a training step's attention: prefill
+forward and backward in one graph."""
 import numpy as np
 import pytest
 import torch
@@ -68,3 +69,30 @@ def test_decode_step_replays_bit_identically(va, fmt):
         torch.cuda.synchronize()
         assert torch.equal(out, eager[i]), f"replay {i}"
     assert cg.seq_lens.cpu().tolist() == [p + steps for p in prompts]
+
+
+def test_forward_backward_replays_bit_identically(va):
+    # a training step's attention (prefill forward with lse, then dq / dk / dv) in one graph: three launches of the
+    # backward share a workspace the caller owns, nothing is cleared by a memset node
+    B, Hq, Hkv, N, D = 2, 8, 2, 200, 128
+    mk = lambda seed, h: G.to_bf16_dev(I.normal(seed, (B, h, N, D), scale=0.5))
+    sq, sk, sv, sd = mk(1, Hq), mk(2, Hkv), mk(3, Hkv), mk(4, Hq)
+    inputs = [[mk(10 * i + j, h) for j, h in enumerate((Hq, Hkv, Hkv, Hq))] for i in range(1, 4)]
+    eager = []
+    for q, k, v, d in inputs:
+        o, l = va.flash_attention(q, k, v, 0.1, True, return_lse=True)
+        eager.append([o.clone()] + [t.clone() for t in va.flash_attention_backward(d, q, k, v, o, l, 0.1, True)])
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            o, l = va.flash_attention(sq, sk, sv, 0.1, True, return_lse=True)
+            grads = va.flash_attention_backward(sd, sq, sk, sv, o, l, 0.1, True)
+    torch.cuda.synchronize()
+    for i, (q, k, v, d) in enumerate(inputs):
+        sq.copy_(q), sk.copy_(k), sv.copy_(v), sd.copy_(d)   # eager work between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, want in zip([o] + list(grads), eager[i]):
+            assert torch.equal(got, want), f"replay {i}"
