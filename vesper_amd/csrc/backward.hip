@@ -778,7 +778,7 @@ extern "C" int vsp_attn_prefill_backward(const vsp_tensor* dout, const vsp_tenso
     if (!workspace || workspace_bytes < vsp_attn_backward_workspace_bytes((int32_t)B, (int32_t)Hq, (int32_t)N)) return VSP_ERR_WORKSPACE;
     if (((uintptr_t)workspace & 3) != 0) return VSP_ERR_ALIGN;
     if (dt == VSP_BF16) {  // 16-byte row segments are moved whole
-        for (const vsp_tensor* t : {dout, q, k, v, (const vsp_tensor*)dq, (const vsp_tensor*)dk, (const vsp_tensor*)dv}) {
+        for (const vsp_tensor* t : {dout, q, k, v, out, (const vsp_tensor*)dq, (const vsp_tensor*)dk, (const vsp_tensor*)dv}) {
             if (!is_aligned16(t->data)) return VSP_ERR_ALIGN;
             for (int i = 0; i < 3; ++i)
                 if ((t->stride[i] * 2) % 16 != 0) return VSP_ERR_ALIGN;
