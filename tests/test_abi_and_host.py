@@ -109,6 +109,46 @@ def test_validation_that_needs_no_gpu(ffi):
     assert ffi.lib.vsp_kv_cache_reset(C.byref(c), None) == ffi.ERR_NULL  # planes missing
 
 
+def test_backward_validation_that_needs_no_gpu(ffi):
+    # every rejection below is decided on the host before anything is launched (the pointers are never followed)
+    def tens(shape, dtype, ptr=0x10000, strides=None):
+        t = ffi.VspTensor()
+        t.ndim, t.dtype, t.data = len(shape), dtype, ptr
+        st = strides or [int(np.prod(shape[i + 1:])) for i in range(len(shape))]
+        for i, (n, m) in enumerate(zip(shape, st)):
+            t.shape[i], t.stride[i] = n, m
+        return t
+
+    def call(dout, q, k, v, out, lse, dq, dk, dv, ws=0x20000, ws_bytes=1 << 30):
+        a = [C.byref(x) if x is not None else None for x in (dout, q, k, v, out, lse, dq, dk, dv)]
+        return ffi.lib.vsp_attn_prefill_backward(*a, 0.125, 1, ws, ws_bytes, None)
+
+    B, Hq, Hkv, N, D = 1, 4, 2, 8, 64
+    q, k, lse = tens((B, Hq, N, D), ffi.BF16), tens((B, Hkv, N, D), ffi.BF16), tens((B, Hq, N), ffi.F32)
+    assert ffi.lib.vsp_attn_backward_workspace_bytes(B, Hq, N) == 2 * B * Hq * N * 4
+    assert ffi.lib.vsp_attn_backward_workspace_bytes(0, Hq, N) == 0
+    assert call(q, None, k, k, q, lse, q, k, k) == ffi.ERR_NULL
+    assert call(q, tens((B, Hq, N), ffi.BF16), k, k, q, lse, q, k, k) == ffi.ERR_NDIM
+    k3 = tens((B, 3, N, D), ffi.BF16)
+    assert call(q, q, k3, k3, q, lse, q, k3, k3) == ffi.ERR_SHAPE                       # 4 query heads over 3 kv heads
+    assert call(q, q, k, tens((B, Hkv, N + 1, D), ffi.BF16), q, lse, q, k, k) == ffi.ERR_SHAPE
+    assert call(q, q, k, tens((B, Hkv, N, D), ffi.F32), q, lse, q, k, k) == ffi.ERR_DTYPE  # one dtype for all
+    assert call(q, q, k, k, q, tens((B, Hq, N), ffi.BF16), q, k, k) == ffi.ERR_DTYPE       # lse is fp32
+    q32, k32 = tens((B, Hq, N, 32), ffi.BF16), tens((B, Hkv, N, 32), ffi.BF16)
+    assert call(q32, q32, k32, k32, q32, lse, q32, k32, k32) == ffi.ERR_UNSUPPORTED        # head dim 32
+    assert call(q, q, k, k, q, lse, q, k, k, ws=None) == ffi.ERR_WORKSPACE
+    assert call(q, q, k, k, q, lse, q, k, k, ws_bytes=16) == ffi.ERR_WORKSPACE
+    off = tens((B, Hq, N, D), ffi.BF16, ptr=0x10008)                                       # rows not 16-byte aligned
+    assert call(q, off, k, k, q, lse, q, k, k) == ffi.ERR_ALIGN
+    narrow = tens((B, Hq, N, D), ffi.BF16, strides=[Hq * N * 32, N * 32, 32, 1])           # rows overlap: stride < D
+    assert call(q, narrow, k, k, q, lse, q, k, k) == ffi.ERR_STRIDE
+    inner = tens((B, Hq, N, D), ffi.BF16, strides=[Hq * N * D * 2, N * D * 2, D * 2, 2])   # innermost stride != 1
+    assert call(q, inner, k, k, q, lse, q, k, k) == ffi.ERR_STRIDE
+    empty = tens((B, Hq, 0, D), ffi.BF16)
+    ek, el = tens((B, Hkv, 0, D), ffi.BF16), tens((B, Hq, 0), ffi.F32)
+    assert call(empty, empty, ek, ek, empty, el, empty, ek, ek) == 0                       # nothing to do
+
+
 def test_adapter_host_side_checks():
     exe = os.path.join(ROOT, "tests", "cpp", "adapter_test")
     if not os.path.exists(exe):
