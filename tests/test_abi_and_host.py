@@ -149,6 +149,41 @@ def test_backward_validation_that_needs_no_gpu(ffi):
     assert call(empty, empty, ek, ek, empty, el, empty, ek, ek) == 0                       # nothing to do
 
 
+def test_cache_descriptor_validation_that_needs_no_gpu(ffi):
+    # check_cache (behind every cache entry point) through vsp_kv_cache_reset, plus the argument checks of
+    # vsp_kv_read and vsp_seq_lens_advance that come before any launch
+    def cache(fmt=None, **kw):
+        c = ffi.VspKVCache()
+        c.format, c.B, c.Hkv, c.S_max, c.D = ffi.KV_BF16 if fmt is None else fmt, 2, 2, 256, 128
+        c.k = c.v = c.k_scale = c.v_scale = 0x10000
+        for key, val in kw.items():
+            setattr(c, key, val)
+        return c
+
+    reset = lambda c: ffi.lib.vsp_kv_cache_reset(C.byref(c), None)
+    assert reset(cache(len=257)) == ffi.ERR_ARG                      # length beyond the capacity
+    assert reset(cache(D=96)) == ffi.ERR_UNSUPPORTED                 # bf16 / q8_0 planes exist for D 64 and 128
+    assert reset(cache(fmt=ffi.KV_F32, D=6)) == ffi.ERR_UNSUPPORTED
+    assert reset(cache(k=0x10008)) == ffi.ERR_ALIGN
+    assert reset(cache(fmt=ffi.KV_Q8_0, k_scale=None)) == ffi.ERR_NULL
+    paged = dict(page_table=0x30000, page_tokens=64, pages_per_seq=4, n_pages=10)
+    assert reset(cache(fmt=ffi.KV_F32, **paged)) == ffi.ERR_UNSUPPORTED          # paging is for the compact formats
+    assert reset(cache(**dict(paged, page_tokens=48))) == ffi.ERR_ARG            # pages are multiples of 64 tokens
+    assert reset(cache(**dict(paged, pages_per_seq=3))) == ffi.ERR_ARG           # pages_per_seq * page_tokens == S_max
+    assert reset(cache(page_tokens=64)) == ffi.ERR_ARG                           # paging fields without a table
+    c = cache()
+    assert ffi.lib.vsp_kv_read(C.byref(c), 200, 100, None, None, None) == ffi.ERR_ARG    # past the capacity
+    assert ffi.lib.vsp_kv_read(C.byref(c), 0, 10, None, None, None) == ffi.ERR_NULL      # neither output given
+    t = ffi.VspTensor()
+    t.ndim, t.dtype = 4, ffi.BF16
+    for i, n in enumerate((2, 2, 11, 128)):
+        t.shape[i] = n
+    assert ffi.lib.vsp_kv_read(C.byref(c), 0, 10, C.byref(t), None, None) == ffi.ERR_NUMEL
+    assert ffi.lib.vsp_seq_lens_advance(None, None, 1, -1, 8, None) == ffi.ERR_ARG
+    assert ffi.lib.vsp_seq_lens_advance(None, None, 1, 0, 8, None) == 0
+    assert ffi.lib.vsp_seq_lens_advance(None, None, 1, 4, 8, None) == ffi.ERR_NULL
+
+
 def test_adapter_host_side_checks():
     exe = os.path.join(ROOT, "tests", "cpp", "adapter_test")
     if not os.path.exists(exe):
