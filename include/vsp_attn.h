@@ -249,7 +249,11 @@ int vsp_seq_lens_advance(int32_t* seq_lens, const int32_t* n_new, int32_t T, int
  * q, out: [B,Hq,1,D] bf16 (fp32 for a VSP_KV_F32 cache).  Every query head attends, unmasked, to
  * positions [0, L_b) of its kv head, L_b = seq_lens[b] (device int32[B]) or cache->len when
  * seq_lens is NULL.  L_b == 0 yields zeros.  max_len: host-side upper bound of L_b used to size the
- * launch (0 = cache->len if seq_lens is NULL, else S_max).
+ * launch and the workspace (0 = cache->len if seq_lens is NULL, else S_max).  The bound is enforced: with
+ * seq_lens == NULL, cache->len > max_len > 0 is VSP_ERR_ARG; device-side lengths cannot be checked on the
+ * host, so seq_lens[b] is clamped to [0, min(max_len, S_max)] inside the kernels and a row longer than the
+ * bound attends to its first max_len keys only (the reference's cache length never exceeds what its
+ * buffers were sized for, src/nn/transformer.cpp:73-92).
  * Split-K over the context: partial (m, l, acc) per (b, head, split) go to `workspace`
  * (>= vsp_attn_decode_workspace_bytes), then a combine kernel reduces them in a fixed order
  * (bitwise run-to-run deterministic). */

@@ -191,3 +191,39 @@ def test_decode_argument_errors(va):
     assert e.value.status == 2
     out = va.decode_attention(q, c)  # empty cache: zeros, like an empty sum
     assert not out.float().any()
+
+
+@pytest.mark.parametrize("fmt", ["bf16", "q8_0", "f32"])
+def test_device_lengths_above_the_host_bound_are_clamped_inside_the_workspace(va, fmt):
+    # max_len sizes the grid, the split count and the workspace; a device-side length above it must neither write
+    # outside the partials' rows nor change another row's result: the row attends to its first max_len keys.
+    B, Hq, Hkv, S, D, max_len = 2, 8, 2, 1024, 128 if fmt != "f32" else 64, 512
+    lens = [300, 1024]  # the LAST row exceeds the bound: unclamped, its splits 2 and 3 would land past the buffer
+    q, k, v = I.qkv(47, B, Hq, Hkv, 1, S, D)
+    if fmt != "f32":
+        q = O.bf16_round(q)
+    c = fill_cache(va, fmt, k, v)
+    if fmt == "bf16":
+        kc, vc = O.bf16_round(k), O.bf16_round(v)
+    elif fmt == "q8_0":
+        kc, vc = O.q8_0_dequantize(*O.q8_0_quantize(k)), O.q8_0_dequantize(*O.q8_0_quantize(v))
+    else:
+        kc, vc = k, v
+    need = va._ffi.lib.vsp_attn_decode_workspace_bytes(B, Hq, D, max_len)
+    assert need == B * Hq * (max_len // 256) * (D + 2) * 4  # 256-token splits here: the whole workspace is in use
+    guard = 1 << 20
+    ws = torch.full((need + guard,), 0x5A, dtype=torch.uint8, device=G.dev())
+    sl = torch.tensor(lens, dtype=torch.int32, device=G.dev())
+    qd = G.f32_dev(q) if fmt == "f32" else G.to_bf16_dev(q)
+    out = va.decode_attention(qd, c, seq_lens=sl, max_len=max_len, workspace=ws[:need])
+    torch.cuda.synchronize()
+    assert bool((ws[need:] == 0x5A).all()), "partials written past the workspace"
+    want = oracle_decode(q, kc, vc, [300, max_len])
+    if fmt == "f32":
+        G.assert_f32_close(out.cpu().numpy(), want, "clamped decode")
+    else:
+        G.assert_bf16_close(G.bf16_to_np(out), want, "clamped decode")
+    # host-side length above the bound: a caller error, reported before any launch
+    with pytest.raises(va.VspError) as e:
+        va.decode_attention(qd, c, max_len=max_len)  # cache.len == 1024
+    assert e.value.status == va._ffi.ERR_ARG

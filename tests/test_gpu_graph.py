@@ -51,7 +51,8 @@ def test_decode_step_replays_bit_identically(va, fmt):
     sv = torch.empty(B, Hkv, 1, D, device=G.dev())
     q_rot = torch.empty(B, Hq, 1, D, device=G.dev(), dtype=torch.bfloat16)
     out = torch.empty_like(q_rot)
-    va.decode_attention(q_rot, cg, seq_lens=cg.seq_lens, max_len=cg.upper, out=out)  # sizes the shared workspace
+    # the graph keeps the workspace's address, so the test owns it (the per-stream default refuses to grow in capture)
+    ws = torch.empty(va._ffi.lib.vsp_attn_decode_workspace_bytes(B, Hq, D, S_max), dtype=torch.uint8, device=G.dev())
     lens0 = cg.seq_lens.clone()
     torch.cuda.synchronize()
     side = torch.cuda.Stream()
@@ -60,7 +61,7 @@ def test_decode_step_replays_bit_identically(va, fmt):
         with torch.cuda.graph(graph, stream=side):
             cg.rope_update(sq, sk, sv, 0, rope, start_pos_dev=cg.seq_lens, out=q_rot)
             cg._advance(None, 1, sq)
-            va.decode_attention(q_rot, cg, seq_lens=cg.seq_lens, max_len=cg.upper, out=out)
+            va.decode_attention(q_rot, cg, seq_lens=cg.seq_lens, max_len=cg.upper, out=out, workspace=ws)
     torch.cuda.synchronize()
     cg.seq_lens.copy_(lens0)  # capture does not execute; make sure the lengths are the prompt lengths
     for i, (q, k, v) in enumerate(toks):

@@ -248,28 +248,36 @@ _WS = {}
 
 
 def _workspace(device, nbytes):
-    key = (device.type, device.index)
+    """Grow-only split-K workspace, one per (device, stream): calls on different streams never share partials.
+    A buffer that a captured graph may hold must not be replaced, so growth during stream capture is refused:
+    size it with one eager call (or pass `workspace=`) before capturing."""
+    key = (device.type, device.index, torch.cuda.current_stream(device).cuda_stream)
     ws = _WS.get(key)
     if ws is None or ws.numel() < nbytes:
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("decode_attention: the workspace would have to grow during stream capture; "
+                               "run one eager call of this size first, or pass workspace=")
         ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
         _WS[key] = ws
     return ws
 
 
-def decode_attention(q, cache, seq_lens=None, max_len=0, scale=None, out=None):
-    """One new token per sequence attending to the cache: q [B,Hq,1,D] -> [B,Hq,1,D]."""
+def decode_attention(q, cache, seq_lens=None, max_len=0, scale=None, out=None, workspace=None):
+    """One new token per sequence attending to the cache: q [B,Hq,1,D] -> [B,Hq,1,D].
+    workspace: a caller-owned uint8 device tensor for the split-K partials (default: a cached one per stream)."""
     c = cache._c
     if scale is None:
         scale = 1.0 / math.sqrt(q.shape[-1])  # src/nn/functional.cpp:403
     if out is None:
         out = torch.empty_like(q)
-    bound = max_len or (c.S_max if seq_lens is not None else c.len)
-    nbytes = lib.vsp_attn_decode_workspace_bytes(q.shape[0], q.shape[1], q.shape[3], max(int(bound), 1))
-    ws = _workspace(q.device, nbytes)
+    if workspace is None:
+        bound = max_len or (c.S_max if seq_lens is not None else c.len)
+        nbytes = lib.vsp_attn_decode_workspace_bytes(q.shape[0], q.shape[1], q.shape[3], max(int(bound), 1))
+        workspace = _workspace(q.device, nbytes)
     dq, do = _desc(q), _desc(out)
     sl = C.c_void_p(seq_lens.data_ptr()) if seq_lens is not None else None
     check(lib.vsp_attn_decode(C.byref(dq), C.byref(c), sl, int(max_len), C.byref(do), float(scale),
-                              C.c_void_p(ws.data_ptr()), ws.numel(), _stream(q)))
+                              C.c_void_p(workspace.data_ptr()), workspace.numel(), _stream(q)))
     return out
 
 

@@ -38,7 +38,9 @@ struct DecodeArgs {
     int32_t len;              // used when seq_lens == nullptr
     int32_t B, Hq, Hkv, n_rep;
     int64_t S;  // physical token capacity of the planes
-    int32_t S_max;  // logical capacity; lengths are clamped to it
+    int32_t S_max;  // logical capacity
+    int32_t L_cap;  // min(S_max, the host's upper bound of the lengths): every length is clamped to it, because the
+                    // grid, max_splits and the workspace are sized from that bound
     int32_t chunk;
     int32_t max_splits;
     float scale_log2;  // scale * log2(e)
@@ -96,7 +98,7 @@ __device__ inline uint4 mask_tail_u16x8(uint4 v, int nvalid) {
 // interleaved with real work and cost launch slots all the way through).
 __device__ inline bool locate_work(const DecodeArgs& a, int item, int lane, int& b, int& split, int& L) {
     if (!a.seq_lens) {
-        L = min(a.len, a.S_max);
+        L = min(a.len, a.L_cap);
         const int ns = (L + a.chunk - 1) / a.chunk;
         if (ns == 0 || item >= ns * a.B) return false;
         b = item / ns;
@@ -106,7 +108,7 @@ __device__ inline bool locate_work(const DecodeArgs& a, int item, int lane, int&
     int base = 0;
     for (int b0 = 0; b0 < a.B; b0 += 64) {
         const int bb = b0 + lane;
-        const int Lb = bb < a.B ? min(max(a.seq_lens[bb], 0), a.S_max) : 0;
+        const int Lb = bb < a.B ? min(max(a.seq_lens[bb], 0), a.L_cap) : 0;
         const int ns = (Lb + a.chunk - 1) / a.chunk;
         int incl = ns;
 #pragma unroll
@@ -588,9 +590,9 @@ template <typename OutT>
 __global__ void __launch_bounds__(256) decode_combine_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
                                                              const int32_t* __restrict__ seq_lens, int32_t len, int32_t chunk,
                                                              int32_t max_splits, int32_t Hq, int32_t D, OutT* __restrict__ out,
-                                                             int64_t so_b, int64_t so_h, int32_t S_max) {
+                                                             int64_t so_b, int64_t so_h, int32_t L_cap) {
     const int hq = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
-    const int L = min(seq_lens ? seq_lens[b] : len, S_max);
+    const int L = min(max(seq_lens ? seq_lens[b] : len, 0), L_cap);  // the producers' clamp (locate_work)
     const int ns = min((L + chunk - 1) / chunk, max_splits);
     const int64_t row0 = ((int64_t)b * Hq + hq) * max_splits;
     float M = -INFINITY;
@@ -644,13 +646,6 @@ int device_cu_count() {
 // upper bound of the lengths).  The quantised kernel has the heavier per-item cost and the lighter
 // stream, hence its larger cap.  Workspace sizing assumes >= 256.
 int pick_chunk(int format, int64_t B, int64_t Hkv, int64_t max_len) {
-    static int forced = -1;
-    if (forced < 0) {
-        const char* e = getenv("VSP_DECODE_CHUNK");
-        forced = e ? atoi(e) : 0;
-        if (forced != 0 && (forced < 256 || forced % 256 != 0 || forced > 16384)) forced = 0;
-    }
-    if (forced > 0) return forced;
     const int64_t want = 4LL * device_cu_count();
     const int cap = format == VSP_KV_Q8_0 ? 8192 : 1024;
     for (int chunk = cap; chunk > 256; chunk >>= 1) {
@@ -664,16 +659,11 @@ int pick_chunk(int format, int64_t B, int64_t Hkv, int64_t max_len) {
 
 using namespace vsp;
 
-extern "C" {
+namespace {
 
-size_t vsp_attn_decode_workspace_bytes(int32_t B, int32_t Hq, int32_t D, int32_t max_len) {
-    if (B <= 0 || Hq <= 0 || D <= 0 || max_len <= 0) return 0;
-    const int64_t splits = ceil_div(max_len, 256);
-    return (size_t)((int64_t)B * Hq * splits * (D + 2) * 4);
-}
-
-int vsp_attn_decode(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, int32_t max_len,
-                    vsp_tensor* out, float scale, void* workspace, size_t workspace_bytes, void* stream) {
+// vsp_attn_decode: validation, split sizing and the two launches.
+int decode_impl(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, int32_t max_len, vsp_tensor* out,
+                float scale, void* workspace, size_t workspace_bytes, void* stream) {
     if (!q || !out) return VSP_ERR_NULL;
     int rc = check_kv_cache(cache);
     if (rc != VSP_OK) return rc;
@@ -695,6 +685,9 @@ int vsp_attn_decode(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_
     const int esz = q->dtype == VSP_F32 ? 4 : 2;
     if (!is_aligned16(q->data) || (q->stride[0] * esz) % 16 || (q->stride[1] * esz) % 16) return VSP_ERR_ALIGN;
     if (max_len < 0 || max_len > cache->S_max) return VSP_ERR_ARG;
+    // a host-side length above the bound the launch is sized from is a caller error; device-side lengths
+    // cannot be read here and are clamped to the bound inside the kernels instead
+    if (!seq_lens && max_len > 0 && cache->len > max_len) return VSP_ERR_ARG;
     if (max_len == 0) max_len = seq_lens ? cache->S_max : cache->len;
     hipStream_t st = (hipStream_t)stream;
 
@@ -721,6 +714,7 @@ int vsp_attn_decode(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_
     a.n_rep = n_rep;
     a.S = cache->page_table ? cache->page_tokens : kv_s_pad(cache->format, cache->S_max);
     a.S_max = cache->S_max;
+    a.L_cap = max_len < cache->S_max ? max_len : cache->S_max;
     a.page_table = cache->page_table;
     a.page_tokens = cache->page_tokens;
     a.pages_per_seq = cache->pages_per_seq;
@@ -757,17 +751,33 @@ int vsp_attn_decode(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_
         rc = check_launch();
         if (rc != VSP_OK) return rc;
     }
+    // with max_len == 0 every row is empty: the combine kernel reads nothing and writes zeros
     dim3 cgrid((unsigned)Hq, (unsigned)B);
     const int cthreads = D <= 64 ? 64 : (D <= 128 ? 128 : 256);
     if (out->dtype == VSP_F32)
         hipLaunchKernelGGL(decode_combine_kernel<float>, cgrid, dim3(cthreads), 0, st, a.ws_o, a.ws_ml, seq_lens,
                            max_len > 0 ? cache->len : 0, chunk, max_splits, (int)Hq, (int)D, (float*)out->data,
-                           out->stride[0], out->stride[1], cache->S_max);
+                           out->stride[0], out->stride[1], a.L_cap);
     else
         hipLaunchKernelGGL(decode_combine_kernel<uint16_t>, cgrid, dim3(cthreads), 0, st, a.ws_o, a.ws_ml, seq_lens,
                            max_len > 0 ? cache->len : 0, chunk, max_splits, (int)Hq, (int)D, (uint16_t*)out->data,
-                           out->stride[0], out->stride[1], cache->S_max);
+                           out->stride[0], out->stride[1], a.L_cap);
     return check_launch();
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t vsp_attn_decode_workspace_bytes(int32_t B, int32_t Hq, int32_t D, int32_t max_len) {
+    if (B <= 0 || Hq <= 0 || D <= 0 || max_len <= 0) return 0;
+    const int64_t splits = ceil_div(max_len, 256);
+    return (size_t)((int64_t)B * Hq * splits * (D + 2) * 4);
+}
+
+int vsp_attn_decode(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, int32_t max_len,
+                    vsp_tensor* out, float scale, void* workspace, size_t workspace_bytes, void* stream) {
+    return decode_impl(q, cache, seq_lens, max_len, out, scale, workspace, workspace_bytes, stream);
 }
 
 }  // extern "C"
