@@ -261,6 +261,18 @@ size_t vsp_attn_decode_workspace_bytes(int32_t B, int32_t Hq, int32_t D, int32_t
 int vsp_attn_decode(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, int32_t max_len,
                     vsp_tensor* out, float scale, void* workspace, size_t workspace_bytes, void* stream);
 
+/* vsp_attn_decode for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments,
+ * validation, kernels and results (bit for bit) as vsp_attn_decode, minus the workspace: the split-K
+ * partials go to a fixed 32 MiB array that is part of the library's code object (one copy per GPU, held
+ * until the process ends), located on the first call on each device.  The call allocates and frees nothing.
+ * Calls whose partials need more than that -- B * Hq * ceil(max_len / chunk) * (D + 2) * 4 bytes, chunk being
+ * the split length the library picks (>= 256 tokens) -- return VSP_ERR_WORKSPACE: config 4 (B 32, 32 heads,
+ * D 128, max_len 32768) needs 17 MiB.  Every call on one GPU shares that GPU's array: calls that overlap in
+ * time on one GPU (different streams, different threads) race; serialise them or use vsp_attn_decode. */
+int vsp_attn_decode_noalloc(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, int32_t max_len,
+                            vsp_tensor* out, float scale, void* stream);
+
 /* ---- host-side, bit-exact format helpers (pure CPU; exported for tests and callers) ---- */
 uint16_t vsp_f32_to_bf16(float f);   /* include/vesper/core/half.h:162-173 */
 float vsp_bf16_to_f32(uint16_t b);   /* include/vesper/core/half.h:175-181 */

@@ -281,6 +281,18 @@ def decode_attention(q, cache, seq_lens=None, max_len=0, scale=None, out=None, w
     return out
 
 
+def decode_attention_noalloc(q, cache, out, seq_lens=None, max_len=0, scale=None):
+    """decode_attention through vsp_attn_decode_noalloc: the partials go to the library's fixed per-GPU array
+    and the call allocates nothing (`out` is the caller's).  Calls overlapping on one GPU race."""
+    if scale is None:
+        scale = 1.0 / math.sqrt(q.shape[-1])
+    dq, do = _desc(q), _desc(out)
+    sl = C.c_void_p(seq_lens.data_ptr()) if seq_lens is not None else None
+    check(lib.vsp_attn_decode_noalloc(C.byref(dq), C.byref(cache._c), sl, int(max_len), C.byref(do), float(scale),
+                                      _stream(q)))
+    return out
+
+
 def scaled_dot_product_attention(q, k, v, is_causal=False, dropout_p=0.0):
     """functional::scaled_dot_product_attention (src/nn/functional.cpp:370-422) on explicit tensors.
     The reference switches algorithm at T >= 512 for speed; here one kernel serves every T.

@@ -16,6 +16,8 @@
 // any cross-lane movement.  Online softmax in fp32, exp2 with the scale folded in.
 #include <stdlib.h>
 
+#include <mutex>
+
 #include "kv_layout.hpp"
 #include "vsp_common.hpp"
 
@@ -661,9 +663,43 @@ using namespace vsp;
 
 namespace {
 
-// vsp_attn_decode: validation, split sizing and the two launches.
+// Split-K partials for callers that cannot allocate (vsp_attn_decode_noalloc): one fixed array per GPU, part of
+// the library's code object, held until the process ends.  In host code the array's name is only a handle for
+// hipGetSymbolAddress; kernels and launches use the per-device address looked up through it.
+constexpr size_t kScratchBytes = 32u << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices];  // per device, filled on the first call on that device
+std::mutex g_scratch_mutex;
+
+// Address of the current device's copy of `scratch` (each GPU holds its own at its own address).
+int scratch_for_current_device(void** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) {
+        set_hip_error(e);
+        return VSP_ERR_LAUNCH;
+    }
+    if (dev < 0 || dev >= kMaxDevices) return VSP_ERR_ARG;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            set_hip_error(e);
+            return VSP_ERR_LAUNCH;
+        }
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return VSP_OK;
+}
+
+// Both decode entry points: validation, split sizing and the two launches.  `own_scratch` selects the
+// library's fixed per-device array instead of a caller workspace.
 int decode_impl(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, int32_t max_len, vsp_tensor* out,
-                float scale, void* workspace, size_t workspace_bytes, void* stream) {
+                float scale, void* workspace, size_t workspace_bytes, bool own_scratch, void* stream) {
     if (!q || !out) return VSP_ERR_NULL;
     int rc = check_kv_cache(cache);
     if (rc != VSP_OK) return rc;
@@ -694,7 +730,11 @@ int decode_impl(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* s
     const int chunk = max_len > 0 ? pick_chunk(cache->format, B, cache->Hkv, max_len) : 256;
     const int max_splits = max_len > 0 ? (int)ceil_div(max_len, chunk) : 1;
     const size_t need = (size_t)(B * Hq * max_splits * (D + 2) * 4);
-    if (max_len > 0) {
+    if (own_scratch) {
+        if (need > kScratchBytes) return VSP_ERR_WORKSPACE;
+        rc = scratch_for_current_device(&workspace);
+        if (rc != VSP_OK) return rc;
+    } else if (max_len > 0) {
         if (!workspace || workspace_bytes < need) return VSP_ERR_WORKSPACE;
         if (!is_aligned16(workspace)) return VSP_ERR_ALIGN;
     }
@@ -777,7 +817,12 @@ size_t vsp_attn_decode_workspace_bytes(int32_t B, int32_t Hq, int32_t D, int32_t
 
 int vsp_attn_decode(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, int32_t max_len,
                     vsp_tensor* out, float scale, void* workspace, size_t workspace_bytes, void* stream) {
-    return decode_impl(q, cache, seq_lens, max_len, out, scale, workspace, workspace_bytes, stream);
+    return decode_impl(q, cache, seq_lens, max_len, out, scale, workspace, workspace_bytes, false, stream);
+}
+
+int vsp_attn_decode_noalloc(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, int32_t max_len,
+                            vsp_tensor* out, float scale, void* stream) {
+    return decode_impl(q, cache, seq_lens, max_len, out, scale, nullptr, 0, true, stream);
 }
 
 }  // extern "C"
