@@ -439,6 +439,392 @@ __global__ void __launch_bounds__(256, 3) prefill_bf16_kernel(PrefillArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// Software-pipelined bf16 kernel, D = 128, dense K/V.  Same tiles, fragment layouts and arithmetic as
+// prefill_bf16_kernel; what changes is the order of work inside a wavefront.  Step tau of a wavefront issues, as
+// three independent instruction streams,
+//     S(tau+2) = K(tau+2) Q^T          8 MFMAs into the "next" score registers
+//     P(tau+1) = exp2(S(tau+1) - m)    the vector-ALU work, on scores finished one step earlier
+//     O       += V(tau)^T P(tau)       8 MFMAs with the P computed one step earlier
+// so no MFMA of a step waits for vector-ALU work of the same step and vice versa: the matrix pipe and the vector ALU
+// of one SIMD run side by side from a single wavefront's instruction stream.  The 16 MFMAs of a step are "slots";
+// each slot is followed by its share of the softmax instructions and by the LDS reads of the operand needed kLead
+// slots later (the reads run ahead across step boundaries).  Four ring slots per operand in LDS: the tiles a step
+// needs were requested three steps earlier and published by the barrier one step earlier, so neither the barrier nor
+// the global loads sit on a wavefront's critical path.
+// Vector-ALU instructions of one wavefront hardly overlap with MFMAs of ANOTHER wavefront on the same SIMD (a wavefront
+// of nothing but vector-ALU work gets about one instruction in per MFMA of its neighbour), while those that follow an
+// MFMA in the same instruction stream are nearly free; hence this structure, and the diet of the softmax stage:
+//   - scale * log2(e) is folded into Q once per workgroup, and -m (the row's reference maximum) enters as the C
+//     operand of the first QK^T MFMA, so the scores arrive as s' = s - m and P is a bare exp2;
+//   - the row sum uses plain adds (v_dot2c_f32_bf16 occupies the matrix pipe);
+//   - no row maximum per tile: m is raised only when the row sum shows that it has fallen behind (rare), and is
+//     kept integer-valued (log2 domain) so that the rescale factor is a power of two and the P tile that has been
+//     computed but not yet multiplied into O rescales exactly.
+// ---------------------------------------------------------------------------------------------
+constexpr int kLead = 6;  // LDS operand reads run this many MFMA slots ahead
+
+// MFMA slot order of a step: Q = a QK^T MFMA (k-step index), P = a PV MFMA (index p: key half p / 4, d block p % 4).
+// The QK chain finishes at slot 10, so that the row maximum of the new scores is taken under the last PV MFMAs.
+constexpr int kSlotIsQ[16] = {1, 1, 0, 1, 1, 0, 1, 1, 0, 1, 1, 0, 0, 0, 0, 0};
+constexpr int kSlotIdx[16] = {0, 1, 0, 2, 3, 1, 4, 5, 2, 6, 7, 3, 4, 5, 6, 7};
+constexpr int slot_reads(int s) { return kSlotIsQ[s & 15] ? 1 : 2; }
+// LDS reads issued after the operand of slot s and before the wait at slot s: those of slots s+1 .. s+kLead-1
+constexpr int reads_behind(int s) {
+    int n = 0;
+    for (int k = 1; k < kLead; ++k) n += slot_reads(s + k);
+    return n;
+}
+
+struct Frag {  // one MFMA A operand on its way from LDS
+    u32x4_t k;     // K rows (ds_read_b128)
+    uint2 t0, t1;  // V^T halves (two transposing reads)
+};
+
+template <int N>
+__device__ inline void frag_wait_k(u32x4_t& k) {
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(k) : "n"(N));
+}
+template <int N>
+__device__ inline void frag_wait_v(uint2& t0, uint2& t1) {
+    asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(t0), "+v"(t1) : "n"(N));
+}
+
+__global__ void __launch_bounds__(256, 2) prefill_bf16_pipe_kernel(PrefillArgs a) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the body uses device-only builtins
+    constexpr int D = 128;
+    constexpr int KS = D / 16;
+    constexpr int DB = D / 32;
+    constexpr int CPR = D / 8;
+    constexpr int RP = 256 / (2 * D);
+    constexpr int NR = 1024 / (2 * D);
+    constexpr int NGRP = kUnit / NR;
+    constexpr int NLD = NGRP / 4;
+    constexpr int SLOT = kUnit * D;
+    constexpr int SLOTB = 2 * SLOT;
+    constexpr int NRING = 4;
+    static_assert(KS == 8 && DB == 4 && NLD == 2, "written for D = 128");
+
+    // K ring (4 slots) | V ring (4 slots)
+    __shared__ __attribute__((aligned(1024))) uint16_t smem[2 * NRING * SLOT];
+    const uint32_t lds0 = lds_addr(smem);
+
+    const int nbh = a.B * a.Hq;
+    const int bid = blockIdx.x;
+    const int qt = a.n_qtiles - 1 - bid / nbh;
+    const int pos = bid % nbh;
+    int bh = pos;
+    const int ngroups = a.B * a.Hkv;
+    if ((ngroups & 7) == 0) {
+        const int xcd = pos & 7, slot = pos >> 3;
+        const int grp = xcd + 8 * (slot / a.n_rep);
+        bh = grp * a.n_rep + slot % a.n_rep;
+    }
+    const int b = bh / a.Hq, hq = bh % a.Hq, kvh = hq / a.n_rep;
+    const int L = a.L;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ql = lane & 31, h = lane >> 5;
+    const int q0 = qt * kBM + wave * 32;
+    const int off = L - a.T;
+    const int qrow = min(q0 + ql, a.T - 1);
+
+    const uint16_t* Qp = (const uint16_t*)a.q + (int64_t)b * a.sq[0] + (int64_t)hq * a.sq[1];
+    const uint16_t* Kp = (const uint16_t*)a.k + (int64_t)b * a.sk[0] + (int64_t)kvh * a.sk[1];
+    const uint16_t* Vp = (const uint16_t*)a.v + (int64_t)b * a.sv[0] + (int64_t)kvh * a.sv[1];
+
+    uint4 qraw[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qraw[ks] = *(const uint4*)(Qp + (int64_t)qrow * a.sq[2] + 16 * ks + 8 * h);
+    bf16x8_t qf[KS];
+    auto prescale_q = [&]() {
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        const uint4 w = qraw[ks];
+        // fold scale * log2(e) (and the sign of a negative scale) into Q: one more bf16 rounding of Q
+        const float c = a.negate_q ? -a.scale_log2 : a.scale_log2;
+        const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+        uint32_t o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            o[i] = cvt_pk_bf16(__builtin_bit_cast(float, ww[i] << 16) * c, __builtin_bit_cast(float, ww[i] & 0xffff0000u) * c);
+        qf[ks] = __builtin_bit_cast(bf16x8_t, uint4{o[0], o[1], o[2], o[3]});
+    }
+    };
+
+    const int wg_qmax = min(qt * kBM + kBM - 1, a.T - 1);
+    const int kv_end_wg = a.causal ? min(L, wg_qmax + off + 1) : L;
+    const int n_tiles = (kv_end_wg + kUnit - 1) / kUnit;  // tiles the workgroup loads
+    const int wave_qmax = min(q0 + 31, a.T - 1);
+    const int kv_end_wave = (q0 < a.T) ? (a.causal ? min(L, wave_qmax + off + 1) : L) : 0;
+    const int nt_w = (kv_end_wave + kUnit - 1) / kUnit;  // tiles this wavefront uses
+    // first tile of this wavefront that needs the mask (straddles the diagonal or the end of the context)
+    int first_masked = min(nt_w, L / kUnit);
+    if (a.causal) first_masked = min(first_masked, q0 + off - 31 < 0 ? 0 : (q0 + off - 31) / kUnit + 1);
+    const int n_fast = max(0, first_masked - 2);  // steps [0, n_fast): all three stages active, no mask
+    const int n_mid = max(0, nt_w - 2);           // steps [0, n_mid): all three stages active
+
+    f32x16_t acc[DB];
+#pragma unroll
+    for (int i = 0; i < DB; ++i)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) acc[i][j] = 0.f;
+    float m_ref = -INFINITY;
+    float l = 0.f;
+
+    // global -> LDS, as in prefill_bf16_kernel
+    const int ld_row = lane / CPR, ld_pos = lane % CPR;
+    uint32_t voffK[NLD], voffV[NLD];
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+        const int r = NR * (wave + 4 * i) + ld_row;
+        voffK[i] = (uint32_t)r * (uint32_t)a.sk[2] * 2u + 16u * (uint32_t)(ld_pos ^ ((r / RP) % CPR));
+        voffV[i] = (uint32_t)r * (uint32_t)a.sv[2] * 2u + 16u * (uint32_t)(ld_pos ^ (((r / RP) % (CPR / 4)) << 2));
+    }
+    const int64_t rowK = a.sk[2] * 2, rowV = a.sv[2] * 2;
+    auto load_k_tile = [&](int t, int slot) {
+        const int key0 = t * kUnit;
+        __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)Kp + (int64_t)key0 * rowK), 0, (int)((int64_t)(L - key0) * rowK), 0x00020000);
+        uint16_t* dst = smem + slot * SLOT;
+#pragma unroll
+        for (int i = 0; i < NLD; ++i)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (__attribute__((address_space(3))) void*)(dst + (wave + 4 * i) * 512), 16, voffK[i], 0, 0, 0);
+    };
+    auto load_v_tile = [&](int t, int slot) {
+        const int key0 = t * kUnit;
+        __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)Vp + (int64_t)key0 * rowV), 0, (int)((int64_t)(L - key0) * rowV), 0x00020000);
+        uint16_t* dst = smem + (NRING + slot) * SLOT;
+#pragma unroll
+        for (int i = 0; i < NLD; ++i)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (__attribute__((address_space(3))) void*)(dst + (wave + 4 * i) * 512), 16, voffV[i], 0, 0, 0);
+    };
+
+    // loop-constant LDS read addresses (ring slot 0 of each operand; the slot is an immediate offset)
+    const int kswz = (ql / RP) % CPR;
+    uint32_t kaddr[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) kaddr[ks] = lds0 + 2u * (uint32_t)(ql * D + 8 * ((2 * ks + h) ^ kswz));
+    const int i16 = lane & 15;
+    const int vswz = ((i16 >> 2) / RP) % (CPR / 4);
+    const int v_lane_off = (4 * h + (i16 >> 2)) * D + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+    uint32_t va[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) va[db] = lds0 + 2u * (uint32_t)v_lane_off + 64u * (uint32_t)(db ^ vswz);
+
+    Frag fr[16];         // operand of MFMA slot s of the current step (slots < kLead: already requested)
+    // Scores are kept as S' = s * scale * log2(e) - m: the factor is folded into Q (below), and -m, the row's reference
+    // maximum, enters as the C operand of the first QK^T MFMA from a tile of 16 registers that all hold -m.
+    f32x16_t sb[2];      // step tau finishes S'(tau+2) in sb[tau & 1] and consumes S'(tau+1) from sb[(tau+1) & 1]
+    uint32_t pb[2][8];   // packed bf16 P: step tau consumes P(tau) from pb[tau & 1] and writes P(tau+1) to pb[(tau+1) & 1]
+    f32x16_t negm;       // every element = -m_ref of this lane's query
+#pragma unroll
+    for (int j = 0; j < 16; ++j) negm[j] = 0.f;
+    m_ref = 0.f;  // "no reference yet": the first tile sets it
+
+    // Request the operand of MFMA slot S of the step whose ring slot is RS.
+    auto request = [&](auto s_c, auto rs_c) {
+        constexpr int S = decltype(s_c)::value;
+        constexpr int RS = decltype(rs_c)::value;
+        if constexpr (kSlotIsQ[S]) {
+            constexpr int ks = kSlotIdx[S];
+            fr[S].k = lds_read_b128_asm<RS * SLOTB>(kaddr[ks]);
+        } else {
+            constexpr int p = kSlotIdx[S], j = p / 4, db = p % 4;
+            constexpr int VOFF = (NRING + RS) * SLOTB + 16 * j * D * 2;
+            fr[S].t0 = lds_read_tr16_b64_asm<VOFF>(va[db]);
+            fr[S].t1 = lds_read_tr16_b64_asm<VOFF + 8 * D * 2>(va[db]);
+        }
+    };
+
+    // One step.  PH = tau & 3 (ring slot of the step's tiles: K(tau+2), V(tau)).  MODE 0: all three stages are active
+    // and the new scores need no mask, so the body is one straight line of code; 1: the same with the mask applied
+    // under one wavefront-uniform branch; 2: every stage guarded (the first and last steps of a wavefront).
+    auto step = [&](int tau, auto ph_c, auto fast_c) {
+        constexpr int PH = decltype(ph_c)::value;
+        constexpr int MODE = decltype(fast_c)::value;
+        constexpr bool FAST = MODE < 2;     // all three stages active: no per-slot guards
+        constexpr bool MASK = MODE > 0;     // the new scores may need the mask
+        constexpr bool FIRST = MODE == 4;   // step -1: the softmax stage sees tile 0 and sets the reference
+        f32x16_t& s_cur = sb[(PH + 1) & 1];
+        f32x16_t& s_nxt = sb[PH & 1];
+        uint32_t(&p_cur)[8] = pb[PH & 1];
+        uint32_t(&p_nxt)[8] = pb[(PH + 1) & 1];
+
+        if constexpr (MODE == 3) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");  // first step: K(1) has landed
+        else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");  // the tiles of step tau+1 have landed; those of tau+2 may be in flight
+        __builtin_amdgcn_s_barrier();  // waits are explicit: no fence, which would drain every load in flight
+        // always four loads per wavefront and step, so that the vmcnt arithmetic holds: past the end the tile index is
+        // clamped (the rows fall outside the buffer bound and arrive as zeros, or re-read the last tile; never consumed)
+        if constexpr (MODE != 3) {
+            load_k_tile(min(tau + 5, n_tiles - 1), (PH + 3) & 3);
+            load_v_tile(min(tau + 3, n_tiles - 1), (PH + 3) & 3);
+        }
+
+        const bool qk_on = FAST || (tau + 2 < nt_w);
+        const bool sm_on = FAST || (tau + 1 >= 0 && tau + 1 < nt_w);
+        const bool pv_on = FAST || (tau >= 0 && tau < nt_w);
+
+        float es[16];
+        float lsum = 0.f, lsum2 = 0.f;
+        // instruction i of the 32 that turn s_cur into p_nxt: per pair of scores 2 exp2, 1 pack, and the row sum.
+        // Steady-state steps sum the fp32 values with plain adds (a dot2 occupies the matrix pipe); against the sum of
+        // the bf16-rounded P that the PV MFMAs consume this is zero-mean rounding noise of relative size
+        // 2^-9 / sqrt(keys), and such steps only exist in contexts of more than a hundred keys.  The first and last
+        // steps of a wavefront sum the rounded values themselves (packed dot product against (1, 1)), so that short
+        // contexts are normalised by exactly what was accumulated (a single key reproduces V bit for bit).
+        auto softmax_op = [&](auto i_c) {
+            constexpr int i = decltype(i_c)::value, p = i / 4, k = i % 4;
+            if constexpr (k < 2) es[2 * p + k] = __builtin_amdgcn_exp2f(s_cur[2 * p + k]);
+            else if constexpr (k == 2) p_nxt[p] = cvt_pk_bf16(es[2 * p], es[2 * p + 1]);
+            else if constexpr (FAST && !MASK) { lsum += es[2 * p]; lsum2 += es[2 * p + 1]; }
+            else lsum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, p_nxt[p]), __builtin_bit_cast(bf16x2_t, 0x3f803f80u), lsum, false);
+        };
+
+        static_for<16>([&](auto s_c) {
+            constexpr int S = decltype(s_c)::value;
+            // ---- the MFMA of this slot
+            if constexpr (kSlotIsQ[S]) {
+                constexpr int ks = kSlotIdx[S];
+                frag_wait_k<reads_behind(S)>(fr[S].k);
+                if (qk_on) {
+                    if constexpr (ks == 0) s_nxt = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, fr[S].k), qf[ks], negm, 0, 0, 0);
+                    else s_nxt = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, fr[S].k), qf[ks], s_nxt, 0, 0, 0);
+                }
+            } else {
+                constexpr int p = kSlotIdx[S], j = p / 4, db = p % 4;
+                frag_wait_v<reads_behind(S)>(fr[S].t0, fr[S].t1);
+                if (pv_on) {
+                    const bf16x8_t vf = __builtin_bit_cast(bf16x8_t, uint4{fr[S].t0.x, fr[S].t0.y, fr[S].t1.x, fr[S].t1.y});
+                    const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, uint4{p_cur[4 * j], p_cur[4 * j + 1], p_cur[4 * j + 2], p_cur[4 * j + 3]});
+                    acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf, acc[db], 0, 0, 0);
+                }
+            }
+            // ---- the operand of the slot kLead ahead (next step's tiles once the index wraps)
+            if constexpr (S + kLead < 16) request(std::integral_constant<int, S + kLead>{}, std::integral_constant<int, PH>{});
+            else request(std::integral_constant<int, S + kLead - 16>{}, std::integral_constant<int, (PH + 1) & 3>{});
+            // ---- this slot's share of the vector-ALU work
+            if constexpr (!FIRST) {
+                if (sm_on) static_for<2>([&](auto k_c) { softmax_op(std::integral_constant<int, 2 * S + decltype(k_c)::value>{}); });
+            }
+            if constexpr (MASK && S == 12) {
+                if (qk_on) {
+                    const int k0 = (tau + 2) * kUnit;
+                    if ((a.causal && k0 + kUnit - 1 > q0 + off) || (k0 + kUnit > L)) {
+                        const int q_abs = q0 + ql + off;
+                        const int lim = a.causal ? min(q_abs, L - 1) : L - 1;
+#pragma unroll
+                        for (int v = 0; v < 16; ++v)
+                            if (k0 + 8 * (v >> 2) + 4 * h + (v & 3) > lim) s_nxt[v] = -INFINITY;
+                    }
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        if (sm_on) {
+            // A reference that has fallen behind shows in the row sum: below 2^10 no P of the tile exceeds 2^10, far
+            // from overflow; otherwise (rare; and always for the first tile, which has no reference yet) take the true
+            // maximum of these scores, raise the reference to an integer at or above it (alpha is then a power of
+            // two, so everything computed against the old reference rescales exactly) and redo this tile's P.
+            constexpr bool first = FIRST;
+            if (first || __any(!(lsum + lsum2 < 1024.f))) {
+                float mx = s_cur[0];
+#pragma unroll
+                for (int v = 1; v < 16; ++v) mx = fmaxf(mx, s_cur[v]);
+                mx = half_swap_max(mx);
+                float delta = (mx == -INFINITY) ? 0.f : ceilf(mx);  // raise (first tile: set) the reference by delta
+                if (!first) delta = fmaxf(delta, 0.f);
+                if constexpr (!first) {  // nothing has been accumulated before the first tile
+                    const float alpha = __builtin_amdgcn_exp2f(-delta);
+                    l *= alpha;
+#pragma unroll
+                    for (int i = 0; i < DB; ++i)
+#pragma unroll
+                        for (int j = 0; j < 16; ++j) acc[i][j] *= alpha;
+                }
+                lsum = lsum2 = 0.f;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) s_cur[v] -= delta;
+                static_for<32>([&](auto i_c) { softmax_op(i_c); });
+                if (qk_on) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) s_nxt[v] -= delta;  // finished this step against the old reference
+                }
+                m_ref += delta;
+#pragma unroll
+                for (int j = 0; j < 16; ++j) negm[j] = -m_ref;
+            }
+            l += lsum + lsum2;
+        }
+    };
+
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    using I3 = std::integral_constant<int, 3>;
+    using Fast = std::integral_constant<int, 0>;
+    using Mid = std::integral_constant<int, 1>;
+    using Slow = std::integral_constant<int, 2>;
+    using First = std::integral_constant<int, 3>;   // step -2: Slow, and the tiles three steps ahead were requested by the prologue
+    using Second = std::integral_constant<int, 4>;  // step -1: Slow, and its softmax stage sets the reference from tile 0
+
+    // prologue: the tiles of steps -2 and -1 (K(0), K(1)) are requested here, published by the barrier below
+    load_k_tile(0, 2);
+    load_k_tile(min(1, n_tiles - 1), 3);
+    // tiles of steps 0 and 1 (K(2), V(0), K(3), V(1)); from step -1 on every step requests the tiles three steps ahead
+    load_k_tile(min(2, n_tiles - 1), 0);
+    load_v_tile(0, 0);
+    load_k_tile(min(3, n_tiles - 1), 1);
+    load_v_tile(min(1, n_tiles - 1), 1);
+    prescale_q();
+    asm volatile("s_waitcnt vmcnt(10)" ::: "memory");  // K(0) has landed
+    __builtin_amdgcn_s_barrier();  // waits are explicit: no fence, which would drain every load in flight
+    static_for<kLead>([&](auto s_c) { request(s_c, I2{}); });
+
+    step(-2, I2{}, First{});
+    step(-1, I3{}, Second{});
+    int tau = 0;
+    for (; tau + 4 <= n_fast; tau += 4) {
+        step(tau, I0{}, Fast{});
+        step(tau + 1, I1{}, Fast{});
+        step(tau + 2, I2{}, Fast{});
+        step(tau + 3, I3{}, Fast{});
+    }
+    for (; tau + 4 <= n_mid; tau += 4) {
+        step(tau, I0{}, Mid{});
+        step(tau + 1, I1{}, Mid{});
+        step(tau + 2, I2{}, Mid{});
+        step(tau + 3, I3{}, Mid{});
+    }
+    for (; tau < n_tiles; tau += 4) {
+        step(tau, I0{}, Slow{});
+        if (tau + 1 < n_tiles) step(tau + 1, I1{}, Slow{});
+        if (tau + 2 < n_tiles) step(tau + 2, I2{}, Slow{});
+        if (tau + 3 < n_tiles) step(tau + 3, I3{}, Slow{});
+    }
+    // operands requested for a step that does not exist are still in flight: let them land before the registers die
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+
+    l = half_swap_sum(l);
+    const int qi = q0 + ql;
+    if (qi < a.T) {
+        const float inv_l = l > 0.f ? 1.0f / l : 0.f;
+        uint16_t* op = (uint16_t*)a.out + (int64_t)b * a.so[0] + (int64_t)hq * a.so[1] + (int64_t)qi * a.so[2];
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int vq = 0; vq < 4; ++vq) {
+                const int d = 32 * db + 8 * vq + 4 * h;
+                uint2 w;
+                w.x = cvt_pk_bf16(acc[db][4 * vq] * inv_l, acc[db][4 * vq + 1] * inv_l);
+                w.y = cvt_pk_bf16(acc[db][4 * vq + 2] * inv_l, acc[db][4 * vq + 3] * inv_l);
+                *(uint2*)(op + d) = w;
+            }
+        if (a.lse && h == 0)
+            a.lse[(int64_t)b * a.sl[0] + (int64_t)hq * a.sl[1] + (int64_t)qi * a.sl[2]] = (m_ref + __builtin_amdgcn_logf(l)) * 0.6931471805599453f;
+    }
+#endif
+}
+
+// ---------------------------------------------------------------------------------------------
 // fp32 kernel (fp32 inputs, fp32 MFMA 32x32x2, fp32 softmax): the precision the reference computes
 // in.  One wavefront owns 32 queries, a workgroup 128; key tiles of 32 through LDS.
 // ---------------------------------------------------------------------------------------------
@@ -569,7 +955,10 @@ int launch_prefill(const PrefillArgs& a, int dtype, int64_t D, bool cache_planes
             if (D == 128) hipLaunchKernelGGL((prefill_bf16_kernel<128, true>), grid, block, 0, st, a);
             else hipLaunchKernelGGL((prefill_bf16_kernel<64, true>), grid, block, 0, st, a);
         } else {
-            if (D == 128) hipLaunchKernelGGL((prefill_bf16_kernel<128, false>), grid, block, 0, st, a);
+            // the software-pipelined kernel takes one context length for the batch; dense K/V with per-row lengths
+            // (a Q8_0 cache read out into the workspace) stay with the general kernel
+            if (D == 128 && !a.seq_lens && !a.chunk_lens) hipLaunchKernelGGL(prefill_bf16_pipe_kernel, grid, block, 0, st, a);
+            else if (D == 128) hipLaunchKernelGGL((prefill_bf16_kernel<128, false>), grid, block, 0, st, a);
             else hipLaunchKernelGGL((prefill_bf16_kernel<64, false>), grid, block, 0, st, a);
         }
     } else {
