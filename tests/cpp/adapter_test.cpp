@@ -307,6 +307,174 @@ static void test_sdpa_routing() {
     CHECK(ok);
 }
 
+static void test_backward_dispatch_seam() {
+    // flash_attention_backward_hip_dispatch with the reference's parameter list (include/vesper/ops/flash_attention.h:80-92):
+    // caller-allocated gradients, GQA operands (dk/dv summed over each group's query heads), dropout mask refused.
+    std::printf("test_backward_dispatch_seam\n");
+    const int64_t B = 1, Hq = 4, Hkv = 2, N = 40, D = 64, n = Hq / Hkv;
+    const float scale = 1.0f / std::sqrt((float)D);
+    auto q = randn(B * Hq * N * D, 41), k = randn(B * Hkv * N * D, 42), v = randn(B * Hkv * N * D, 43), dout = randn(B * Hq * N * D, 44);
+    // oracle on repeated K/V, then the group sums
+    std::vector<float> kr(q.size()), vr(q.size()), out(q.size()), lse(B * Hq * N), wq(q.size()), wkr(q.size()), wvr(q.size());
+    for (int64_t h = 0; h < Hq; ++h) {
+        std::memcpy(&kr[(size_t)(h * N * D)], &k[(size_t)((h / n) * N * D)], N * D * sizeof(float));
+        std::memcpy(&vr[(size_t)(h * N * D)], &v[(size_t)((h / n) * N * D)], N * D * sizeof(float));
+    }
+    orc_flash_attention_f32(q.data(), kr.data(), vr.data(), out.data(), lse.data(), B, Hq, N, D, scale, 1);
+    orc_flash_attention_backward_f32(dout.data(), q.data(), kr.data(), vr.data(), out.data(), lse.data(), wq.data(), wkr.data(), wvr.data(),
+                                     B, Hq, N, D, scale, 1);
+    std::vector<float> wk(k.size(), 0.f), wv(v.size(), 0.f);
+    for (int64_t h = 0; h < Hq; ++h)
+        for (int64_t i = 0; i < N * D; ++i) {
+            wk[(size_t)((h / n) * N * D + i)] += wkr[(size_t)(h * N * D + i)];
+            wv[(size_t)((h / n) * N * D + i)] += wvr[(size_t)(h * N * D + i)];
+        }
+    Tensor tq = to_dev(q, {B, Hq, N, D}, DType::Float32), tk = to_dev(k, {B, Hkv, N, D}, DType::Float32);
+    Tensor tv = to_dev(v, {B, Hkv, N, D}, DType::Float32), tdo = to_dev(dout, {B, Hq, N, D}, DType::Float32);
+    Tensor o = empty({B, Hq, N, D}, DType::Float32), l = empty({B, Hq, N}, DType::Float32);
+    ops::flash_attention_hip_dispatch(tq, ops::repeat_kv(tk, n), ops::repeat_kv(tv, n), o, l, scale, true, 0.0f, false, nullptr);
+    Tensor gq = empty({B, Hq, N, D}, DType::Float32), gk = empty({B, Hkv, N, D}, DType::Float32), gv = empty({B, Hkv, N, D}, DType::Float32);
+    ops::flash_attention_backward_hip_dispatch(tdo, tq, tk, tv, o, l, gq, gk, gv, scale, true, 0.0f, nullptr);
+    CHECK(max_abs_diff(to_host(gq), wq.data(), wq.size()) < 2e-4);
+    CHECK(max_abs_diff(to_host(gk), wk.data(), wk.size()) < 4e-4);
+    CHECK(max_abs_diff(to_host(gv), wv.data(), wv.size()) < 4e-4);
+    // a dropout mask (training with p > 0) is not implemented: refused, as the forward refuses to produce one
+    Tensor mask = empty({B, Hq, N, N}, DType::Float32);
+    CHECK(thrown<std::runtime_error>([&] { ops::flash_attention_backward_hip_dispatch(tdo, tq, tk, tv, o, l, gq, gk, gv, scale, true, 0.1f, &mask); }) !=
+          "<nothing thrown>");
+    // the front end with the reference's defaults (is_causal = true, dropout_p = 0, no mask)
+    auto g = ops::flash_attention_backward(tdo, tq, tk, tv, o, l, scale);
+    CHECK(max_abs_diff(to_host(std::get<0>(g)), wq.data(), wq.size()) < 2e-4);
+}
+
+static void test_multi_head_attention_core() {
+    // MultiHeadAttention's three forward overloads (src/nn/transformer.cpp:108-216) on the attention core
+    std::printf("test_multi_head_attention_core\n");
+    const int64_t B = 2, H = 4, T = 24, D = 64;
+    auto q = randn(B * H * T * D, 51, 0.5f), k = randn(B * H * T * D, 52, 0.5f), v = randn(B * H * T * D, 53, 0.5f);
+    std::vector<float> want(q.size());
+    Tensor tq = to_dev(q, {B, H, T, D}, DType::Float32), tk = to_dev(k, {B, H, T, D}, DType::Float32), tv = to_dev(v, {B, H, T, D}, DType::Float32);
+    {   // use_rope = false: forward(x) is NOT causal (:108-110); forward(x, true) is
+        nn::MultiHeadAttentionCore mha((int)(H * D), (int)H, 0.0f, false);
+        orc_sdpa_f32(q.data(), k.data(), v.data(), want.data(), B, H, T, T, D, 0);
+        CHECK(max_abs_diff(to_host(mha.forward(tq, tk, tv)), want.data(), want.size()) < 1e-4);
+        orc_sdpa_f32(q.data(), k.data(), v.data(), want.data(), B, H, T, T, D, 1);
+        CHECK(max_abs_diff(to_host(mha.forward(tq, tk, tv, true)), want.data(), want.size()) < 1e-4);
+        // the default really is the non-causal result: it differs from the causal one
+        CHECK(max_abs_diff(to_host(mha.forward(tq, tk, tv)), want.data(), want.size()) > 1e-3);
+    }
+    {   // use_rope = true (the constructor's default): q, k rotated at positions 0.. (:132-136), fp32 and bf16
+        nn::MultiHeadAttentionCore mha((int)(H * D), (int)H);
+        std::vector<float> ang((size_t)(T * D / 2)), qr(q.size()), kr(k.size());
+        orc_rope_angles((int)T, (int)D, 0, 10000.0f, ang.data());
+        orc_rope_apply_f32(q.data(), B, H, T, D, ang.data(), qr.data());
+        orc_rope_apply_f32(k.data(), B, H, T, D, ang.data(), kr.data());
+        for (int causal = 0; causal < 2; ++causal) {
+            orc_sdpa_f32(qr.data(), kr.data(), v.data(), want.data(), B, H, T, T, D, causal);
+            Tensor got = causal ? mha.forward(tq, tk, tv, true) : mha.forward(tq, tk, tv);
+            CHECK(max_abs_diff(to_host(got), want.data(), want.size()) < 1e-4);
+        }
+        auto qb = bf16_round(q), kb = bf16_round(k), vb = bf16_round(v);
+        orc_rope_apply_f32(qb.data(), B, H, T, D, ang.data(), qr.data());
+        orc_rope_apply_f32(kb.data(), B, H, T, D, ang.data(), kr.data());
+        auto qrb = bf16_round(qr), krb = bf16_round(kr);
+        orc_sdpa_f32(qrb.data(), krb.data(), vb.data(), want.data(), B, H, T, T, D, 0);
+        Tensor gb = mha.forward(to_dev(qb, {B, H, T, D}, DType::BFloat16), to_dev(kb, {B, H, T, D}, DType::BFloat16),
+                                to_dev(vb, {B, H, T, D}, DType::BFloat16));
+        CHECK(max_abs_diff(to_host(gb), want.data(), want.size()) < 2e-2);
+        // forward(x, cache, start_pos): prefill 16 tokens (causal because T > 1), then token by token (:166-216)
+        nn::KVCache cache((int)B, (int)H, 64, (int)D, Device::HIP);
+        orc_sdpa_f32(qr.data(), kr.data(), v.data(), want.data(), B, H, T, T, D, 1);  // overwritten below with fp32 rotation
+        orc_rope_apply_f32(q.data(), B, H, T, D, ang.data(), qr.data());
+        orc_rope_apply_f32(k.data(), B, H, T, D, ang.data(), kr.data());
+        orc_sdpa_f32(qr.data(), kr.data(), v.data(), want.data(), B, H, T, T, D, 1);
+        auto slice = [&](const std::vector<float>& x, int64_t t0, int64_t t1) {
+            std::vector<float> out((size_t)(B * H * (t1 - t0) * D));
+            for (int64_t bh = 0; bh < B * H; ++bh)
+                for (int64_t t = t0; t < t1; ++t)
+                    std::memcpy(&out[(size_t)((bh * (t1 - t0) + (t - t0)) * D)], &x[(size_t)((bh * T + t) * D)], D * sizeof(float));
+            return out;
+        };
+        auto step = [&](int64_t t0, int64_t t1) {
+            Tensor out = mha.forward(to_dev(slice(q, t0, t1), {B, H, t1 - t0, D}, DType::Float32),
+                                     to_dev(slice(k, t0, t1), {B, H, t1 - t0, D}, DType::Float32),
+                                     to_dev(slice(v, t0, t1), {B, H, t1 - t0, D}, DType::Float32), &cache, (int)t0);
+            auto w = slice(want, t0, t1);
+            CHECK(max_abs_diff(to_host(out), w.data(), w.size()) < 1e-4);
+            CHECK(cache.current_seq_len() == (int)t1);
+        };
+        step(0, 16);
+        for (int64_t t = 16; t < T; ++t) step(t, t + 1);
+        // training-mode attention dropout is not implemented on this path
+        nn::MultiHeadAttentionCore drop((int)(H * D), (int)H, 0.1f, false);
+        drop.train();
+        CHECK(thrown<std::runtime_error>([&] { drop.forward(tq, tk, tv); }) != "<nothing thrown>");
+        drop.eval();
+        orc_sdpa_f32(q.data(), k.data(), v.data(), want.data(), B, H, T, T, D, 0);
+        CHECK(max_abs_diff(to_host(drop.forward(tq, tk, tv)), want.data(), want.size()) < 1e-4);
+    }
+}
+
+static void test_token_loop_allocates_nothing_and_keeps_pace() {
+    // One decode step of the drop-in layer = forward_rope (RoPE + append, split-K decode + combine).  After warm-up the
+    // step must not reach the driver's allocator and must not wait for the stream; its time per token is compared with
+    // the same three launches issued straight through the C ABI on preallocated buffers.
+    std::printf("test_token_loop_allocates_nothing_and_keeps_pace\n");
+    const int64_t B = 32, Hq = 32, Hkv = 8, D = 128, S_max = 4096, L0 = 2048, tokens = 64;
+    nn::GroupedQueryAttentionCore attn(Hq * D, Hq, Hkv);
+    nn::RopeTable rope(S_max, D);
+    nn::GQAKVCache cache(B, Hkv, S_max, D, Device::HIP, KVFormat::BFloat16);
+    {   // a context of L0 tokens
+        Tensor k0 = to_dev(randn(B * Hkv * L0 * D, 61, 0.5f), {B, Hkv, L0, D}, DType::BFloat16);
+        cache.update(k0, k0, 0);
+    }
+    Tensor tq = to_dev(randn(B * Hq * D, 62, 0.5f), {B, Hq, 1, D}, DType::BFloat16);
+    Tensor tk = to_dev(randn(B * Hkv * D, 63, 0.5f), {B, Hkv, 1, D}, DType::BFloat16);
+    hipEvent_t e0, e1;
+    hip_check(hipEventCreate(&e0), "event");
+    hip_check(hipEventCreate(&e1), "event");
+    auto adapter_loop = [&](int64_t pos0) {
+        for (int64_t t = 0; t < tokens; ++t) (void)attn.forward_rope(tq, tk, tk, &cache, pos0 + t, rope, DType::BFloat16);
+    };
+    adapter_loop(L0);  // warm-up: fills the block cache
+    hip_check(hipStreamSynchronize(current_stream()), "sync");
+    const size_t blocks_before = BlockCache::instance().driver_allocations();
+    hip_check(hipEventRecord(e0, current_stream()), "record");
+    adapter_loop(L0 + tokens);
+    hip_check(hipEventRecord(e1, current_stream()), "record");
+    hip_check(hipEventSynchronize(e1), "sync");
+    float ms_adapter = 0.f;
+    hip_check(hipEventElapsedTime(&ms_adapter, e0, e1), "elapsed");
+    CHECK(BlockCache::instance().driver_allocations() == blocks_before);  // no hipMalloc inside the timed loop
+    // the same launches through the C ABI
+    vsp_kv_cache c = cache.raw();
+    Tensor q_rot = empty({B, Hq, 1, D}, DType::BFloat16), out = empty({B, Hq, 1, D}, DType::BFloat16);
+    const size_t ws_bytes = vsp_attn_decode_workspace_bytes((int32_t)B, (int32_t)Hq, (int32_t)D, (int32_t)S_max);
+    Storage ws(ws_bytes);
+    vsp_tensor dq = tq.desc(), dk = tk.desc(), dqo = q_rot.desc(), dout = out.desc();
+    const float scale = 1.0f / std::sqrt((float)D);
+    auto abi_loop = [&](int64_t pos0) {
+        for (int64_t t = 0; t < tokens; ++t) {
+            c.len = (int32_t)(pos0 + t);
+            throw_status(vsp_rope_kv_append(&c, &dq, &dk, &dk, &dqo, rope.data(), rope.length(), pos0 + t, nullptr, current_stream()));
+            throw_status(vsp_attn_decode(&dqo, &c, nullptr, 0, &dout, scale, ws.data(), ws_bytes, current_stream()));
+        }
+    };
+    abi_loop(L0 + 2 * tokens);
+    hip_check(hipStreamSynchronize(current_stream()), "sync");
+    hip_check(hipEventRecord(e0, current_stream()), "record");
+    abi_loop(L0 + 3 * tokens);
+    hip_check(hipEventRecord(e1, current_stream()), "record");
+    hip_check(hipEventSynchronize(e1), "sync");
+    float ms_abi = 0.f;
+    hip_check(hipEventElapsedTime(&ms_abi, e0, e1), "elapsed");
+    std::printf("  %lld tokens, B %lld, context %lld..: adapter %.1f us/token, C ABI %.1f us/token (ratio %.3f)\n", (long long)tokens,
+                (long long)B, (long long)(L0 + tokens), 1e3 * ms_adapter / tokens, 1e3 * ms_abi / tokens, ms_adapter / ms_abi);
+    CHECK(ms_adapter < 1.25f * ms_abi);  // a loose bound for a shared test machine; the measured ratio is printed above
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+}
+
 int main(int argc, char** argv) {
     const bool cpu_only = argc > 1 && std::string(argv[1]) == "--cpu-only";
     test_gqa_constructor_validation();
@@ -319,6 +487,9 @@ int main(int argc, char** argv) {
         run_rope_generation<nn::KVCache>(KVFormat::Float32, DType::Float32, 1e-4, "KVCache fp32");
         run_rope_generation<nn::GQAKVCache>(KVFormat::BFloat16, DType::BFloat16, 2e-2, "GQAKVCache bf16");
         test_sdpa_routing();
+        test_backward_dispatch_seam();
+        test_multi_head_attention_core();
+        test_token_loop_allocates_nothing_and_keeps_pace();
     }
     std::printf(g_fail ? "FAILED: %d check(s)\n" : "all adapter tests passed\n", g_fail);
     return g_fail ? 1 : 0;

@@ -18,10 +18,13 @@
 
 #include <cmath>
 #include <cstdint>
+#include <map>
 #include <memory>
+#include <mutex>
 #include <stdexcept>
 #include <string>
 #include <tuple>
+#include <unordered_map>
 #include <utility>
 #include <vector>
 
@@ -55,14 +58,71 @@ inline hipStream_t& current_stream() {
     return s;
 }
 
+// Device blocks are recycled instead of returned to the driver, like the reference's CachingAllocator
+// (include/vesper/core/allocator.h:28-68: "keep a pool of free blocks sorted by size; when freeing, return to pool"):
+// after warm-up no call on this path reaches hipMalloc / hipFree (hipFree waits for the device).  A block is handed out
+// again only to the stream it was released on, so reuse is ordered behind the work that last touched it and nobody
+// has to synchronise before letting a scratch buffer go.
+class BlockCache {
+public:
+    static BlockCache& instance() {
+        static BlockCache c;
+        return c;
+    }
+    void* take(size_t bytes, hipStream_t stream) {
+        if (bytes == 0) return nullptr;
+        const size_t want = round_size(bytes);
+        {
+            std::lock_guard<std::mutex> lock(mu_);
+            auto range = free_.equal_range(Key{stream, want});
+            if (range.first != range.second) {
+                void* p = range.first->second;
+                free_.erase(range.first);
+                return p;
+            }
+        }
+        void* p = nullptr;
+        hip_check(hipMalloc(&p, want), "hipMalloc");
+        std::lock_guard<std::mutex> lock(mu_);
+        size_[p] = want;
+        return p;
+    }
+    void give(void* p, hipStream_t stream) {
+        if (!p) return;
+        std::lock_guard<std::mutex> lock(mu_);
+        free_.emplace(Key{stream, size_.at(p)}, p);
+    }
+    // CachingAllocator::empty_cache(): release every free block to the driver (blocks in use stay)
+    void empty_cache() {
+        std::lock_guard<std::mutex> lock(mu_);
+        for (auto& kv : free_) {
+            size_.erase(kv.second);
+            (void)hipFree(kv.second);
+        }
+        free_.clear();
+    }
+    size_t driver_allocations() const {
+        std::lock_guard<std::mutex> lock(mu_);
+        return size_.size();
+    }
+
+private:
+    using Key = std::pair<hipStream_t, size_t>;
+    // sizes are rounded to 512-byte multiples up to 1 MiB and to 2 MiB multiples above, so that buffers whose size
+    // drifts slowly (a workspace that follows the context length) keep hitting the same bin
+    static size_t round_size(size_t b) {
+        const size_t q = b <= (1u << 20) ? 512 : (2u << 20);
+        return (b + q - 1) / q * q;
+    }
+    mutable std::mutex mu_;
+    std::multimap<Key, void*> free_;
+    std::unordered_map<void*, size_t> size_;
+};
+
 class Storage {
 public:
-    explicit Storage(size_t bytes) : bytes_(bytes) {
-        if (bytes) hip_check(hipMalloc(&ptr_, bytes), "hipMalloc");
-    }
-    ~Storage() {
-        if (ptr_) (void)hipFree(ptr_);
-    }
+    explicit Storage(size_t bytes) : bytes_(bytes), stream_(current_stream()) { ptr_ = BlockCache::instance().take(bytes, stream_); }
+    ~Storage() { BlockCache::instance().give(ptr_, stream_); }
     Storage(const Storage&) = delete;
     Storage& operator=(const Storage&) = delete;
     void* data() const { return ptr_; }
@@ -71,6 +131,7 @@ public:
 private:
     void* ptr_ = nullptr;
     size_t bytes_ = 0;
+    hipStream_t stream_ = nullptr;
 };
 
 // What a Tensor returned by KVCache::update refers to.
@@ -277,8 +338,7 @@ public:
         const float scale = 1.0f / std::sqrt(static_cast<float>(q.shape()[3]));
         throw_status(vsp_attn_prefill_cached(&dq, &st_->c, nullptr, nullptr, &dout, nullptr, scale, is_causal ? 1 : 0,
                                              ws ? ws->data() : nullptr, ws_bytes, current_stream()));
-        hip_check(hipStreamSynchronize(current_stream()), "attend");  // the scratch buffer dies with this scope
-        return out;
+        return out;  // the scratch block goes back to the cache; its next user is ordered behind this call on the stream
     }
     void reset() { throw_status(vsp_kv_cache_reset(&st_->c, current_stream())); }
     LenT current_seq_len() const { return (LenT)st_->c.len; }
@@ -361,22 +421,34 @@ inline Tensor flash_attention(const Tensor& q, const Tensor& k, const Tensor& v,
     return output;
 }
 
-// include/vesper/ops/flash_attention.h:61-66, src/ops/flash_attention.cpp:165-216: (grad_q, grad_k, grad_v).
+// include/vesper/ops/flash_attention.h:80-92 (defined src/ops/hip/flash_attention.hip:183-299): the gradients are
+// caller-allocated.  A dropout mask can only come from a training forward with dropout_p > 0, which this path
+// rejects, so a non-null mask with dropout_p > 0 is VSP_ERR_UNSUPPORTED here too.
+inline void flash_attention_backward_hip_dispatch(const Tensor& grad_output, const Tensor& q, const Tensor& k, const Tensor& v,
+                                                  const Tensor& output, const Tensor& lse, Tensor& grad_q, Tensor& grad_k,
+                                                  Tensor& grad_v, float scale, bool is_causal, float dropout_p,
+                                                  const Tensor* dropout_mask) {
+    if (dropout_p > 0.0f && dropout_mask && dropout_mask->defined()) throw_status(VSP_ERR_UNSUPPORTED);
+    if (dropout_p > 0.0f) throw_status(VSP_ERR_UNSUPPORTED);
+    vsp_tensor d0 = grad_output.desc(), d1 = q.desc(), d2 = k.desc(), d3 = v.desc(), d4 = output.desc(), d5 = lse.desc();
+    vsp_tensor o0 = grad_q.desc(), o1 = grad_k.desc(), o2 = grad_v.desc();
+    const size_t ws_bytes = q.ndim() == 4 ? vsp_attn_backward_workspace_bytes((int32_t)q.shape()[0], (int32_t)q.shape()[1], (int32_t)q.shape()[2]) : 0;
+    Storage ws(ws_bytes ? ws_bytes : 4);
+    throw_status(vsp_attn_prefill_backward(&d0, &d1, &d2, &d3, &d4, &d5, &o0, &o1, &o2, scale, is_causal ? 1 : 0, ws.data(), ws_bytes,
+                                           current_stream()));
+}
+
+// include/vesper/ops/flash_attention.h:61-71, src/ops/flash_attention.cpp:165-216: (grad_q, grad_k, grad_v).
 // `output` and `lse` are the forward's results (flash_attention_hip_dispatch writes both).  k and v may carry
 // fewer heads than q: their gradients are then already summed over each group's query heads.
 inline std::tuple<Tensor, Tensor, Tensor> flash_attention_backward(const Tensor& grad_output, const Tensor& q, const Tensor& k,
                                                                    const Tensor& v, const Tensor& output, const Tensor& lse, float scale,
-                                                                   bool is_causal, float dropout_p = 0.0f) {
-    if (dropout_p > 0.0f) throw_status(VSP_ERR_UNSUPPORTED);
+                                                                   bool is_causal = true, float dropout_p = 0.0f,
+                                                                   const Tensor& dropout_mask = Tensor()) {
     if (q.ndim() != 4 || k.ndim() != 4 || v.ndim() != 4) throw_status(VSP_ERR_NDIM);
     Tensor gq = empty(q.shape(), q.dtype()), gk = empty(k.shape(), k.dtype()), gv = empty(v.shape(), v.dtype());
-    vsp_tensor d0 = grad_output.desc(), d1 = q.desc(), d2 = k.desc(), d3 = v.desc(), d4 = output.desc(), d5 = lse.desc();
-    vsp_tensor o0 = gq.desc(), o1 = gk.desc(), o2 = gv.desc();
-    const size_t ws_bytes = vsp_attn_backward_workspace_bytes((int32_t)q.shape()[0], (int32_t)q.shape()[1], (int32_t)q.shape()[2]);
-    Storage ws(ws_bytes ? ws_bytes : 4);
-    throw_status(vsp_attn_prefill_backward(&d0, &d1, &d2, &d3, &d4, &d5, &o0, &o1, &o2, scale, is_causal ? 1 : 0, ws.data(), ws_bytes,
-                                           current_stream()));
-    hip_check(hipStreamSynchronize(current_stream()), "flash_attention_backward");  // the scratch buffer dies with this scope
+    flash_attention_backward_hip_dispatch(grad_output, q, k, v, output, lse, gq, gk, gv, scale, is_causal, dropout_p,
+                                          dropout_mask.defined() ? &dropout_mask : nullptr);
     return {gq, gk, gv};
 }
 
@@ -400,10 +472,9 @@ inline Tensor scaled_dot_product_attention(const Tensor& query, const Tensor& ke
         const vsp_kv_cache& c = key.cache->c;
         const size_t ws_bytes = vsp_attn_decode_workspace_bytes((int32_t)query.shape()[0], (int32_t)query.shape()[1], (int32_t)D,
                                                                c.len > 0 ? c.len : 1);
-        Storage ws(ws_bytes);
+        Storage ws(ws_bytes);  // a recycled block after the first call; released without waiting (see BlockCache)
         vsp_tensor dq = query.desc(), dout = out.desc();
         throw_status(vsp_attn_decode(&dq, &c, nullptr, 0, &dout, scale, ws.data(), ws_bytes, current_stream()));
-        hip_check(hipStreamSynchronize(current_stream()), "hipStreamSynchronize");  // ws is freed on return
         return out;
     }
     return ops::flash_attention(query, key, value, scale, is_causal && T > 1);
@@ -476,6 +547,84 @@ public:
 
 private:
     int64_t embed_dim_, num_heads_, num_kv_heads_, head_dim_ = 0, num_rep_ = 0;
+};
+
+// The attention core of MultiHeadAttention (include/vesper/nn/transformer.h:41-56, src/nn/transformer.cpp:96-216):
+// q, k, v [B,n_head,T,head_dim] are the three slices of c_attn's output viewed per head (:127-129, :182-184; any
+// strides, so the .contiguous() transposes can go).  The three overloads keep the reference's semantics:
+//   forward(q,k,v)                    = forward(q,k,v,false): NOT causal (:108-110)
+//   forward(q,k,v,causal)             RoPE at positions 0.. when use_rope (:132-136), then SDPA (:141)
+//   forward(q,k,v,cache,start_pos)    RoPE at start_pos.. (:187-191), cache->update (:193-197), SDPA with
+//                                     use_causal_mask = (T > 1) (:202-206)
+// dropout > 0 only matters in training mode, which this path does not implement (VSP_ERR_UNSUPPORTED if asked for).
+class MultiHeadAttentionCore {
+public:
+    MultiHeadAttentionCore(int embed_dim, int num_heads, float dropout = 0.0f, bool use_rope = true)
+        : n_head(num_heads), n_embd(embed_dim), dropout_(dropout), use_rope_(use_rope) {}
+
+    Tensor forward(const Tensor& q, const Tensor& k, const Tensor& v) { return forward(q, k, v, false); }
+
+    Tensor forward(const Tensor& q, const Tensor& k, const Tensor& v, bool causal) {
+        if (training_ && dropout_ > 0.0f) throw_status(VSP_ERR_UNSUPPORTED);
+        if (!use_rope_) return functional::scaled_dot_product_attention(q, k, v, causal, 0.0);
+        // RoPE without a cache of the caller's: a cache of exactly T tokens holds the rotated K and V for this call
+        // (one launch rotates q and k and writes it), then the attention reads it like any other cache
+        if (q.ndim() != 4) throw_status(VSP_ERR_NDIM);
+        const int64_t B = q.shape()[0], H = k.shape()[1], T = q.shape()[2], D = q.shape()[3];
+        const RopeTable& rope = rope_for(T, D);
+        KVCache scratch((int)B, (int)H, (int)T, (int)D, Device::HIP, q.dtype() == DType::Float32 ? KVFormat::Float32 : KVFormat::BFloat16);
+        Tensor qr = q;
+        auto kv = scratch.rope_update(qr, k, v, 0, rope, q.dtype());
+        if (q.dtype() == DType::Float32) return functional::scaled_dot_product_attention(qr, kv.first, kv.second, causal, 0.0);
+        return scratch.attend(qr, causal);
+    }
+
+    Tensor forward(const Tensor& q, Tensor k, Tensor v, KVCache* cache, int start_pos = 0) {
+        if (training_ && dropout_ > 0.0f) throw_status(VSP_ERR_UNSUPPORTED);
+        if (q.ndim() != 4) throw_status(VSP_ERR_NDIM);
+        const int64_t T = q.shape()[2], D = q.shape()[3];
+        Tensor qq = q;
+        if (cache) {
+            std::pair<Tensor, Tensor> kv = use_rope_ ? cache->rope_update(qq, k, v, start_pos, rope_for(start_pos + T, D), q.dtype())
+                                                     : cache->update(k, v, start_pos);
+            k = kv.first;
+            v = kv.second;
+        } else if (use_rope_) {
+            // no cache: rotate at start_pos.. through a cache of this call's own, as above
+            const int64_t B = q.shape()[0], H = k.shape()[1];
+            KVCache scratch((int)B, (int)H, (int)(start_pos + T), (int)D, Device::HIP,
+                            q.dtype() == DType::Float32 ? KVFormat::Float32 : KVFormat::BFloat16);
+            // only rows [start_pos, start_pos + T) are written and read back: SDPA over exactly these T keys
+            scratch.rope_update(qq, k, v, start_pos, rope_for(start_pos + T, D), q.dtype());
+            Tensor kr = empty(k.shape(), q.dtype()), vr = empty(v.shape(), q.dtype());
+            vsp_tensor dk = kr.desc(), dv = vr.desc();
+            throw_status(vsp_kv_read(&scratch.raw(), start_pos, T, &dk, &dv, current_stream()));
+            k = kr;
+            v = vr;
+        }
+        const bool use_causal_mask = (T > 1);
+        return functional::scaled_dot_product_attention(qq, k, v, use_causal_mask, 0.0);
+    }
+
+    void train(bool on = true) { training_ = on; }
+    void eval() { training_ = false; }
+
+    int n_head;
+    int n_embd;
+    float dropout_;
+    bool use_rope_;
+
+private:
+    const RopeTable& rope_for(int64_t positions, int64_t head_dim) {
+        if (!rope_ || rope_->length() < positions || rope_->head_dim() != head_dim) {
+            int64_t len = 256;
+            while (len < positions) len *= 2;
+            rope_ = std::make_unique<RopeTable>(len, head_dim, 10000.0f);  // theta of :133, :188
+        }
+        return *rope_;
+    }
+    bool training_ = false;
+    std::unique_ptr<RopeTable> rope_;
 };
 
 }  // namespace nn
