@@ -189,7 +189,8 @@ int vsp_kv_view_f32(const vsp_kv_cache* cache, vsp_tensor* k_view, vsp_tensor* v
  * (include/vesper/ops/attention_ops.h:35) folded in: q [B,Hq,T,D]; k, v [B,Hkv,L,D] with
  * Hq % Hkv == 0, query head h reading kv head h / (Hq/Hkv) (src/ops/attention_ops.cpp:47).
  * out [B,Hq,T,D] same dtype as q; lse [B,Hq,T] fp32 or NULL (= m + log l, src/ops/flash_attention.cpp:359).
- * dtype bf16 (MFMA, fp32 accumulation) or fp32.  D in {64,128}.  q/k/v/out may be strided
+ * dtype bf16 (MFMA, fp32 accumulation) or fp32.  D in {64,128}; fp32 also takes D = 32 (the shapes of the
+ * reference's own tests, tests/test_flash_attention.cpp:110-179).  q/k/v/out may be strided
  * (stride[3]==1, rows 16-byte aligned), e.g. VSP_KV_F32 cache views.
  * is_causal: key j visible to query t iff j <= t + (L - T): the reference's mask when T == L
  * (src/ops/flash_attention.cpp:293-296), and its natural extension to a chunk appended at the end
@@ -206,7 +207,7 @@ int vsp_attn_prefill(const vsp_tensor* q, const vsp_tensor* k, const vsp_tensor*
  * its query heads, the gradient of ops::repeat_kv), lse [B,Hq,N] fp32 as written by vsp_attn_prefill; fp32 or bf16
  * (one dtype).  fp32: fp32 matrix-core arithmetic, any strides with stride[3]==1.  bf16: bf16 matrix cores with fp32
  * accumulation, P and dS rounded to bf16 between the products, gradients rounded to nearest even; base pointers and
- * strides multiples of 16 bytes (VSP_ERR_ALIGN), stride[2] >= D (VSP_ERR_STRIDE).  D in {64,128}.  dq/dk/dv are
+ * strides multiples of 16 bytes (VSP_ERR_ALIGN), stride[2] >= D (VSP_ERR_STRIDE).  D in {64,128}, fp32 also 32.  dq/dk/dv are
  * overwritten.  No atomics: results are bitwise reproducible (the reference's
  * HIP kernel accumulates dQ with atomicAdd).  workspace: vsp_attn_backward_workspace_bytes(B, Hq, N) bytes. */
 size_t vsp_attn_backward_workspace_bytes(int32_t B, int32_t Hq, int32_t N);

@@ -33,7 +33,7 @@ def _forward_then_backward(va, q, k, v, dout, scale, causal, bf16=False):
 
 def test_fixture_written_from_the_reference(va):
     z = np.load(os.path.join(GOLD, "flash_backward.npz"), allow_pickle=False)
-    for tag in ("r70", "nc33", "d128"):   # t16 has D = 32, which the kernels do not implement
+    for tag in ("r70", "nc33", "d128", "t16"):   # t16: the reference's own {1,1,8,32} shape
         B, H, N, D, causal, seed = [int(x) for x in z[tag + "_meta"]]
         q, k, v = I.qkv(seed, B, H, H, N, N, D)
         dout = I.normal(seed + 5, (B, H, N, D))
@@ -182,8 +182,11 @@ def test_argument_errors(va):
     q = torch.zeros(1, 4, 8, 64, device=d)
     k = torch.zeros(1, 2, 8, 64, device=d)
     lse = torch.zeros(1, 4, 8, device=d)
-    with pytest.raises(va.VspError):   # head dim 32 is not implemented
-        z = torch.zeros(1, 2, 8, 32, device=d)
+    with pytest.raises(va.VspError):   # head dim 32 exists in fp32 only; head dim 48 not at all
+        z = torch.zeros(1, 2, 8, 32, device=d, dtype=torch.bfloat16)
+        va.flash_attention_backward(z, z, z, z, z, torch.zeros(1, 2, 8, device=d), 0.1)
+    with pytest.raises(va.VspError):
+        z = torch.zeros(1, 2, 8, 48, device=d)
         va.flash_attention_backward(z, z, z, z, z, torch.zeros(1, 2, 8, device=d), 0.1)
     with pytest.raises(va.VspError):   # 3 query heads over 2 kv heads
         q3 = torch.zeros(1, 3, 8, 64, device=d)

@@ -734,9 +734,12 @@ int launch_backward(const BwdArgs& a, int64_t D, hipStream_t st) {
     if (D == 128) {
         hipLaunchKernelGGL((bwd_dq_kernel<128, T>), gq, dim3(256), 0, st, a);
         hipLaunchKernelGGL((bwd_dkdv_kernel<128, T>), gk, dim3(256), 0, st, a);
-    } else {
+    } else if (D == 64) {
         hipLaunchKernelGGL((bwd_dq_kernel<64, T>), gq, dim3(256), 0, st, a);
         hipLaunchKernelGGL((bwd_dkdv_kernel<64, T>), gk, dim3(256), 0, st, a);
+    } else {
+        hipLaunchKernelGGL((bwd_dq_kernel<32, T>), gq, dim3(256), 0, st, a);
+        hipLaunchKernelGGL((bwd_dkdv_kernel<32, T>), gk, dim3(256), 0, st, a);
     }
     return check_launch();
 }
@@ -772,7 +775,7 @@ extern "C" int vsp_attn_prefill_backward(const vsp_tensor* dout, const vsp_tenso
     if (lse->dtype != VSP_F32) return VSP_ERR_DTYPE;
     if (B * Hq * N * D == 0) return VSP_OK;
     if (!lse->data) return VSP_ERR_NULL;
-    if (D != 64 && D != 128) return VSP_ERR_UNSUPPORTED;
+    if (D != 64 && D != 128 && !(D == 32 && dt == VSP_F32)) return VSP_ERR_UNSUPPORTED;  // fp32 also takes head_dim 32
     if (!(fabsf(scale) < INFINITY)) return VSP_ERR_ARG;
     if (N > INT32_MAX / 2) return VSP_ERR_ARG;
     if (!workspace || workspace_bytes < vsp_attn_backward_workspace_bytes((int32_t)B, (int32_t)Hq, (int32_t)N)) return VSP_ERR_WORKSPACE;

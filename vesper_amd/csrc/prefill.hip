@@ -872,10 +872,17 @@ __global__ void __launch_bounds__(256) prefill_f32_kernel(PrefillArgs a) {
 
     for (int kt = 0; kt < n_tiles; ++kt) {
         __syncthreads();
-        for (int id = tid; id < BN * D; id += 256) {
-            const int row = id / D, col = id % D, key = kt * BN + row;
-            sK[row * PITCH + col] = key < L ? Kp[(int64_t)key * a.sk[2] + col] : 0.f;
-            sV[row * PITCH + col] = key < L ? Vp[(int64_t)key * a.sv[2] + col] : 0.f;
+        for (int id = tid; id < BN * (D / 4); id += 256) {  // 16-byte loads (rows are 16-byte aligned), padded LDS rows
+            const int row = id / (D / 4), col = 4 * (id % (D / 4)), key = kt * BN + row;
+            float4 kk = {0.f, 0.f, 0.f, 0.f}, vv = kk;
+            if (key < L) {
+                kk = *(const float4*)(Kp + (int64_t)key * a.sk[2] + col);
+                vv = *(const float4*)(Vp + (int64_t)key * a.sv[2] + col);
+            }
+            float* dk = sK + row * PITCH + col;
+            float* dv = sV + row * PITCH + col;
+            dk[0] = kk.x, dk[1] = kk.y, dk[2] = kk.z, dk[3] = kk.w;
+            dv[0] = vv.x, dv[1] = vv.y, dv[2] = vv.z, dv[3] = vv.w;
         }
         __syncthreads();
         const int k0 = kt * BN;
@@ -963,7 +970,8 @@ int launch_prefill(const PrefillArgs& a, int dtype, int64_t D, bool cache_planes
         }
     } else {
         if (D == 128) hipLaunchKernelGGL(prefill_f32_kernel<128>, grid, block, 0, st, a);
-        else hipLaunchKernelGGL(prefill_f32_kernel<64>, grid, block, 0, st, a);
+        else if (D == 64) hipLaunchKernelGGL(prefill_f32_kernel<64>, grid, block, 0, st, a);
+        else hipLaunchKernelGGL(prefill_f32_kernel<32>, grid, block, 0, st, a);
     }
     return check_launch();
 }
@@ -1007,7 +1015,7 @@ extern "C" int vsp_attn_prefill_cached(const vsp_tensor* q, const vsp_kv_cache* 
         if (lse->dtype != VSP_F32) return VSP_ERR_DTYPE;
     }
     if (B * Hq * T * D == 0) return VSP_OK;
-    if (D != 64 && D != 128) return VSP_ERR_UNSUPPORTED;
+    if (D != 64 && D != 128 && !(D == 32 && q->dtype == VSP_F32)) return VSP_ERR_UNSUPPORTED;  // fp32 also takes head_dim 32
     if (!(fabsf(scale) > 0.0f) || !(fabsf(scale) < INFINITY)) return VSP_ERR_ARG;
     const int esz = q->dtype == VSP_F32 ? 4 : 2;
     if ((rc = check_tensor4(q, esz)) != VSP_OK || (rc = check_tensor4(out, esz)) != VSP_OK) return rc;
@@ -1101,7 +1109,7 @@ extern "C" int vsp_attn_prefill(const vsp_tensor* q, const vsp_tensor* k, const 
         if (lse->dtype != VSP_F32) return VSP_ERR_DTYPE;
     }
     if (B * Hq * T * D == 0) return VSP_OK;
-    if (D != 64 && D != 128) return VSP_ERR_UNSUPPORTED;
+    if (D != 64 && D != 128 && !(D == 32 && q->dtype == VSP_F32)) return VSP_ERR_UNSUPPORTED;  // fp32 also takes head_dim 32
     if (L == 0) return VSP_ERR_SHAPE;  // softmax over an empty context is undefined
     if (!(fabsf(scale) > 0.0f) || !(fabsf(scale) < INFINITY)) return VSP_ERR_ARG;
     const int esz = q->dtype == VSP_F32 ? 4 : 2;
