@@ -85,7 +85,7 @@ class Runner:
             self.scale = 1.0 / math.sqrt(D)
             self.work = prefill_flops(w)
             self.unit, self.peak, self.bound = "TFLOP/s", MFMA_BF16_PEAK_TFLOPS, "mfma"
-            self.kernel = "prefill_bf16_kernel<128, false>"
+            self.kernel = "prefill_bf16_pipe_kernel"
         elif w["kind"] == "prefill_cached":
             B, Hq, Hkv, D, N = w["B"], w["Hq"], w["Hkv"], w["D"], w["N"]
             mk = lambda h: (torch.randn(B, h, N, D, device=dev, generator=g) * 0.5).to(torch.bfloat16)
@@ -204,22 +204,25 @@ def condition(torch, fn, seconds=CONDITION_SECONDS):
 
 def time_steps(torch, fn, steps, warmup, conditioning=True):
     """clock conditioning and `warmup` steps untimed, then exactly `steps` steps: wall clock bracketed by
-    synchronize, and device time from events recorded on the launch stream around the same region."""
+    synchronize, and device time from events recorded on the launch stream around the same region.  An event after
+    every step gives the per-step durations (median and minimum) without touching the timed region's length."""
     if conditioning:
         condition(torch, fn)
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
     t0 = time.perf_counter()
-    e0.record()
-    for _ in range(steps):
+    ev[0].record()
+    for i in range(steps):
         fn()
-    e1.record()
+        ev[i + 1].record()
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / steps
-    dev = e0.elapsed_time(e1) * 1e-3 / steps
-    return wall, dev
+    dev = ev[0].elapsed_time(ev[steps]) * 1e-3 / steps
+    per_step = sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(steps))
+    stats = {"median_ms": round(per_step[len(per_step) // 2], 5), "min_ms": round(per_step[0], 5)}
+    return wall, dev, stats
 
 
 def cpu_baseline(key):
@@ -272,16 +275,49 @@ def cpu_baseline(key):
                 seconds=dt * reps)
 
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs of this
-# script (summaries under profiles/). The raw counters are scaled by what they read for a 1 GiB read + 1 GiB write
-# elementwise kernel launched by --copy-calibration: FETCH_SIZE x 2.0 = KiB, WRITE_SIZE x 1.0 = KiB. Counters
-# cannot be collected inside a timed run, so these are constants of the workload shapes, not live values.
-MEASURED_TRAFFIC = {
-    "c2": {"fetch_bytes": 64616 * 2 * 1024, "write_bytes": 65730 * 1024, "algorithmic_bytes": 96 * 2**20 + 65 * 2**20},
-    "c3": {"fetch_bytes": 66900 * 2 * 1024, "write_bytes": 65554 * 1024, "algorithmic_bytes": 96 * 2**20 + 65 * 2**20},
-    "c4": {"fetch_bytes": 1280065 * 2 * 1024, "write_bytes": 10880 * 1024, "algorithmic_bytes": 2614935552},
-    "c5": {"fetch_bytes": 1115375 * 2 * 1024, "write_bytes": 4352 * 1024, "algorithmic_bytes": 2282225664},
+# HBM bytes per launch of the dominant kernel come from the rocprofv3 summaries committed under profiles/ (FETCH_SIZE and
+# WRITE_SIZE runs of this script, see the command lines at the top of each file).  The raw counters are scaled by what
+# they read for a 1 GiB read + 1 GiB write elementwise kernel launched by --copy-calibration in the same run.  Counters
+# cannot be collected inside a timed run, so these are properties of the workload shapes, not live values.
+PROFILE_OF = {
+    "c2": ("prefill_bf16_config2.txt", "prefill_bf16", 96 * 2**20 + 65 * 2**20),
+    "c3": ("prefill_bf16_config3.txt", "prefill_bf16", 96 * 2**20 + 65 * 2**20),
+    "c4": ("decode_bf16_config4.txt", "decode_bf16_kernel", 2614935552),
+    "c5": ("decode_q8_0_config5.txt", "decode_q8_kernel", 2282225664),
 }
+CALIBRATION_KERNEL, CALIBRATION_KIB = "CUDAFunctorOnSelf_add<int>", 1048576.0
+
+
+def traffic_from_profile(key):
+    """{"fetch_bytes", "write_bytes", "algorithmic_bytes", "source"} parsed from profiles/<file>, or None."""
+    if key not in PROFILE_OF:
+        return None
+    fname, kernel, algorithmic = PROFILE_OF[key]
+    path = os.path.join(ROOT, "profiles", fname)
+    if not os.path.exists(path):
+        return None
+    out, section = {}, None
+    raw = {"FETCH_SIZE": {}, "WRITE_SIZE": {}}
+    for line in open(path):
+        if line.startswith("## "):
+            section = "FETCH_SIZE" if "FETCH_SIZE" in line else ("WRITE_SIZE" if "WRITE_SIZE" in line else None)
+            continue
+        if section and section in line:
+            left, right = line.rsplit(section, 1)
+            cols = right.split()
+            if len(cols) >= 2:
+                name = "calibration" if CALIBRATION_KERNEL in left else ("kernel" if kernel in left else None)
+                if name and name not in raw[section]:
+                    raw[section][name] = float(cols[1])  # columns after the counter name: n, avg, min, max
+    try:
+        for section, field in (("FETCH_SIZE", "fetch_bytes"), ("WRITE_SIZE", "write_bytes")):
+            scale = CALIBRATION_KIB / raw[section]["calibration"]
+            out[field] = int(raw[section]["kernel"] * scale * 1024)
+    except KeyError:
+        return None
+    out["algorithmic_bytes"] = algorithmic
+    out["source"] = "profiles/" + fname
+    return out
 
 
 def main():
@@ -317,7 +353,7 @@ def main():
         del src, dst
 
     primary = Runner(args.workload, torch, va)
-    wall, dev = time_steps(torch, primary.step, args.steps, args.warmup, not args.no_conditioning)
+    wall, dev, stats = time_steps(torch, primary.step, args.steps, args.warmup, not args.no_conditioning)
     value = primary.rate(wall)
     achieved = primary.rate(dev)
     result = {
@@ -328,6 +364,8 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(wall * 1e3, 5),
+        "median_ms": stats["median_ms"],
+        "min_ms": stats["min_ms"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -338,9 +376,11 @@ def main():
                    "work_unit": "FLOP" if primary.bound == "mfma" else "bytes"},
         "roofline": {"bound": primary.bound, "achieved": round(achieved, 3), "peak": primary.peak,
                      "unit": primary.unit, "frac": round(achieved / primary.peak, 4),
-                     "traffic": MEASURED_TRAFFIC.get(args.workload),
+                     "traffic": traffic_from_profile(args.workload),
                      "kernel": primary.kernel, "kernel_ms": round(dev * 1e3, 5),
                      "timing": "HIP events on the launch stream around the timed steps / steps"},
+        "clock_state": ("cold start" if args.no_conditioning else
+                        f"steady state: {CONDITION_SECONDS} s of untimed load before the warm-up steps (clocks settled)"),
         "clock_conditioning_s": 0.0 if args.no_conditioning else CONDITION_SECONDS,
         "device": {"name": props.name, "cus": props.multi_processor_count,
                    "peak_used": f"{primary.peak} {primary.unit}"},
@@ -354,11 +394,14 @@ def main():
             if key == args.workload:
                 continue
             r = Runner(key, torch, va)
-            steps = max(10, args.steps // 2)
-            w_, d_ = time_steps(torch, r.step, steps, max(3, args.warmup // 2), not args.no_conditioning)
+            steps = max(50, args.steps)
+            w_, d_, st_ = time_steps(torch, r.step, steps, max(3, args.warmup // 2), not args.no_conditioning)
             others[key] = {"workload": r.w["name"], "value": round(r.rate(w_), 3), "unit": r.unit,
                            "ms_per_step": round(w_ * 1e3, 5), "kernel_ms": round(d_ * 1e3, 5),
+                           "median_ms": st_["median_ms"], "min_ms": st_["min_ms"],
                            "roofline_frac": round(r.rate(d_) / r.peak, 4), "bound": r.bound, "steps": steps}
+            if traffic_from_profile(key):
+                others[key]["traffic"] = traffic_from_profile(key)
             del r
             torch.cuda.empty_cache()
         result["other_workloads"] = others
@@ -366,6 +409,10 @@ def main():
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(args.workload)
         result["cpu_baseline"]["host_cores_available"] = os.cpu_count()
+        # the decode configs get their own CPU figure (a one-sequence slice, about a second each)
+        for key in ("c4", "c5"):
+            if key in result.get("other_workloads", {}):
+                result["other_workloads"][key]["cpu_baseline"] = cpu_baseline(key)
 
     print(json.dumps(result))
 
