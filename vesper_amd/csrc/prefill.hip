@@ -467,11 +467,15 @@ constexpr int kLead = 6;  // LDS operand reads run this many MFMA slots ahead
 // The QK chain finishes at slot 10, so that the row maximum of the new scores is taken under the last PV MFMAs.
 constexpr int kSlotIsQ[16] = {1, 1, 0, 1, 1, 0, 1, 1, 0, 1, 1, 0, 0, 0, 0, 0};
 constexpr int kSlotIdx[16] = {0, 1, 0, 2, 3, 1, 4, 5, 2, 6, 7, 3, 4, 5, 6, 7};
-constexpr int slot_reads(int s) { return kSlotIsQ[s & 15] ? 1 : 2; }
+// LDS read instructions per operand: one ds_read_b128 for K rows and for V^T taken from a token-blocked plane, two
+// transposing reads for V^T taken from row-major V
+template <bool VBLK>
+constexpr int slot_reads(int s) { return (kSlotIsQ[s & 15] || VBLK) ? 1 : 2; }
 // LDS reads issued after the operand of slot s and before the wait at slot s: those of slots s+1 .. s+kLead-1
+template <bool VBLK>
 constexpr int reads_behind(int s) {
     int n = 0;
-    for (int k = 1; k < kLead; ++k) n += slot_reads(s + k);
+    for (int k = 1; k < kLead; ++k) n += slot_reads<VBLK>(s + k);
     return n;
 }
 
@@ -489,6 +493,9 @@ __device__ inline void frag_wait_v(uint2& t0, uint2& t1) {
     asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(t0), "+v"(t1) : "n"(N));
 }
 
+// VBLK: K and V are the planes of a bf16 KV cache (K row-major, V token-blocked by 8), possibly paged, with the context
+// length per batch row from a device array; see prefill_bf16_kernel for the operand layouts this implies.
+template <bool VBLK>
 __global__ void __launch_bounds__(256, 2) prefill_bf16_pipe_kernel(PrefillArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the body uses device-only builtins
     constexpr int D = 128;
@@ -520,12 +527,19 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_pipe_kernel(PrefillArgs a
         bh = grp * a.n_rep + slot % a.n_rep;
     }
     const int b = bh / a.Hq, hq = bh % a.Hq, kvh = hq / a.n_rep;
-    const int L = a.L;
+    int L = a.L;
+    // cache mode: per-row context length (clamped to the bound a.L) and per-row chunk length n <= T: query t < n sits
+    // at absolute position L - n + t; rows t >= n carry no query and their output is unspecified
+    int n_chunk = a.T;
+    if constexpr (VBLK) {
+        if (a.chunk_lens) n_chunk = min(max(a.chunk_lens[b], 0), a.T);
+        if (a.seq_lens) L = min(max(a.seq_lens[b], n_chunk), a.L);
+    }
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int ql = lane & 31, h = lane >> 5;
     const int q0 = qt * kBM + wave * 32;
-    const int off = L - a.T;
+    const int off = L - n_chunk;
     const int qrow = min(q0 + ql, a.T - 1);
 
     const uint16_t* Qp = (const uint16_t*)a.q + (int64_t)b * a.sq[0] + (int64_t)hq * a.sq[1];
@@ -578,20 +592,48 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_pipe_kernel(PrefillArgs a
     for (int i = 0; i < NLD; ++i) {
         const int r = NR * (wave + 4 * i) + ld_row;
         voffK[i] = (uint32_t)r * (uint32_t)a.sk[2] * 2u + 16u * (uint32_t)(ld_pos ^ ((r / RP) % CPR));
-        voffV[i] = (uint32_t)r * (uint32_t)a.sv[2] * 2u + 16u * (uint32_t)(ld_pos ^ (((r / RP) % (CPR / 4)) << 2));
+        if constexpr (VBLK) voffV[i] = (uint32_t)(wave + 4 * i) * 1024u + 16u * (uint32_t)lane;  // the tile is contiguous
+        else voffV[i] = (uint32_t)r * (uint32_t)a.sv[2] * 2u + 16u * (uint32_t)(ld_pos ^ (((r / RP) % (CPR / 4)) << 2));
     }
     const int64_t rowK = a.sk[2] * 2, rowV = a.sv[2] * 2;
+    // where the 32-token tile starting at key0 lives: the head's slab and the first token inside it (a tile never
+    // straddles a page: pages are multiples of 64 tokens)
+    auto locate_tile = [&](int key0, const char*& kb, const char*& vb, int& local, int& cap, int& rows) {
+        kb = (const char*)Kp;
+        vb = (const char*)Vp;
+        local = key0;
+        cap = a.s_pad;
+        rows = L - key0;
+        if constexpr (VBLK) {
+            if (a.page_table) {
+                const int pg = key0 / a.page_tokens;
+                local = key0 - pg * a.page_tokens;
+                cap = a.page_tokens;
+                const int64_t slab = (int64_t)a.page_table[(int64_t)b * a.pages_per_seq + pg] * a.Hkv + kvh;
+                kb = (const char*)a.k + slab * cap * D * 2;
+                vb = (const char*)a.v + slab * cap * D * 2;
+                rows = min(rows, cap - local);
+            }
+        }
+    };
     auto load_k_tile = [&](int t, int slot) {
-        const int key0 = t * kUnit;
-        __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)Kp + (int64_t)key0 * rowK), 0, (int)((int64_t)(L - key0) * rowK), 0x00020000);
+        const char *kb, *vb;
+        int local, cap, rows;
+        locate_tile(t * kUnit, kb, vb, local, cap, rows);
+        __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc((void*)(kb + (int64_t)local * rowK), 0, (int)((int64_t)rows * rowK), 0x00020000);
         uint16_t* dst = smem + slot * SLOT;
 #pragma unroll
         for (int i = 0; i < NLD; ++i)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (__attribute__((address_space(3))) void*)(dst + (wave + 4 * i) * 512), 16, voffK[i], 0, 0, 0);
     };
     auto load_v_tile = [&](int t, int slot) {
-        const int key0 = t * kUnit;
-        __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)Vp + (int64_t)key0 * rowV), 0, (int)((int64_t)(L - key0) * rowV), 0x00020000);
+        const char *kb, *vb;
+        int local, cap, rows;
+        locate_tile(t * kUnit, kb, vb, local, cap, rows);
+        // VBLK: 32 tokens = 4 token blocks = kUnit * D contiguous elements; bound = the rest of this head's slab
+        const int64_t v_base = VBLK ? (int64_t)local * D * 2 : (int64_t)local * rowV;
+        const int64_t v_bytes = VBLK ? ((int64_t)cap - local) * D * 2 : (int64_t)rows * rowV;
+        __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc((void*)(vb + v_base), 0, (int)v_bytes, 0x00020000);
         uint16_t* dst = smem + (NRING + slot) * SLOT;
 #pragma unroll
         for (int i = 0; i < NLD; ++i)
@@ -599,16 +641,18 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_pipe_kernel(PrefillArgs a
     };
 
     // loop-constant LDS read addresses (ring slot 0 of each operand; the slot is an immediate offset)
-    const int kswz = (ql / RP) % CPR;
+    const int krow = VBLK ? ((ql & ~12) | ((ql & 4) << 1) | ((ql & 8) >> 1)) : ql;  // tile row this lane's S^T row holds
+    const int kswz = (krow / RP) % CPR;
     uint32_t kaddr[KS];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) kaddr[ks] = lds0 + 2u * (uint32_t)(ql * D + 8 * ((2 * ks + h) ^ kswz));
+    for (int ks = 0; ks < KS; ++ks) kaddr[ks] = lds0 + 2u * (uint32_t)(krow * D + 8 * ((2 * ks + h) ^ kswz));
     const int i16 = lane & 15;
     const int vswz = ((i16 >> 2) / RP) % (CPR / 4);
     const int v_lane_off = (4 * h + (i16 >> 2)) * D + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
     uint32_t va[DB];
 #pragma unroll
-    for (int db = 0; db < DB; ++db) va[db] = lds0 + 2u * (uint32_t)v_lane_off + 64u * (uint32_t)(db ^ vswz);
+    for (int db = 0; db < DB; ++db)
+        va[db] = VBLK ? lds0 + 16u * (uint32_t)(h * D + ql) : lds0 + 2u * (uint32_t)v_lane_off + 64u * (uint32_t)(db ^ vswz);
 
     Frag fr[16];         // operand of MFMA slot s of the current step (slots < kLead: already requested)
     // Scores are kept as S' = s * scale * log2(e) - m: the factor is folded into Q (below), and -m, the row's reference
@@ -629,9 +673,13 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_pipe_kernel(PrefillArgs a
             fr[S].k = lds_read_b128_asm<RS * SLOTB>(kaddr[ks]);
         } else {
             constexpr int p = kSlotIdx[S], j = p / 4, db = p % 4;
-            constexpr int VOFF = (NRING + RS) * SLOTB + 16 * j * D * 2;
-            fr[S].t0 = lds_read_tr16_b64_asm<VOFF>(va[db]);
-            fr[S].t1 = lds_read_tr16_b64_asm<VOFF + 8 * D * 2>(va[db]);
+            if constexpr (VBLK) {  // token block 2j + h of the tile, rows d = 32 db + ql: one 16-byte read
+                fr[S].k = lds_read_b128_asm<(NRING + RS) * SLOTB + (2 * j * D + 32 * db) * 16>(va[db]);
+            } else {
+                constexpr int VOFF = (NRING + RS) * SLOTB + 16 * j * D * 2;
+                fr[S].t0 = lds_read_tr16_b64_asm<VOFF>(va[db]);
+                fr[S].t1 = lds_read_tr16_b64_asm<VOFF + 8 * D * 2>(va[db]);
+            }
         }
     };
 
@@ -684,16 +732,31 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_pipe_kernel(PrefillArgs a
             // ---- the MFMA of this slot
             if constexpr (kSlotIsQ[S]) {
                 constexpr int ks = kSlotIdx[S];
-                frag_wait_k<reads_behind(S)>(fr[S].k);
+                frag_wait_k<reads_behind<VBLK>(S)>(fr[S].k);
                 if (qk_on) {
                     if constexpr (ks == 0) s_nxt = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, fr[S].k), qf[ks], negm, 0, 0, 0);
                     else s_nxt = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, fr[S].k), qf[ks], s_nxt, 0, 0, 0);
                 }
             } else {
                 constexpr int p = kSlotIdx[S], j = p / 4, db = p % 4;
-                frag_wait_v<reads_behind(S)>(fr[S].t0, fr[S].t1);
+                if constexpr (VBLK) frag_wait_k<reads_behind<VBLK>(S)>(fr[S].k);
+                else frag_wait_v<reads_behind<VBLK>(S)>(fr[S].t0, fr[S].t1);
                 if (pv_on) {
-                    const bf16x8_t vf = __builtin_bit_cast(bf16x8_t, uint4{fr[S].t0.x, fr[S].t0.y, fr[S].t1.x, fr[S].t1.y});
+                    if constexpr (VBLK && MODE >= 2) {
+                        // the planes hold stale tokens past L: P is 0 there, V must not be NaN
+                        const int nvalid = L - (tau * kUnit + 16 * j + 8 * h);  // slots e >= nvalid are past the context
+                        if (nvalid < 8) {
+#pragma unroll
+                            for (int w = 0; w < 4; ++w) {
+                                uint32_t x = fr[S].k[w];
+                                if (2 * w + 1 >= nvalid) x &= 0x0000ffffu;
+                                if (2 * w >= nvalid) x = 0;
+                                fr[S].k[w] = x;
+                            }
+                        }
+                    }
+                    const bf16x8_t vf = VBLK ? __builtin_bit_cast(bf16x8_t, fr[S].k)
+                                             : __builtin_bit_cast(bf16x8_t, uint4{fr[S].t0.x, fr[S].t0.y, fr[S].t1.x, fr[S].t1.y});
                     const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, uint4{p_cur[4 * j], p_cur[4 * j + 1], p_cur[4 * j + 2], p_cur[4 * j + 3]});
                     acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf, acc[db], 0, 0, 0);
                 }
@@ -713,7 +776,7 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_pipe_kernel(PrefillArgs a
                         const int lim = a.causal ? min(q_abs, L - 1) : L - 1;
 #pragma unroll
                         for (int v = 0; v < 16; ++v)
-                            if (k0 + 8 * (v >> 2) + 4 * h + (v & 3) > lim) s_nxt[v] = -INFINITY;
+                            if ((VBLK ? k0 + 16 * (v >> 3) + 8 * h + (v & 7) : k0 + 8 * (v >> 2) + 4 * h + (v & 3)) > lim) s_nxt[v] = -INFINITY;
                     }
                 }
             }
@@ -766,6 +829,7 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_pipe_kernel(PrefillArgs a
     using First = std::integral_constant<int, 3>;   // step -2: Slow, and the tiles three steps ahead were requested by the prologue
     using Second = std::integral_constant<int, 4>;  // step -1: Slow, and its softmax stage sets the reference from tile 0
 
+    if (n_tiles > 0) {  // an empty context (cache mode, length 0) has nothing to attend to: zeros below
     // prologue: the tiles of steps -2 and -1 (K(0), K(1)) are requested here, published by the barrier below
     load_k_tile(0, 2);
     load_k_tile(min(1, n_tiles - 1), 3);
@@ -802,6 +866,9 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_pipe_kernel(PrefillArgs a
     }
     // operands requested for a step that does not exist are still in flight: let them land before the registers die
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    } else {
+        prescale_q();
+    }
 
     l = half_swap_sum(l);
     const int qi = q0 + ql;
@@ -959,12 +1026,12 @@ int launch_prefill(const PrefillArgs& a, int dtype, int64_t D, bool cache_planes
     dim3 grid((unsigned)blocks), block(256);
     if (dtype == VSP_BF16) {
         if (cache_planes) {
-            if (D == 128) hipLaunchKernelGGL((prefill_bf16_kernel<128, true>), grid, block, 0, st, a);
+            if (D == 128) hipLaunchKernelGGL(prefill_bf16_pipe_kernel<true>, grid, block, 0, st, a);
             else hipLaunchKernelGGL((prefill_bf16_kernel<64, true>), grid, block, 0, st, a);
         } else {
             // the software-pipelined kernel takes one context length for the batch; dense K/V with per-row lengths
             // (a Q8_0 cache read out into the workspace) stay with the general kernel
-            if (D == 128 && !a.seq_lens && !a.chunk_lens) hipLaunchKernelGGL(prefill_bf16_pipe_kernel, grid, block, 0, st, a);
+            if (D == 128 && !a.seq_lens && !a.chunk_lens) hipLaunchKernelGGL(prefill_bf16_pipe_kernel<false>, grid, block, 0, st, a);
             else if (D == 128) hipLaunchKernelGGL((prefill_bf16_kernel<128, false>), grid, block, 0, st, a);
             else hipLaunchKernelGGL((prefill_bf16_kernel<64, false>), grid, block, 0, st, a);
         }
