@@ -55,6 +55,10 @@ struct AppendArgs {
     int64_t Hq, T;
     int64_t kv_items;      // threads of the K/V part; the Q part follows
     int32_t q_out_bf16;
+    int32_t q_vec;         // q rows and q_out rows are 16-byte aligned: whole 16-byte loads and stores
+    int32_t small_index;   // every item count of the launch is below 2^31
+    int64_t blocks_per_row;  // tile kernels: token blocks one (batch row, head) slot can touch
+    int64_t q_tblocks;       // tile kernels: workgroups of the Q rotation per (batch row, query head)
     // paged cache (kv_locate): table == nullptr for a contiguous one
     const int32_t* page_table;
     int32_t page_tokens, pages_per_seq;
@@ -76,39 +80,109 @@ __device__ inline void rope_rotate(float (&x)[N], int64_t d0, int64_t pos, const
 #pragma clang fp contract(off)  // no fused multiply-add: the products are rounded before the sum
     if (pos >= a.table_len) pos = a.table_len - 1;
     if (pos < 0) pos = 0;
-    const float2* t = (const float2*)a.table + pos * (a.D / 2) + d0 / 2;
+    // N is a multiple of 4 and d0 of N: two {cos, sin} pairs per 16-byte load
+    const float4* t = (const float4*)((const float2*)a.table + pos * (a.D / 2) + d0 / 2);
 #pragma unroll
-    for (int j = 0; j < N / 2; ++j) {
-        const float2 cs = t[j];
-        const float x0 = x[2 * j], x1 = x[2 * j + 1];
-        const float t1 = x0 * cs.x, t2 = x1 * cs.y, t3 = x0 * cs.y, t4 = x1 * cs.x;
-        x[2 * j] = t1 - t2;
-        x[2 * j + 1] = t3 + t4;
+    for (int j = 0; j < N / 4; ++j) {
+        const float4 cs = t[j];
+        {
+            const float x0 = x[4 * j], x1 = x[4 * j + 1];
+            const float t1 = x0 * cs.x, t2 = x1 * cs.y, t3 = x0 * cs.y, t4 = x1 * cs.x;
+            x[4 * j] = t1 - t2;
+            x[4 * j + 1] = t3 + t4;
+        }
+        {
+            const float x0 = x[4 * j + 2], x1 = x[4 * j + 3];
+            const float t1 = x0 * cs.z, t2 = x1 * cs.w, t3 = x0 * cs.w, t4 = x1 * cs.z;
+            x[4 * j + 2] = t1 - t2;
+            x[4 * j + 3] = t3 + t4;
+        }
     }
 }
 
-// The Q part of the fused launch: item i rotates 8 consecutive d of one query row.
+template <typename SrcT>
+__device__ inline void load8(const SrcT* p, float (&x)[8]) {
+    if constexpr (sizeof(SrcT) == 2) {
+        const uint4 w = *(const uint4*)p;
+        const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            x[2 * j] = __builtin_bit_cast(float, ww[j] << 16);
+            x[2 * j + 1] = __builtin_bit_cast(float, ww[j] & 0xffff0000u);
+        }
+    } else {
+        const float4 lo = *(const float4*)p, hi = *(const float4*)(p + 4);
+        x[0] = lo.x, x[1] = lo.y, x[2] = lo.z, x[3] = lo.w, x[4] = hi.x, x[5] = hi.y, x[6] = hi.z, x[7] = hi.w;
+    }
+}
+// two fp32 -> packed bf16 pair with the reference's rounding (f32_to_bf16_bits): both words are rounded in place and one
+// byte permute picks their high halves
+__device__ inline uint32_t round_pack_bf16x2(float lo, float hi) {
+    uint32_t a = __builtin_bit_cast(uint32_t, lo), b = __builtin_bit_cast(uint32_t, hi);
+    a += 0x7FFFu + ((a >> 16) & 1u);
+    b += 0x7FFFu + ((b >> 16) & 1u);
+    return __builtin_amdgcn_perm(b, a, 0x07060302u);
+}
+__device__ inline uint4 pack8_bf16(const float (&x)[8]) {
+    return uint4{round_pack_bf16x2(x[0], x[1]), round_pack_bf16x2(x[2], x[3]), round_pack_bf16x2(x[4], x[5]), round_pack_bf16x2(x[6], x[7])};
+}
+
+// The Q part of the fused launch: 8 consecutive d (from d0) of query row (b, h, t) are rotated into q_out.
+template <typename SrcT>
+__device__ inline void rope_q_row(const AppendArgs& a, int64_t b, int64_t h, int64_t t, int64_t d0);
+
+// item i of the per-element launches: (row, 8-element piece) in row-major order
 template <typename SrcT>
 __device__ inline void rope_q_item(const AppendArgs& a, int64_t i) {
-    const int64_t per_row = a.D / 8;
-    const int64_t r = i / per_row, d0 = (i % per_row) * 8;
-    const int64_t t = r % a.T, bh = r / a.T;
-    const int64_t h = bh % a.Hq, b = bh / a.Hq;
+    int64_t d0, t, h, b;
+    if (a.small_index) {  // every count fits 32 bits: 64-bit divisions cost several times the rest of the item
+        const uint32_t per_row = (uint32_t)a.D / 8, ii = (uint32_t)i;
+        const uint32_t r = ii / per_row, bh = r / (uint32_t)a.T;
+        d0 = (ii % per_row) * 8;
+        t = r % (uint32_t)a.T;
+        h = bh % (uint32_t)a.Hq;
+        b = bh / (uint32_t)a.Hq;
+    } else {
+        const int64_t per_row = a.D / 8;
+        const int64_t r = i / per_row, bh = r / a.T;
+        d0 = (i % per_row) * 8;
+        t = r % a.T;
+        h = bh % a.Hq;
+        b = bh / a.Hq;
+    }
+    rope_q_row<SrcT>(a, b, h, t, d0);
+}
+
+template <typename SrcT>
+__device__ inline void rope_q_row(const AppendArgs& a, int64_t b, int64_t h, int64_t t, int64_t d0) {
     const int64_t start = a.start_dev ? (int64_t)a.start_dev[b] : a.slot_start;
     const SrcT* p = (const SrcT*)a.q + b * a.sq[0] + h * a.sq[1] + t * a.sq[2] + d0;
     float x[8];
+    if (a.q_vec) {
+        load8<SrcT>(p, x);
+    } else {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) x[j] = load_src<SrcT>(p + j);
+        for (int j = 0; j < 8; ++j) x[j] = load_src<SrcT>(p + j);
+    }
     rope_rotate<8>(x, d0, start + t, a);
     const int64_t o = b * a.so[0] + h * a.so[1] + t * a.so[2] + d0;
     if (a.q_out_bf16) {
         uint16_t* dst = (uint16_t*)a.q_out + o;
+        if (a.q_vec) {
+            *(uint4*)dst = pack8_bf16(x);
+        } else {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) dst[j] = f32_to_bf16_bits(x[j]);
+            for (int j = 0; j < 8; ++j) dst[j] = f32_to_bf16_bits(x[j]);
+        }
     } else {
         float* dst = (float*)a.q_out + o;
+        if (a.q_vec) {
+            *(float4*)dst = float4{x[0], x[1], x[2], x[3]};
+            *(float4*)(dst + 4) = float4{x[4], x[5], x[6], x[7]};
+        } else {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) dst[j] = x[j];
+            for (int j = 0; j < 8; ++j) dst[j] = x[j];
+        }
     }
 }
 
@@ -280,6 +354,188 @@ __global__ void __launch_bounds__(128) append_q8_kernel(AppendArgs a) {
 #pragma unroll
         for (int j = 0; j < kQBlock; ++j) dv[j * kVBlkQ8] = q[j];
         ((uint16_t*)a.v_scale)[kv_off_vscale(a.H, a.S, a.D, m.b, m.h, m.s, blk)] = sc;
+    }
+}
+
+// ---- appends of eight tokens or more: one workgroup per (batch row, kv head, token block) ---------------------
+// The per-element kernels above write the token-blocked V planes two bytes (bf16) or one byte (Q8_0) at a time, 16
+// bytes apart.  Here a workgroup owns one token block (8 bf16 / 16 int8 tokens of one head): the rows are loaded and
+// converted in 16-byte pieces, V is transposed through LDS, and whole blocks leave as 16-byte stores to consecutive
+// addresses.  Blocks the slot covers only partly (its first and last) keep their other tokens: those are written
+// element by element.  Same arithmetic as the per-element kernels, so the planes come out bit for bit the same.
+// Preconditions (checked on the host): source shape == slot shape, source rows 16-byte aligned.
+constexpr int kQPerThread = 4;     // rows of the Q rotation per thread in the token-block launches
+constexpr int kQRowsPerPass = 8;   // a workgroup of D threads covers D / (D / 8) = 8 rows at a time
+constexpr int kQRows = kQPerThread * kQRowsPerPass;
+struct TileRow {
+    int64_t pb, ps0;   // plane coordinates of the block's first token (page and token within it when paged)
+    int64_t start;     // first position of the slot in this batch row
+    int lo, hi;        // tokens [lo, hi) of the block belong to the slot (and to the cache)
+};
+template <int BLK>
+__device__ inline TileRow tile_row(const AppendArgs& a, int64_t b, int64_t j) {
+    TileRow r;
+    r.start = a.start_dev ? (int64_t)a.start_dev[b] : a.slot_start;
+    const int64_t first_blk = r.start >= 0 ? r.start / BLK : -((-r.start + BLK - 1) / BLK);
+    const int64_t s0 = (first_blk + j) * BLK;
+    const int64_t lo = max(max(r.start, (int64_t)0), s0), hi = min(min(r.start + a.slot_len, a.S_logical), s0 + BLK);
+    r.lo = (int)(lo - s0);
+    r.hi = (int)(hi - s0);
+    r.pb = b;
+    r.ps0 = s0;
+    if (r.lo < r.hi) kv_locate(a.page_table, a.page_tokens, a.pages_per_seq, r.pb, r.ps0);
+    return r;
+}
+
+template <typename SrcT, bool ROPE, int D>
+__global__ void __launch_bounds__(D) append_bf16_tile_kernel(AppendArgs a, int64_t n_tile_wgs) {
+    constexpr int BLK = kVBlkBf16;
+    constexpr int CH = D / 8;          // 16-byte pieces per row
+    constexpr int PITCH = D + 8;       // LDS row pitch in elements: rows start 16 bytes apart modulo the bank cycle
+    __shared__ __attribute__((aligned(16))) uint16_t tile[BLK * PITCH];
+    const int tid = threadIdx.x;
+    if constexpr (ROPE) {
+        if ((int64_t)blockIdx.x >= n_tile_wgs) {
+            // a workgroup rotates kQRows consecutive rows of one (batch row, query head): its place is decoded once
+            // per workgroup, and every lane has kQPerThread independent 16-byte loads in flight
+            const uint32_t qi = (uint32_t)(blockIdx.x - n_tile_wgs), n_tb = (uint32_t)a.q_tblocks;
+            const uint32_t bh = qi / n_tb, tb = qi % n_tb;
+            const int64_t b = bh / (uint32_t)a.Hq, h = bh % (uint32_t)a.Hq;
+#pragma unroll
+            for (int u = 0; u < kQPerThread; ++u) {
+                const int64_t t = (int64_t)tb * kQRows + u * kQRowsPerPass + tid / (D / 8);
+                if (t < a.T) rope_q_row<SrcT>(a, b, h, t, 8 * (tid % (D / 8)));
+            }
+            return;
+        }
+    }
+    const uint32_t bpr = (uint32_t)a.blocks_per_row, bh = blockIdx.x / bpr;
+    const int64_t j = blockIdx.x % bpr, h = bh % (uint32_t)a.H, b = bh / (uint32_t)a.H;
+    const TileRow r = tile_row<BLK>(a, b, j);
+    if (r.lo >= r.hi) return;  // uniform for the workgroup
+    const int tok = tid / CH, d0 = 8 * (tid % CH);
+    if (tok >= r.lo && tok < r.hi) {
+        const int64_t s = r.ps0 + tok;                                   // token inside its slab
+        const int64_t pos = (int64_t)((r.start >= 0 ? r.start / BLK : -((-r.start + BLK - 1) / BLK)) + j) * BLK + tok;  // position in the sequence
+        const int64_t t = pos - r.start;
+        const SrcT* pk = (const SrcT*)a.src_k + b * a.sk[0] + h * a.sk[1] + t * a.sk[2] + d0;
+        const SrcT* pv = (const SrcT*)a.src_v + b * a.sv[0] + h * a.sv[1] + t * a.sv[2] + d0;
+        uint4 kq, vq;
+        if constexpr (sizeof(SrcT) == 2 && !ROPE) {
+            kq = *(const uint4*)pk;  // bf16 to bf16: the bits travel as they are
+        } else {
+            float xk[8];
+            load8<SrcT>(pk, xk);
+            if constexpr (ROPE) rope_rotate<8>(xk, d0, pos, a);
+            kq = pack8_bf16(xk);
+        }
+        if constexpr (sizeof(SrcT) == 2) {
+            vq = *(const uint4*)pv;
+        } else {
+            float xv[8];
+            load8<SrcT>(pv, xv);
+            vq = pack8_bf16(xv);
+        }
+        *(uint4*)((uint16_t*)a.k + kv_off_rowmajor(a.H, a.S, a.D, r.pb, h, s, d0)) = kq;
+        *(uint4*)(tile + tok * PITCH + d0) = vq;
+    }
+    __syncthreads();
+    // thread d owns one row of the transposed block: [d][8 tokens]
+    const int d = tid;
+    uint16_t* dv = (uint16_t*)a.v + kv_off_vblocked(a.H, a.S, a.D, BLK, r.pb, h, r.ps0, d);
+    if (r.lo == 0 && r.hi == BLK) {
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[i] = tile[(2 * i) * PITCH + d] | ((uint32_t)tile[(2 * i + 1) * PITCH + d] << 16);
+        *(uint4*)dv = uint4{w[0], w[1], w[2], w[3]};
+    } else {
+        for (int i = r.lo; i < r.hi; ++i) dv[i] = tile[i * PITCH + d];
+    }
+}
+
+// Q8_0: a token block is 16 tokens; thread i < D/2 quantises a 32-wide block of K, thread i >= D/2 one of V.
+template <typename SrcT, bool ROPE, int D>
+__global__ void __launch_bounds__(D) append_q8_tile_kernel(AppendArgs a, int64_t n_tile_wgs) {
+    constexpr int BLK = kVBlkQ8;
+    constexpr int NQ = D / kQBlock;    // quantisation blocks per row
+    constexpr int PITCH = D + 16;      // bytes
+    __shared__ __attribute__((aligned(16))) int8_t tile[BLK * PITCH];
+    __shared__ uint16_t tile_sc[NQ * BLK];  // [blk][token], the layout of the V scale plane inside a token block
+    const int tid = threadIdx.x;
+    if constexpr (ROPE) {
+        if ((int64_t)blockIdx.x >= n_tile_wgs) {
+            // a workgroup rotates kQRows consecutive rows of one (batch row, query head): its place is decoded once
+            // per workgroup, and every lane has kQPerThread independent 16-byte loads in flight
+            const uint32_t qi = (uint32_t)(blockIdx.x - n_tile_wgs), n_tb = (uint32_t)a.q_tblocks;
+            const uint32_t bh = qi / n_tb, tb = qi % n_tb;
+            const int64_t b = bh / (uint32_t)a.Hq, h = bh % (uint32_t)a.Hq;
+#pragma unroll
+            for (int u = 0; u < kQPerThread; ++u) {
+                const int64_t t = (int64_t)tb * kQRows + u * kQRowsPerPass + tid / (D / 8);
+                if (t < a.T) rope_q_row<SrcT>(a, b, h, t, 8 * (tid % (D / 8)));
+            }
+            return;
+        }
+    }
+    const uint32_t bpr = (uint32_t)a.blocks_per_row, bh = blockIdx.x / bpr;
+    const int64_t j = blockIdx.x % bpr, h = bh % (uint32_t)a.H, b = bh / (uint32_t)a.H;
+    const TileRow r = tile_row<BLK>(a, b, j);
+    if (r.lo >= r.hi) return;
+    const bool is_v = tid >= D / 2;
+    const int item = is_v ? tid - D / 2 : tid;  // BLK tokens x NQ blocks = D / 2 items per plane
+    const int tok = item / NQ, blk = item % NQ, d0 = blk * kQBlock;
+    if (tok >= r.lo && tok < r.hi) {
+        const int64_t s = r.ps0 + tok;
+        const int64_t pos = (int64_t)((r.start >= 0 ? r.start / BLK : -((-r.start + BLK - 1) / BLK)) + j) * BLK + tok;
+        const int64_t t = pos - r.start;
+        const SrcT* p = is_v ? (const SrcT*)a.src_v + b * a.sv[0] + h * a.sv[1] + t * a.sv[2] + d0
+                             : (const SrcT*)a.src_k + b * a.sk[0] + h * a.sk[1] + t * a.sk[2] + d0;
+        float x[kQBlock];
+#pragma unroll
+        for (int c = 0; c < kQBlock / 8; ++c) {
+            float y[8];
+            load8<SrcT>(p + 8 * c, y);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[8 * c + e] = y[e];
+        }
+        if constexpr (ROPE) {
+            if (!is_v) rope_rotate<kQBlock>(x, d0, pos, a);
+        }
+        int8_t q[kQBlock];
+        uint16_t sc;
+        quantize_block(x, q, &sc);
+        uint32_t w[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            w[e] = (uint32_t)(uint8_t)q[4 * e] | ((uint32_t)(uint8_t)q[4 * e + 1] << 8) | ((uint32_t)(uint8_t)q[4 * e + 2] << 16) |
+                   ((uint32_t)(uint8_t)q[4 * e + 3] << 24);
+        if (!is_v) {
+            uint4* dk = (uint4*)((int8_t*)a.k + kv_off_rowmajor(a.H, a.S, a.D, r.pb, h, s, d0));
+            dk[0] = uint4{w[0], w[1], w[2], w[3]};
+            dk[1] = uint4{w[4], w[5], w[6], w[7]};
+            ((uint16_t*)a.k_scale)[kv_off_kscale(a.H, a.S, a.D, r.pb, h, s, blk)] = sc;
+        } else {
+            uint4* dt = (uint4*)(tile + tok * PITCH + d0);
+            dt[0] = uint4{w[0], w[1], w[2], w[3]};
+            dt[1] = uint4{w[4], w[5], w[6], w[7]};
+            tile_sc[blk * BLK + tok] = sc;
+        }
+    }
+    __syncthreads();
+    const int d = tid;  // row d of the transposed block: [d][16 tokens]
+    int8_t* dv = (int8_t*)a.v + kv_off_vblocked(a.H, a.S, a.D, BLK, r.pb, h, r.ps0, d);
+    uint16_t* ds = (uint16_t*)a.v_scale + kv_off_vscale(a.H, a.S, a.D, r.pb, h, r.ps0, 0);  // NQ x 16 scales, contiguous
+    if (r.lo == 0 && r.hi == BLK) {
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            w[i] = (uint32_t)(uint8_t)tile[(4 * i) * PITCH + d] | ((uint32_t)(uint8_t)tile[(4 * i + 1) * PITCH + d] << 8) |
+                   ((uint32_t)(uint8_t)tile[(4 * i + 2) * PITCH + d] << 16) | ((uint32_t)(uint8_t)tile[(4 * i + 3) * PITCH + d] << 24);
+        *(uint4*)dv = uint4{w[0], w[1], w[2], w[3]};
+        if (tid < NQ * BLK) ds[tid] = tile_sc[tid];
+    } else {
+        for (int i = r.lo; i < r.hi; ++i) dv[i] = tile[i * PITCH + d];
+        if (tid < NQ * BLK && (tid % BLK) >= r.lo && (tid % BLK) < r.hi) ds[tid] = tile_sc[tid];
     }
 }
 
@@ -538,7 +794,45 @@ static int append_impl(vsp_kv_cache* cache, const vsp_tensor* new_k, const vsp_t
             a.kv_items = ceil_div(kv_items, threads) * threads;
             return dim3((unsigned)(a.kv_items / threads + ceil_div(q_items, threads)));
         };
-        if (cache->format == VSP_KV_F32) {
+        auto rows_aligned16 = [](const vsp_tensor* t) {
+            const int esz = t->dtype == VSP_F32 ? 4 : 2;
+            if (!is_aligned16(t->data)) return false;
+            for (int i = 0; i < 3; ++i)
+                if ((t->stride[i] * esz) % 16 != 0) return false;
+            return true;
+        };
+        if (rope) a.q_vec = rows_aligned16(rope->q) && rows_aligned16(rope->q_out) ? 1 : 0;
+        a.small_index = (q_items < INT32_MAX && slot_numel < INT32_MAX) ? 1 : 0;
+        // eight tokens or more of the cache's own shape, rows 16-byte aligned: the token-block kernels
+        const bool tiles = cache->format != VSP_KV_F32 && (a.D == 64 || a.D == 128) && slot_len >= 8 && a.nB == a.B && a.nH == a.H &&
+                           a.nT == slot_len && rows_aligned16(new_k) && rows_aligned16(new_v);
+        if (tiles) {
+            const int BLK = cache->format == VSP_KV_BF16 ? kVBlkBf16 : kVBlkQ8;
+            a.blocks_per_row = ceil_div(slot_len, BLK) + 1;  // a slot that starts inside a block touches one more
+            const int64_t n_tile_wgs = a.B * a.H * a.blocks_per_row;
+            const int threads = (int)a.D;
+            a.q_tblocks = rope ? ceil_div(T, kQRows) : 0;
+            const int64_t total = n_tile_wgs + (rope ? a.nB * a.Hq * a.q_tblocks : 0);
+            if (total > INT32_MAX) return VSP_ERR_ARG;
+            const dim3 grid((unsigned)total), block((unsigned)threads);
+#define VSP_LAUNCH_TILE(KERNEL)                                                                                               \
+    do {                                                                                                                      \
+        if (a.D == 128) {                                                                                                     \
+            if (f32src && r) hipLaunchKernelGGL((KERNEL<float, true, 128>), grid, block, 0, st, a, n_tile_wgs);                \
+            else if (f32src) hipLaunchKernelGGL((KERNEL<float, false, 128>), grid, block, 0, st, a, n_tile_wgs);               \
+            else if (r) hipLaunchKernelGGL((KERNEL<uint16_t, true, 128>), grid, block, 0, st, a, n_tile_wgs);                  \
+            else hipLaunchKernelGGL((KERNEL<uint16_t, false, 128>), grid, block, 0, st, a, n_tile_wgs);                        \
+        } else {                                                                                                              \
+            if (f32src && r) hipLaunchKernelGGL((KERNEL<float, true, 64>), grid, block, 0, st, a, n_tile_wgs);                 \
+            else if (f32src) hipLaunchKernelGGL((KERNEL<float, false, 64>), grid, block, 0, st, a, n_tile_wgs);                \
+            else if (r) hipLaunchKernelGGL((KERNEL<uint16_t, true, 64>), grid, block, 0, st, a, n_tile_wgs);                   \
+            else hipLaunchKernelGGL((KERNEL<uint16_t, false, 64>), grid, block, 0, st, a, n_tile_wgs);                         \
+        }                                                                                                                     \
+    } while (0)
+            if (cache->format == VSP_KV_BF16) VSP_LAUNCH_TILE(append_bf16_tile_kernel);
+            else VSP_LAUNCH_TILE(append_q8_tile_kernel);
+#undef VSP_LAUNCH_TILE
+        } else if (cache->format == VSP_KV_F32) {
             dim3 grid = blocks(a.rows * (a.D / 4), 256);
             if (f32src && r) hipLaunchKernelGGL((append_f32_kernel<float, true>), grid, dim3(256), 0, st, a);
             else if (f32src) hipLaunchKernelGGL((append_f32_kernel<float, false>), grid, dim3(256), 0, st, a);
