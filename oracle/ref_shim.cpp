@@ -17,6 +17,7 @@
 #include <vesper/nn/functional.h>
 #include <vesper/nn/transformer.h>
 #include <vesper/nn/gqa_attention.h>
+#include <vesper/nn/linear.h>
 #include <vesper/core/half.h>
 
 #include <cstring>
@@ -276,6 +277,19 @@ int vref_gqa_rope_core(void* c, const float* q, const float* new_k, const float*
 }
 
 // BFloat16(float) / operator float (include/vesper/core/half.h:162-181).
+// nn::Linear::forward (src/nn/linear.cpp:41-49) on a 3-D activation [B, T, K], the way the attention modules
+// call their output projection (src/nn/gqa_attention.cpp:151-152): weight [N, K], bias [N] or NULL.
+int vref_linear(const float* x, const float* w, const float* bias, float* y, int64_t B, int64_t T, int64_t K, int64_t N) {
+    return guarded([&] {
+        vesper::nn::Linear lin(K, N, bias != nullptr, Device::CPU);
+        lin.weight.copy_from_host(w);
+        if (bias) lin.bias.copy_from_host(bias);
+        Tensor tx = from_host(x, {B, T, K});
+        Tensor ty = lin.forward(tx);
+        to_host(ty, y);
+    });
+}
+
 uint16_t vref_f32_to_bf16(float f) { return vesper::BFloat16(f).to_bits(); }
 float vref_bf16_to_f32(uint16_t b) { return float(vesper::BFloat16::from_bits(b)); }
 

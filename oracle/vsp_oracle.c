@@ -254,6 +254,22 @@ int orc_gqa_config(int64_t embed_dim, int64_t num_heads, int64_t num_kv_heads, i
 }
 
 /* ------------------------------------------------------------------------ */
+/* The output projection of the attention modules: out = wo_.forward(out) with out [B, T, C_in]
+ * (src/nn/gqa_attention.cpp:151-152, src/nn/transformer.cpp:148-151,207-210).  Linear::forward
+ * (src/nn/linear.cpp:41-49) is ops::matmul(input, weight.transpose(0, 1)) followed by ops::add(output, bias);
+ * a 3-D input against a 2-D weight takes gemm's batched branch (src/ops/gemm.cpp:130-138), whose CPU loop
+ * (:254-279) sums the K products of every output element in index order into one fp32 accumulator.
+ * x [M, K] (M = B * T rows), w [N, K] = Linear::weight, bias [N] or NULL, y [M, N]. */
+void orc_linear_f32(const float* x, const float* w, const float* bias, float* y, int64_t M, int64_t K, int64_t N) {
+    for (int64_t m = 0; m < M; ++m)
+        for (int64_t n = 0; n < N; ++n) {
+            float sum = 0.0f;
+            for (int64_t k = 0; k < K; ++k) sum += x[m * K + k] * w[n * K + k];
+            y[m * N + n] = bias ? sum + bias[n] : sum;
+        }
+}
+
+/* ------------------------------------------------------------------------ */
 /* src/ops/view_ops.cpp:266-316 */
 int orc_slice_bounds(int64_t dim_size, int has_start, int64_t start_in, int has_stop, int64_t stop_in,
                      int has_step, int64_t step_in, int64_t* out_start, int64_t* out_len) {

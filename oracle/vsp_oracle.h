@@ -114,6 +114,11 @@ int orc_gqa_attention_f32(const float* q, const float* k, const int64_t* ks, con
                           int64_t D, int64_t n_rep, int is_causal);
 
 /* GroupedQueryAttention constructor checks, src/nn/gqa_attention.cpp:38-57. */
+/* Linear::forward on a 3-D activation (the modules' output projection wo_ / c_proj): y = x w^T + bias,
+ * src/nn/linear.cpp:41-49 over src/ops/gemm.cpp:254-279.  Pinned bit-exact to the compiled reference
+ * (tests/test_oracle_linear.py) and to a float64 product within rounding. */
+void orc_linear_f32(const float* x, const float* w, const float* bias, float* y, int64_t M, int64_t K, int64_t N);
+
 int orc_gqa_config(int64_t embed_dim, int64_t num_heads, int64_t num_kv_heads, int64_t* head_dim,
                    int64_t* num_rep);
 

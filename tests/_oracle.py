@@ -79,6 +79,8 @@ def _load_oracle():
     L.orc_rope_angles.argtypes = [C.c_int, C.c_int, C.c_int, C.c_float, f32p]
     L.orc_rope_angles.restype = None
     L.orc_rope_apply_f32.argtypes = [f32p] + [i64] * 4 + [f32p, f32p]
+    L.orc_linear_f32.argtypes = [f32p, f32p, f32p, f32p, i64, i64, i64]
+    L.orc_linear_f32.restype = None
     L.orc_rope_apply_f32.restype = None
     return L
 
@@ -289,6 +291,18 @@ def rope_apply(x, angles):
     return out
 
 
+def linear(x, w, bias=None):
+    """Linear::forward on a [..., K] activation: x w^T + bias, the modules' output projection."""
+    x, w = _f32(x), _f32(w)
+    K, N = x.shape[-1], w.shape[0]
+    assert w.shape == (N, K)
+    M = x.size // K
+    y = np.empty(x.shape[:-1] + (N,), np.float32)
+    b = _f32(bias) if bias is not None else None
+    orc.orc_linear_f32(_p(x), _p(w), _p(b) if b is not None else None, _p(y), M, K, N)
+    return y
+
+
 # ---- the compiled reference (optional) ----------------------------------------------------
 
 def _load_ref():
@@ -324,6 +338,8 @@ def _load_ref():
         L.vref_rope_frequencies.argtypes = [C.c_int, C.c_int, C.c_int, C.c_float, f32p]
         L.vref_apply_rotary_emb.argtypes = [f32p] + [i64] * 4 + [f32p, f32p]
         L.vref_gqa_rope_core.argtypes = [C.c_void_p, f32p, f32p, f32p] + [i64] * 5 + [C.c_int, C.c_float, f32p, f32p]
+    if hasattr(L, "vref_linear"):
+        L.vref_linear.argtypes = [f32p, f32p, f32p, f32p] + [i64] * 4
     L.vref_f32_to_bf16.argtypes = [C.c_float]
     L.vref_f32_to_bf16.restype = C.c_uint16
     L.vref_bf16_to_f32.argtypes = [C.c_uint16]
@@ -458,6 +474,17 @@ def ref_rope_apply(x, angles):
     out = np.empty_like(x)
     _rchk(ref.vref_apply_rotary_emb(_p(x), B, H, S, D, _p(angles), _p(out)))
     return out
+
+
+def ref_linear(x, w, bias=None):
+    """x [B, T, K] through the compiled reference's nn::Linear(K, N) with the given weight [N, K] and bias [N]."""
+    x, w = _f32(x), _f32(w)
+    B, T, K = x.shape
+    N = w.shape[0]
+    y = np.empty((B, T, N), np.float32)
+    b = _f32(bias) if bias is not None else None
+    _rchk(ref.vref_linear(_p(x), _p(w), _p(b) if b is not None else None, _p(y), B, T, K, N))
+    return y
 
 
 def ref_gqa_ctor(embed_dim, num_heads, num_kv_heads):
