@@ -274,6 +274,21 @@ int vsp_attn_decode(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_
 int vsp_attn_decode_noalloc(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, int32_t max_len,
                             vsp_tensor* out, float scale, void* stream);
 
+/* Decode step plus the attention module's output projection in one call: replaces, for T == 1, the chain above
+ * together with what follows it in GroupedQueryAttention::forward and MultiHeadAttention::forward -- the heads
+ * merged by transpose(1,2).reshape({B,T,C}) and wo_ / out_proj applied (src/nn/gqa_attention.cpp:151-152,
+ * src/nn/transformer.cpp:207-215; Linear::forward, src/nn/linear.cpp:41-49: y = x W^T + bias).
+ * q, cache, seq_lens, max_len, scale: as vsp_attn_decode.  wo: [N, Hq*D], row pitch and base 16-byte aligned;
+ * bias: [N] or NULL; y: [B, 1, N]; all of q's dtype (bf16 over VSP_KV_BF16 / VSP_KV_Q8_0 caches, fp32 over
+ * VSP_KV_F32).  The merged heads never become a caller tensor: the combine kernel leaves them, rounded to q's dtype
+ * exactly as vsp_attn_decode's `out` would hold them, at the head of `workspace`, and a projection kernel streams
+ * W over them once (bf16: 16x16x32 MFMA, fp32 accumulation, the four K-partials of a tile summed in a fixed order;
+ * bitwise run-to-run deterministic).  workspace >= vsp_attn_decode_proj_workspace_bytes(), 16-byte aligned. */
+size_t vsp_attn_decode_proj_workspace_bytes(int32_t B, int32_t Hq, int32_t D, int32_t max_len);
+int vsp_attn_decode_proj(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, int32_t max_len,
+                         const vsp_tensor* wo, const vsp_tensor* bias, vsp_tensor* y, float scale, void* workspace,
+                         size_t workspace_bytes, void* stream);
+
 /* ---- host-side, bit-exact format helpers (pure CPU; exported for tests and callers) ---- */
 uint16_t vsp_f32_to_bf16(float f);   /* include/vesper/core/half.h:162-173 */
 float vsp_bf16_to_f32(uint16_t b);   /* include/vesper/core/half.h:175-181 */

@@ -278,6 +278,43 @@ static void run_rope_generation(KVFormat fmt, DType qdt, double tol, const char*
     CHECK(c2.current_seq_len() == 0);
 }
 
+static void run_token_with_output_projection(KVFormat fmt, DType dt, double tol, const char* name) {
+    // GroupedQueryAttention::forward(x, cache, start_pos) for one generated token, through wo_ (src/nn/gqa_attention.cpp:124-152):
+    // the fused call equals the step-by-step route (attention output, heads merged, Linear::forward by the oracle)
+    std::printf("test_token_with_output_projection[%s]\n", name);
+    const int64_t B = 3, Hq = 8, Hkv = 2, D = 64, T0 = 9, S_max = 32, C = Hq * D;
+    nn::GroupedQueryAttentionCore attn(C, Hq, Hkv);
+    nn::RopeTable rope(S_max, D);
+    auto round = [&](std::vector<float> x) { return dt == DType::BFloat16 ? bf16_round(std::move(x)) : x; };
+    auto q0 = round(randn(B * Hq * T0 * D, 61, 0.5f)), k0 = round(randn(B * Hkv * T0 * D, 62, 0.5f)), v0 = round(randn(B * Hkv * T0 * D, 63, 0.5f));
+    auto q1 = round(randn(B * Hq * D, 64, 0.5f)), k1 = round(randn(B * Hkv * D, 65, 0.5f)), v1 = round(randn(B * Hkv * D, 66, 0.5f));
+    auto w = round(randn(C * C, 67, 1.0f / std::sqrt((float)C))), bias = round(randn(C, 68, 0.5f));
+    Tensor tw = to_dev(w, {C, C}, dt), tb = to_dev(bias, {C}, dt);
+    nn::KVCache ca(B, Hkv, S_max, D, Device::HIP, fmt), cb(B, Hkv, S_max, D, Device::HIP, fmt);
+    for (nn::KVCache* c : {&ca, &cb})
+        attn.forward_rope(to_dev(q0, {B, Hq, T0, D}, dt), to_dev(k0, {B, Hkv, T0, D}, dt), to_dev(v0, {B, Hkv, T0, D}, dt), c, 0, rope, dt);
+    Tensor o = attn.forward_rope(to_dev(q1, {B, Hq, 1, D}, dt), to_dev(k1, {B, Hkv, 1, D}, dt), to_dev(v1, {B, Hkv, 1, D}, dt), &ca, T0, rope, dt);
+    auto x = to_host(o);  // [B,Hq,1,D] == [B,1,C] once the heads are merged (T == 1)
+    for (int with_bias = 0; with_bias < 2; ++with_bias) {
+        nn::KVCache cc(B, Hkv, S_max, D, Device::HIP, fmt);
+        attn.forward_rope(to_dev(q0, {B, Hq, T0, D}, dt), to_dev(k0, {B, Hkv, T0, D}, dt), to_dev(v0, {B, Hkv, T0, D}, dt), &cc, 0, rope, dt);
+        Tensor y = attn.forward_token_proj(to_dev(q1, {B, Hq, 1, D}, dt), to_dev(k1, {B, Hkv, 1, D}, dt), to_dev(v1, {B, Hkv, 1, D}, dt), &cc, T0,
+                                           rope, dt, tw, with_bias ? &tb : nullptr);
+        CHECK(y.ndim() == 3 && y.shape()[0] == B && y.shape()[1] == 1 && y.shape()[2] == C);
+        CHECK((int64_t)cc.current_seq_len() == T0 + 1);
+        std::vector<float> want((size_t)(B * C));
+        orc_linear_f32(x.data(), w.data(), with_bias ? bias.data() : nullptr, want.data(), B, C, C);
+        double err = max_abs_diff(to_host(y), want.data(), want.size());
+        if (!(err < tol)) std::printf("  bias %d: max-abs %.3g\n", with_bias, err);
+        CHECK(err < tol);
+    }
+    // a weight whose inner size is not Hq * D is refused with the shape error
+    Tensor bad = to_dev(std::vector<float>((size_t)(C * (C - 8))), {C, C - 8}, dt);
+    CHECK(thrown<std::runtime_error>([&] {
+              attn.forward_token_proj(to_dev(q1, {B, Hq, 1, D}, dt), to_dev(k1, {B, Hkv, 1, D}, dt), to_dev(v1, {B, Hkv, 1, D}, dt), &cb, T0, rope, dt, bad);
+          }) != "<nothing thrown>");
+}
+
 static void test_sdpa_routing() {
     std::printf("test_sdpa_routing\n");
     const int64_t B = 1, H = 2, D = 64;
@@ -489,6 +526,8 @@ int main(int argc, char** argv) {
         test_sdpa_routing();
         test_backward_dispatch_seam();
         test_multi_head_attention_core();
+        run_token_with_output_projection(KVFormat::Float32, DType::Float32, 1e-4, "f32");
+        run_token_with_output_projection(KVFormat::BFloat16, DType::BFloat16, 1e-2, "bf16");
         test_token_loop_allocates_nothing_and_keeps_pace();
     }
     std::printf(g_fail ? "FAILED: %d check(s)\n" : "all adapter tests passed\n", g_fail);

@@ -209,6 +209,36 @@ static void test_validation() {
     CHECK(vsp_attn_decode(&dq3, &c, nullptr, 0, &dq3, 0.1f, mem, 1 << 16, nullptr) == VSP_ERR_GQA_HEADS);
     CHECK(vsp_attn_decode_workspace_bytes(2, 8, 128, 1000) == (size_t)2 * 8 * 4 * 130 * 4);
     CHECK(vsp_attn_decode_workspace_bytes(0, 8, 128, 1000) == 0);
+    // decode + output projection: weight [N, Hq*D], bias [N], y [B,1,N], workspace = merged heads + the partials
+    {
+        vsp_tensor w{}, bias{}, y{};
+        w.data = mem, w.dtype = VSP_BF16, w.ndim = 2, w.shape[0] = 32, w.shape[1] = 256, w.stride[0] = 256, w.stride[1] = 1;
+        bias.data = mem, bias.dtype = VSP_BF16, bias.ndim = 1, bias.shape[0] = 32, bias.stride[0] = 1;
+        y.data = mem, y.dtype = VSP_BF16, y.ndim = 3, y.shape[0] = 1, y.shape[1] = 1, y.shape[2] = 32;
+        y.stride[0] = 32, y.stride[1] = 32, y.stride[2] = 1;
+        CHECK(vsp_attn_decode_proj(&dq, &c, nullptr, 0, &w, &bias, &y, 0.1f, nullptr, 0, nullptr) == VSP_ERR_WORKSPACE);
+        CHECK(vsp_attn_decode_proj(&dq, &c, nullptr, 0, nullptr, &bias, &y, 0.1f, mem, 1 << 16, nullptr) == VSP_ERR_NULL);
+        vsp_tensor w2 = w;
+        w2.shape[1] = 128;
+        CHECK(vsp_attn_decode_proj(&dq, &c, nullptr, 0, &w2, &bias, &y, 0.1f, mem, 1 << 16, nullptr) == VSP_ERR_SHAPE);
+        w2 = w, w2.dtype = VSP_F32;
+        CHECK(vsp_attn_decode_proj(&dq, &c, nullptr, 0, &w2, &bias, &y, 0.1f, mem, 1 << 16, nullptr) == VSP_ERR_DTYPE);
+        w2 = w, w2.stride[0] = 260;
+        CHECK(vsp_attn_decode_proj(&dq, &c, nullptr, 0, &w2, &bias, &y, 0.1f, mem, 1 << 16, nullptr) == VSP_ERR_ALIGN);
+        vsp_tensor b2 = bias;
+        b2.shape[0] = 31;
+        CHECK(vsp_attn_decode_proj(&dq, &c, nullptr, 0, &w, &b2, &y, 0.1f, mem, 1 << 16, nullptr) == VSP_ERR_SHAPE);
+        vsp_tensor y2 = y;
+        y2.shape[1] = 2;
+        CHECK(vsp_attn_decode_proj(&dq, &c, nullptr, 0, &w, &bias, &y2, 0.1f, mem, 1 << 16, nullptr) == VSP_ERR_SHAPE);
+        // the attention step's own refusals come through: a length above the bound, a head count the cache does not divide
+        CHECK(vsp_attn_decode_proj(&dq, &c, nullptr, 32, &w, &bias, &y, 0.1f, mem, 1 << 16, nullptr) == VSP_ERR_ARG);
+        vsp_tensor w3 = w;
+        w3.shape[1] = 192, w3.stride[0] = 192;
+        CHECK(vsp_attn_decode_proj(&dq3, &c, nullptr, 0, &w3, &bias, &y, 0.1f, mem, 1 << 16, nullptr) == VSP_ERR_GQA_HEADS);
+        CHECK(vsp_attn_decode_proj_workspace_bytes(2, 8, 128, 1000) == (size_t)2 * 8 * 128 * 4 + (size_t)2 * 8 * 4 * 130 * 4);
+        CHECK(vsp_attn_decode_proj_workspace_bytes(0, 8, 128, 1000) == 0);
+    }
     // the entry point without a workspace refuses what its fixed array cannot hold, before anything else happens
     vsp_kv_cache big = c;
     big.B = 64, big.Hkv = 8, big.S_max = 65536, big.D = 128, big.len = 65536;

@@ -281,6 +281,26 @@ def decode_attention(q, cache, seq_lens=None, max_len=0, scale=None, out=None, w
     return out
 
 
+def decode_attention_proj(q, cache, wo, bias=None, seq_lens=None, max_len=0, scale=None, out=None, workspace=None):
+    """decode_attention followed by the module's output projection (src/nn/gqa_attention.cpp:151-152, Linear::forward
+    src/nn/linear.cpp:41-49) in one call: q [B,Hq,1,D], wo [N, Hq*D], bias [N] or None -> y [B,1,N]."""
+    c = cache._c
+    if scale is None:
+        scale = 1.0 / math.sqrt(q.shape[-1])
+    if out is None:
+        out = torch.empty((q.shape[0], 1, wo.shape[0]), dtype=q.dtype, device=q.device)
+    if workspace is None:
+        bound = max_len or (c.S_max if seq_lens is not None else c.len)
+        nbytes = lib.vsp_attn_decode_proj_workspace_bytes(q.shape[0], q.shape[1], q.shape[3], max(int(bound), 1))
+        workspace = _workspace(q.device, nbytes)
+    dq, dw, dy = _desc(q), _desc(wo), _desc(out)
+    db = _desc(bias) if bias is not None else None
+    sl = C.c_void_p(seq_lens.data_ptr()) if seq_lens is not None else None
+    check(lib.vsp_attn_decode_proj(C.byref(dq), C.byref(c), sl, int(max_len), C.byref(dw), C.byref(db) if db is not None else None,
+                                   C.byref(dy), float(scale), C.c_void_p(workspace.data_ptr()), workspace.numel(), _stream(q)))
+    return out
+
+
 def decode_attention_noalloc(q, cache, out, seq_lens=None, max_len=0, scale=None):
     """decode_attention through vsp_attn_decode_noalloc: the partials go to the library's fixed per-GPU array
     and the call allocates nothing (`out` is the caller's).  Calls overlapping on one GPU race."""

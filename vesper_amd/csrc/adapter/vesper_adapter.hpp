@@ -480,6 +480,27 @@ inline Tensor scaled_dot_product_attention(const Tensor& query, const Tensor& ke
     return ops::flash_attention(query, key, value, scale, is_causal && T > 1);
 }
 
+// T == 1 over a cache handle with the module's output projection behind it: what GroupedQueryAttention::forward
+// and MultiHeadAttention::forward do after SDPA -- transpose(1,2).reshape({B,T,C}) and wo_ / out_proj
+// (src/nn/gqa_attention.cpp:151-152, src/nn/transformer.cpp:207-215) -- in the same call.  wo: the Linear's weight
+// [N, C] (include/vesper/nn/linear.h), bias: its bias [N] or nullptr.  Returns [B, 1, N].
+inline Tensor decode_attention_proj(const Tensor& query, const Tensor& key, const Tensor& value, const Tensor& wo,
+                                    const Tensor* bias = nullptr) {
+    if (query.ndim() != 4) throw_status(VSP_ERR_NDIM);
+    if (!(key.cache && value.cache && !key.is_v && value.is_v)) throw std::runtime_error("decode_attention_proj: key/value must be cache handles");
+    if (wo.ndim() != 2) throw_status(VSP_ERR_NDIM);
+    const int64_t B = query.shape()[0], Hq = query.shape()[1], D = query.shape()[3];
+    const vsp_kv_cache& c = key.cache->c;
+    const float scale = 1.0f / std::sqrt(static_cast<float>(D));
+    Tensor y = empty({B, 1, wo.shape()[0]}, query.dtype());
+    const size_t ws_bytes = vsp_attn_decode_proj_workspace_bytes((int32_t)B, (int32_t)Hq, (int32_t)D, c.len > 0 ? c.len : 1);
+    Storage ws(ws_bytes);
+    vsp_tensor dq = query.desc(), dw = wo.desc(), dy = y.desc(), db;
+    if (bias) db = bias->desc();
+    throw_status(vsp_attn_decode_proj(&dq, &c, nullptr, 0, &dw, bias ? &db : nullptr, &dy, scale, ws.data(), ws_bytes, current_stream()));
+    return y;
+}
+
 }  // namespace functional
 
 // The attention core shared by GroupedQueryAttention::forward(x, cache, start_pos)
@@ -543,6 +564,17 @@ public:
         if (!cache) throw std::runtime_error("forward_chunk: a cache is required");
         cache->rope_update(q, k, v, (decltype(cache->current_seq_len()))start_pos, rope, q_dtype);
         return cache->attend(q, true);
+    }
+
+    // One generated token from step 3 to the module's end (src/nn/gqa_attention.cpp:124-152): RoPE + append, decode over
+    // the cache, heads merged, wo_ applied.  q [B,Hq,1,D], k/v [B,Hkv,1,D] not yet rotated; wo_weight [C, C].  -> [B,1,C]
+    template <typename CacheT>
+    Tensor forward_token_proj(Tensor q, const Tensor& k, const Tensor& v, CacheT* cache, int64_t start_pos, const RopeTable& rope,
+                              DType q_dtype, const Tensor& wo_weight, const Tensor* wo_bias = nullptr) const {
+        if (!cache) throw std::runtime_error("forward_token_proj: a cache is required");
+        if (q.ndim() != 4 || q.shape()[2] != 1) throw_status(VSP_ERR_SHAPE);
+        auto kv = cache->rope_update(q, k, v, (decltype(cache->current_seq_len()))start_pos, rope, q_dtype);
+        return functional::decode_attention_proj(q, kv.first, kv.second, wo_weight, wo_bias);
     }
 
 private:

@@ -629,6 +629,105 @@ __global__ void __launch_bounds__(256) decode_combine_kernel(const float* __rest
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Output projection behind the combine: y[m][n] = sum_k x[m][k] W[n][k] + bias[n]
+// (Linear::forward, src/nn/linear.cpp:41-49, as GroupedQueryAttention applies it to the merged heads,
+// src/nn/gqa_attention.cpp:151-152).  x is the decode output [B][Hq*D] left in the workspace, so M = B is tiny and
+// the kernel is a stream over W: a workgroup owns 16 output columns, its four wavefronts split K in 32-wide slices
+// (slice c goes to wavefront c % 4), W rows are the A operand of 16x16x32 MFMAs read straight from HBM in 16-byte
+// loads, x^T is the B operand (L2-resident), up to MT tiles of 16 batch rows share one pass over W.  The four
+// partial tiles are summed in a fixed order through LDS.
+// ---------------------------------------------------------------------------------------------
+template <int MT>
+__global__ void __launch_bounds__(256) proj_bf16_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
+                                                        int64_t w_pitch, const uint16_t* __restrict__ bias,
+                                                        uint16_t* __restrict__ y, int64_t y_pitch, int32_t M, int32_t N,
+                                                        int32_t K) {
+    __shared__ float part[kWaves][MT][16][17];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 15, g = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+    const int64_t wrow = min(n0 + r, N - 1);  // rows past N are computed from the last row and never stored
+    const uint16_t* pw = w + wrow * w_pitch + g * 8;
+    const int n_slices = K / 32;
+    for (int m0 = 0; m0 < M; m0 += 16 * MT) {
+        f32x4_t acc[MT];
+        const uint16_t* px[MT];
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            px[t] = x + (int64_t)min(m0 + 16 * t + r, M - 1) * K + g * 8;
+        }
+        int c = wave;
+        for (; c + 3 * kWaves < n_slices; c += 4 * kWaves) {  // four slices of W in flight per wavefront
+            bf16x8_t a[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) a[u] = *(const bf16x8_t*)(pw + (int64_t)(c + u * kWaves) * 32);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+                    const bf16x8_t b = *(const bf16x8_t*)(px[t] + (int64_t)(c + u * kWaves) * 32);
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b, acc[t], 0, 0, 0);
+                }
+            }
+        }
+        for (; c < n_slices; c += kWaves) {
+            const bf16x8_t a = *(const bf16x8_t*)(pw + (int64_t)c * 32);
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                const bf16x8_t b = *(const bf16x8_t*)(px[t] + (int64_t)c * 32);
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[t], 0, 0, 0);
+            }
+        }
+        // the tile a lane holds: column (batch row) r, rows (output columns) 4 g + i
+        __syncthreads();  // the previous pass's readers are done with `part`
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) part[wave][t][r][4 * g + i] = acc[t][i];
+        __syncthreads();
+        for (int e = threadIdx.x; e < MT * 256; e += 256) {
+            const int t = e >> 8, m = (e >> 4) & 15, n = e & 15;
+            const int gm = m0 + 16 * t + m, gn = n0 + n;
+            if (gm < M && gn < N) {
+                float sum = part[0][t][m][n];
+                sum += part[1][t][m][n];
+                sum += part[2][t][m][n];
+                sum += part[3][t][m][n];
+                if (bias) sum += bf16_bits_to_f32(bias[gn]);
+                y[(int64_t)gm * y_pitch + gn] = f32_to_bf16_bits(sum);
+            }
+        }
+    }
+}
+
+// fp32 operands (the reference's own dtype): one wavefront per output column, lanes stride over k, eight batch rows
+// per pass over the row of W.
+__global__ void __launch_bounds__(256) proj_f32_kernel(const float* __restrict__ x, const float* __restrict__ w, int64_t w_pitch,
+                                                       const float* __restrict__ bias, float* __restrict__ y, int64_t y_pitch,
+                                                       int32_t M, int32_t N, int32_t K) {
+    const int lane = threadIdx.x & 63;
+    const int n = blockIdx.x * kWaves + (threadIdx.x >> 6);
+    if (n >= N) return;
+    const float* pw = w + (int64_t)n * w_pitch;
+    for (int m0 = 0; m0 < M; m0 += 8) {
+        float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        for (int k = lane; k < K; k += 64) {
+            const float wk = pw[k];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[j] = fmaf(x[(int64_t)min(m0 + j, M - 1) * K + k], wk, acc[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            float v = acc[j];
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+            if (lane == 0 && m0 + j < M) y[(int64_t)(m0 + j) * y_pitch + n] = bias ? v + bias[n] : v;
+        }
+    }
+}
+
 int device_cu_count() {
     static int cus = 0;
     if (cus == 0) {
@@ -805,6 +904,10 @@ int decode_impl(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* s
     return check_launch();
 }
 
+// Where vsp_attn_decode_proj keeps the merged heads x [B][Hq*D] inside its workspace: in front of the split-K
+// partials, 4 bytes an element whatever the dtype, rounded up to 256 bytes.
+size_t proj_x_bytes(int64_t B, int64_t Hq, int64_t D) { return (size_t)((B * Hq * D * 4 + 255) / 256 * 256); }
+
 }  // namespace
 
 extern "C" {
@@ -823,6 +926,67 @@ int vsp_attn_decode(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_
 int vsp_attn_decode_noalloc(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, int32_t max_len,
                             vsp_tensor* out, float scale, void* stream) {
     return decode_impl(q, cache, seq_lens, max_len, out, scale, nullptr, 0, true, stream);
+}
+
+size_t vsp_attn_decode_proj_workspace_bytes(int32_t B, int32_t Hq, int32_t D, int32_t max_len) {
+    if (B <= 0 || Hq <= 0 || D <= 0) return 0;
+    return proj_x_bytes(B, Hq, D) + vsp_attn_decode_workspace_bytes(B, Hq, D, max_len);
+}
+
+int vsp_attn_decode_proj(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, int32_t max_len,
+                         const vsp_tensor* wo, const vsp_tensor* bias, vsp_tensor* y, float scale, void* workspace,
+                         size_t workspace_bytes, void* stream) {
+    if (!q || !wo || !y) return VSP_ERR_NULL;
+    if (q->ndim != 4) return VSP_ERR_NDIM;
+    if (wo->ndim != 2 || y->ndim != 3 || (bias && bias->ndim != 1)) return VSP_ERR_NDIM;
+    const int64_t B = q->shape[0], Hq = q->shape[1], D = q->shape[3];
+    const int64_t K = Hq * D, N = wo->shape[0];
+    if (wo->shape[1] != K || y->shape[0] != B || y->shape[1] != 1 || y->shape[2] != N) return VSP_ERR_SHAPE;
+    if (bias && bias->shape[0] != N) return VSP_ERR_SHAPE;
+    if (wo->dtype != q->dtype || y->dtype != q->dtype || (bias && bias->dtype != q->dtype)) return VSP_ERR_DTYPE;
+    if (wo->stride[1] != 1 || y->stride[2] != 1 || (bias && bias->stride[0] != 1)) return VSP_ERR_STRIDE;
+    const int esz = q->dtype == VSP_F32 ? 4 : 2;
+    if (N > 0 && B > 0) {
+        if (!wo->data || !y->data || (bias && !bias->data)) return VSP_ERR_NULL;
+        if (!is_aligned16(wo->data) || (wo->stride[0] * esz) % 16) return VSP_ERR_ALIGN;
+    }
+    if (B <= 0 || Hq <= 0 || D <= 0 || B > INT32_MAX || N > INT32_MAX || K > INT32_MAX) {
+        // shapes the attention step rejects are reported by it; an empty batch has nothing to project
+        vsp_tensor none = *q;
+        return decode_impl(q, cache, seq_lens, max_len, &none, scale, workspace, workspace_bytes, false, stream);
+    }
+    // the attention step writes the merged heads x [B][Hq][D] (= [B][K]) to the head of the workspace
+    const size_t xb = proj_x_bytes(B, Hq, D);
+    if (!workspace || workspace_bytes < xb) return VSP_ERR_WORKSPACE;
+    if (!is_aligned16(workspace)) return VSP_ERR_ALIGN;
+    vsp_tensor x = *q;
+    x.data = workspace;
+    x.stride[0] = K;
+    x.stride[1] = D;
+    x.stride[2] = D;
+    x.stride[3] = 1;
+    int rc = decode_impl(q, cache, seq_lens, max_len, &x, scale, (char*)workspace + xb, workspace_bytes - xb, false, stream);
+    if (rc != VSP_OK || N == 0) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    if (q->dtype == VSP_F32) {
+        hipLaunchKernelGGL(proj_f32_kernel, dim3((unsigned)ceil_div(N, kWaves)), dim3(256), 0, st, (const float*)x.data,
+                           (const float*)wo->data, wo->stride[0], bias ? (const float*)bias->data : nullptr,
+                           (float*)y->data, y->stride[0], (int)B, (int)N, (int)K);
+    } else {
+        // K = Hq * D with D 64 or 128 (the bf16 attention kernels' head sizes): a whole number of 32-wide slices
+        const dim3 grid((unsigned)ceil_div(N, 16));
+        const uint16_t* pb = bias ? (const uint16_t*)bias->data : nullptr;
+        if (B <= 16)
+            hipLaunchKernelGGL(proj_bf16_kernel<1>, grid, dim3(256), 0, st, (const uint16_t*)x.data, (const uint16_t*)wo->data,
+                               wo->stride[0], pb, (uint16_t*)y->data, y->stride[0], (int)B, (int)N, (int)K);
+        else if (B <= 32)
+            hipLaunchKernelGGL(proj_bf16_kernel<2>, grid, dim3(256), 0, st, (const uint16_t*)x.data, (const uint16_t*)wo->data,
+                               wo->stride[0], pb, (uint16_t*)y->data, y->stride[0], (int)B, (int)N, (int)K);
+        else
+            hipLaunchKernelGGL(proj_bf16_kernel<4>, grid, dim3(256), 0, st, (const uint16_t*)x.data, (const uint16_t*)wo->data,
+                               wo->stride[0], pb, (uint16_t*)y->data, y->stride[0], (int)B, (int)N, (int)K);
+    }
+    return check_launch();
 }
 
 }  // extern "C"
