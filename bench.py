@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on ONE MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|p4k|c3|c4|c5|c4p|c2c|c3c|r2|b2|b3] [--no-cpu] [--no-extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|p4k|c3|c4|c5|c4p|c4w|c2c|c3c|r2|b2|b3] [--no-cpu] [--no-extra]
 
 A "step" is one pass of the hot path over one batch of synthetic input that is already resident in
 HBM: one prefill launch (c2, p4k, c3) or one decode call = split-K kernel + combine kernel (c4, c5).
@@ -38,6 +38,9 @@ WORKLOADS = {
                name="BASELINE config 5: decode over Q8_0 KV cache, B16, 64 q / 8 kv heads, D128, L=65536"),
     "c4p": dict(kind="decode", fmt="bf16", B=32, Hq=32, Hkv=8, D=128, S=32768, lens=(1024, 32768, 4004), page=256,
                 name="config 4 over a paged cache: pages of 256 tokens in a shuffled page table, otherwise as config 4"),
+    "c4w": dict(kind="decode", fmt="bf16", B=32, Hq=32, Hkv=8, D=128, S=32768, lens=(1024, 32768, 4004), proj=True,
+                name="config 4 through the module's output projection: decode as config 4, heads merged, y = x Wo^T with "
+                     "Wo [4096, 4096] bf16 in the same call (algorithmic bytes: KV + Wo)"),
     "c2c": dict(kind="prefill_cached", fmt="bf16", B=4, Hq=32, Hkv=8, D=128, N=2048,
                 name="config 2 through the cache: causal GQA prefill bf16 reading K/V from the bf16 cache planes, "
                      "B4, 32 q / 8 kv heads, D128, N2048"),
@@ -94,7 +97,7 @@ class Runner:
             self.cache.update(mk(Hkv), mk(Hkv), 0, return_views=False)
             self.work = prefill_flops(w)
             self.unit, self.peak, self.bound = "TFLOP/s", MFMA_BF16_PEAK_TFLOPS, "mfma"
-            self.kernel = "prefill_bf16_kernel<128, true>"
+            self.kernel = "prefill_bf16_pipe_kernel<true>"
         elif w["kind"] == "backward":
             B, Hq, Hkv, D, N = w["B"], w["Hq"], w["Hkv"], w["D"], w["N"]
             mk = lambda h: (torch.randn(B, h, N, D, device=dev, generator=g) * 0.5).to(torch.bfloat16)
@@ -115,7 +118,7 @@ class Runner:
             self.out = torch.empty(B, Hq, N, D, device=dev, dtype=torch.bfloat16)
             self.work = rope_bytes(w)
             self.unit, self.peak, self.bound = "GB/s", HBM_PEAK_GBS, "hbm"
-            self.kernel = "append_bf16_kernel<unsigned short, true>"
+            self.kernel = "append_bf16_tile_kernel<unsigned short, true, 128>"
         else:
             import numpy as np
             B, Hq, Hkv, D, S = w["B"], w["Hq"], w["Hkv"], w["D"], w["S"]
@@ -149,6 +152,11 @@ class Runner:
             self.out = torch.empty_like(self.q)
             self.scale = 1.0 / math.sqrt(D)
             self.work = decode_bytes(w, lens)
+            if w.get("proj"):
+                C_ = Hq * D
+                self.wo = (torch.randn(C_, C_, device=dev, generator=g) * (1.0 / math.sqrt(C_))).to(torch.bfloat16)
+                self.y = torch.empty(B, 1, C_, device=dev, dtype=torch.bfloat16)
+                self.work += C_ * C_ * 2
             self.unit, self.peak, self.bound = "GB/s", HBM_PEAK_GBS, "hbm"
             self.kernel = ("decode_bf16_kernel<128, %s>" if w["fmt"] == "bf16" else "decode_q8_kernel<128, %s>") % ("true" if w.get("page") else "false")
             self.max_len = int(lens.max())
@@ -180,6 +188,9 @@ class Runner:
             return self.cache.prefill(self.q)
         if self.w["kind"] == "rope":
             return self.cache.rope_update(self.q, self.k, self.v, 0, self.rope, out=self.out)
+        if self.w.get("proj"):
+            return self.va.decode_attention_proj(self.q, self.cache, self.wo, None, seq_lens=self.seq_lens, max_len=self.max_len,
+                                                 scale=self.scale, out=self.y)
         return self.va.decode_attention(self.q, self.cache, seq_lens=self.seq_lens, max_len=self.max_len,
                                         scale=self.scale, out=self.out)
 
@@ -390,7 +401,7 @@ def main():
 
     if not args.no_extra:
         others = {}
-        for key in ("c2", "p4k", "c3", "c4", "c5", "c4p", "c2c", "c3c", "r2", "b2", "b3"):
+        for key in ("c2", "p4k", "c3", "c4", "c5", "c4p", "c4w", "c2c", "c3c", "r2", "b2", "b3"):
             if key == args.workload:
                 continue
             r = Runner(key, torch, va)

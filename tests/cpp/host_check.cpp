@@ -236,8 +236,9 @@ static void test_validation() {
         vsp_tensor w3 = w;
         w3.shape[1] = 192, w3.stride[0] = 192;
         CHECK(vsp_attn_decode_proj(&dq3, &c, nullptr, 0, &w3, &bias, &y, 0.1f, mem, 1 << 16, nullptr) == VSP_ERR_GQA_HEADS);
-        CHECK(vsp_attn_decode_proj_workspace_bytes(2, 8, 128, 1000) == (size_t)2 * 8 * 128 * 4 + (size_t)2 * 8 * 4 * 130 * 4);
-        CHECK(vsp_attn_decode_proj_workspace_bytes(0, 8, 128, 1000) == 0);
+        CHECK(vsp_attn_decode_proj_workspace_bytes(2, 8, 128, 1000, 512) ==
+              (size_t)2 * 8 * 128 * 4 + (size_t)8 * 2 * 512 * 4 + (size_t)2 * 8 * 4 * 130 * 4);
+        CHECK(vsp_attn_decode_proj_workspace_bytes(0, 8, 128, 1000, 512) == 0);
     }
     // the entry point without a workspace refuses what its fixed array cannot hold, before anything else happens
     vsp_kv_cache big = c;

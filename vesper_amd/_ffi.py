@@ -53,7 +53,7 @@ SYMBOLS = {
     "vsp_attn_decode_workspace_bytes": (C.c_size_t, [C.c_int32] * 4),
     "vsp_attn_decode": (C.c_int, [_TP, _KP, C.c_void_p, C.c_int32, _TP, C.c_float, C.c_void_p, C.c_size_t, C.c_void_p]),
     "vsp_attn_decode_noalloc": (C.c_int, [_TP, _KP, C.c_void_p, C.c_int32, _TP, C.c_float, C.c_void_p]),
-    "vsp_attn_decode_proj_workspace_bytes": (C.c_size_t, [C.c_int32] * 4),
+    "vsp_attn_decode_proj_workspace_bytes": (C.c_size_t, [C.c_int32] * 5),
     "vsp_attn_decode_proj": (C.c_int, [_TP, _KP, C.c_void_p, C.c_int32, _TP, _TP, _TP, C.c_float, C.c_void_p, C.c_size_t,
                                        C.c_void_p]),
     "vsp_f32_to_bf16": (C.c_uint16, [C.c_float]),

@@ -291,7 +291,7 @@ def decode_attention_proj(q, cache, wo, bias=None, seq_lens=None, max_len=0, sca
         out = torch.empty((q.shape[0], 1, wo.shape[0]), dtype=q.dtype, device=q.device)
     if workspace is None:
         bound = max_len or (c.S_max if seq_lens is not None else c.len)
-        nbytes = lib.vsp_attn_decode_proj_workspace_bytes(q.shape[0], q.shape[1], q.shape[3], max(int(bound), 1))
+        nbytes = lib.vsp_attn_decode_proj_workspace_bytes(q.shape[0], q.shape[1], q.shape[3], max(int(bound), 1), wo.shape[0])
         workspace = _workspace(q.device, nbytes)
     dq, dw, dy = _desc(q), _desc(wo), _desc(out)
     db = _desc(bias) if bias is not None else None

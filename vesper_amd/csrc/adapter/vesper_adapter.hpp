@@ -493,7 +493,7 @@ inline Tensor decode_attention_proj(const Tensor& query, const Tensor& key, cons
     const vsp_kv_cache& c = key.cache->c;
     const float scale = 1.0f / std::sqrt(static_cast<float>(D));
     Tensor y = empty({B, 1, wo.shape()[0]}, query.dtype());
-    const size_t ws_bytes = vsp_attn_decode_proj_workspace_bytes((int32_t)B, (int32_t)Hq, (int32_t)D, c.len > 0 ? c.len : 1);
+    const size_t ws_bytes = vsp_attn_decode_proj_workspace_bytes((int32_t)B, (int32_t)Hq, (int32_t)D, c.len > 0 ? c.len : 1, (int32_t)wo.shape()[0]);
     Storage ws(ws_bytes);
     vsp_tensor dq = query.desc(), dw = wo.desc(), dy = y.desc(), db;
     if (bias) db = bias->desc();

@@ -632,73 +632,118 @@ __global__ void __launch_bounds__(256) decode_combine_kernel(const float* __rest
 // ---------------------------------------------------------------------------------------------
 // Output projection behind the combine: y[m][n] = sum_k x[m][k] W[n][k] + bias[n]
 // (Linear::forward, src/nn/linear.cpp:41-49, as GroupedQueryAttention applies it to the merged heads,
-// src/nn/gqa_attention.cpp:151-152).  x is the decode output [B][Hq*D] left in the workspace, so M = B is tiny and
-// the kernel is a stream over W: a workgroup owns 16 output columns, its four wavefronts split K in 32-wide slices
-// (slice c goes to wavefront c % 4), W rows are the A operand of 16x16x32 MFMAs read straight from HBM in 16-byte
-// loads, x^T is the B operand (L2-resident), up to MT tiles of 16 batch rows share one pass over W.  The four
-// partial tiles are summed in a fixed order through LDS.
+// src/nn/gqa_attention.cpp:151-152).  x is the decode output [B][Hq*D] left in the workspace, so M = B is small and
+// the job is one pass over W at HBM rate.  Workgroup (nb, ks) owns 128 output columns (16 per wavefront) and the
+// ks-th of KS equal ranges of K.  Per 512-wide piece of its range every lane first issues its sixteen 16-byte loads
+// of W rows (the A operands of 16x16x32 MFMAs, straight from HBM into registers), then the workgroup stages the
+// matching piece of x in LDS once for its eight wavefronts (x^T is the B operand; up to MT tiles of 16 batch rows share
+// the pass over W).  The fp32 partial tiles go to P[ks][m][n] (through LDS, so that P is written in whole rows);
+// proj_reduce_kernel adds the KS partials in index order, the bias, and rounds.  The reduction is a second launch on
+// purpose: folding it into the last workgroup to arrive needs device-scope fences, which on this multi-die part write
+// back and invalidate the L2 slices and cost several times the whole projection.
 // ---------------------------------------------------------------------------------------------
+constexpr int kProjWaves = 8;     // wavefronts per workgroup, 16 output columns each
+constexpr int kProjCols = 16 * kProjWaves;
+constexpr int kProjThreads = 64 * kProjWaves;
+constexpr int kProjPiece = 512;   // k values staged in LDS at a time
+constexpr int kProjPitch = kProjPiece + 8;  // LDS row pitch (elements): 16 rows of one 16-byte read fall in 64 distinct banks
+constexpr int kProjMaxSplit = 8;
+
 template <int MT>
-__global__ void __launch_bounds__(256) proj_bf16_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
-                                                        int64_t w_pitch, const uint16_t* __restrict__ bias,
-                                                        uint16_t* __restrict__ y, int64_t y_pitch, int32_t M, int32_t N,
-                                                        int32_t K) {
-    __shared__ float part[kWaves][MT][16][17];
+__global__ void __launch_bounds__(kProjThreads) proj_bf16_partial_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
+                                                                int64_t w_pitch, float* __restrict__ part, int32_t m0, int32_t M,
+                                                                int32_t N, int32_t K, int32_t Kc) {
+    __shared__ __attribute__((aligned(16))) uint16_t sx[16 * MT * kProjPitch];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 15, g = lane >> 4;
-    const int n0 = blockIdx.x * 16;
+    const int n0 = blockIdx.x * kProjCols + 16 * wave;
+    const int ks = blockIdx.y;
     const int64_t wrow = min(n0 + r, N - 1);  // rows past N are computed from the last row and never stored
     const uint16_t* pw = w + wrow * w_pitch + g * 8;
-    const int n_slices = K / 32;
-    for (int m0 = 0; m0 < M; m0 += 16 * MT) {
-        f32x4_t acc[MT];
-        const uint16_t* px[MT];
+    const int rows = min(M - m0, 16 * MT);
+    f32x4_t acc[MT];
 #pragma unroll
-        for (int t = 0; t < MT; ++t) {
-            acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-            px[t] = x + (int64_t)min(m0 + 16 * t + r, M - 1) * K + g * 8;
+    for (int t = 0; t < MT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    constexpr int kItems = 16 * MT * (kProjPiece / 8) / kProjThreads;  // 16-byte items of x a thread stages per piece
+    for (int k0 = ks * Kc; k0 < (ks + 1) * Kc; k0 += kProjPiece) {
+        const int piece = min(kProjPiece, (ks + 1) * Kc - k0);  // a multiple of 32
+        const int n_slices = piece / 32;
+        // x first, W behind it: loads return in order, so x can go to LDS while the W slices are still in flight and
+        // the MFMAs start as the slices arrive
+        u32x4_t xs[kItems];
+#pragma unroll
+        for (int i = 0; i < kItems; ++i) {
+            const int e = threadIdx.x + i * kProjThreads, row = e / (kProjPiece / 8), c = e % (kProjPiece / 8);
+            if (row < rows && 8 * c < piece) xs[i] = *(const u32x4_t*)(x + (int64_t)(m0 + row) * K + k0 + 8 * c);
         }
-        int c = wave;
-        for (; c + 3 * kWaves < n_slices; c += 4 * kWaves) {  // four slices of W in flight per wavefront
-            bf16x8_t a[4];
+        bf16x8_t a[16];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) a[u] = *(const bf16x8_t*)(pw + (int64_t)(c + u * kWaves) * 32);
+        for (int u = 0; u < 16; ++u)
+            if (u < n_slices) a[u] = *(const bf16x8_t*)(pw + k0 + 32 * u);
+        __builtin_amdgcn_s_barrier();  // the previous piece's readers are done with sx (their LDS reads fed MFMAs already issued)
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+        for (int i = 0; i < kItems; ++i) {
+            const int e = threadIdx.x + i * kProjThreads, row = e / (kProjPiece / 8), c = e % (kProjPiece / 8);
+            if (row < rows && 8 * c < piece) *(u32x4_t*)(sx + row * kProjPitch + 8 * c) = xs[i];
+        }
+        // LDS writes landed, then the barrier: a fence here would also wait for the W loads
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            if (u < n_slices) {
 #pragma unroll
                 for (int t = 0; t < MT; ++t) {
-                    const bf16x8_t b = *(const bf16x8_t*)(px[t] + (int64_t)(c + u * kWaves) * 32);
-                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b, acc[t], 0, 0, 0);
+                    // rows past `rows` hold whatever LDS held: they only reach output columns that are never stored
+                    const bf16x8_t bx = *(const bf16x8_t*)(sx + (16 * t + r) * kProjPitch + 32 * u + 8 * g);
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], bx, acc[t], 0, 0, 0);
                 }
             }
         }
-        for (; c < n_slices; c += kWaves) {
-            const bf16x8_t a = *(const bf16x8_t*)(pw + (int64_t)c * 32);
+    }
+    // The partial tile goes through LDS so that P is written in whole rows.  A lane holds batch row r of tile t, output
+    // columns 16 wave + 4 g + i of the workgroup's 128.
+    constexpr int kTilePitch = kProjCols + 4;  // floats; 16 rows of one 16-byte write fall in 64 distinct banks
+    float* tile = (float*)sx;
+    __builtin_amdgcn_s_barrier();  // every wavefront's reads of sx have returned (they fed its MFMAs)
 #pragma unroll
-            for (int t = 0; t < MT; ++t) {
-                const bf16x8_t b = *(const bf16x8_t*)(px[t] + (int64_t)c * 32);
-                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[t], 0, 0, 0);
-            }
-        }
-        // the tile a lane holds: column (batch row) r, rows (output columns) 4 g + i
-        __syncthreads();  // the previous pass's readers are done with `part`
+    for (int t = 0; t < MT; ++t) *(f32x4_t*)(tile + (16 * t + r) * kTilePitch + 16 * wave + 4 * g) = acc[t];
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    const int nb0 = blockIdx.x * kProjCols;
+    const bool vec = (N & 3) == 0;  // then a group of four columns is inside the row and 16-byte aligned in P
+    for (int e = threadIdx.x; e < rows * (kProjCols / 4); e += kProjThreads) {
+        const int m = e / (kProjCols / 4), c = (e % (kProjCols / 4)) * 4, n = nb0 + c;
+        const f32x4_t v = *(const f32x4_t*)(tile + m * kTilePitch + c);
+        float* dst = part + ((int64_t)ks * M + m0 + m) * N + n;
+        if (vec && n < N) *(f32x4_t*)dst = v;
+        else
+            for (int i = 0; i < 4; ++i)
+                if (n + i < N) dst[i] = v[i];
+    }
+}
+
+// y[m][n] = round(sum_ks P[ks][m][n] + bias[n]), the partials added in index order.  VEC consecutive outputs per thread
+// (4 when N is a multiple of 4, so that a group never straddles two rows).
+template <int VEC>
+__global__ void __launch_bounds__(256) proj_reduce_kernel(const float* __restrict__ part, const uint16_t* __restrict__ bias,
+                                                          uint16_t* __restrict__ y, int64_t y_pitch, int32_t M, int32_t N, int32_t KS) {
+    typedef float vec_t __attribute__((ext_vector_type(VEC)));
+    const int64_t e = ((int64_t)blockIdx.x * 256 + threadIdx.x) * VEC;
+    const int64_t plane = (int64_t)M * N;
+    if (e >= plane) return;
+    const int m = (int)(e / N), n = (int)(e - (int64_t)m * N);
+    vec_t v[kProjMaxSplit];
 #pragma unroll
-        for (int t = 0; t < MT; ++t)
+    for (int s = 0; s < kProjMaxSplit; ++s) v[s] = *(const vec_t*)(part + min(s, KS - 1) * plane + e);  // all loads in flight at once
+    vec_t sum = v[0];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) part[wave][t][r][4 * g + i] = acc[t][i];
-        __syncthreads();
-        for (int e = threadIdx.x; e < MT * 256; e += 256) {
-            const int t = e >> 8, m = (e >> 4) & 15, n = e & 15;
-            const int gm = m0 + 16 * t + m, gn = n0 + n;
-            if (gm < M && gn < N) {
-                float sum = part[0][t][m][n];
-                sum += part[1][t][m][n];
-                sum += part[2][t][m][n];
-                sum += part[3][t][m][n];
-                if (bias) sum += bf16_bits_to_f32(bias[gn]);
-                y[(int64_t)gm * y_pitch + gn] = f32_to_bf16_bits(sum);
-            }
-        }
+    for (int s = 1; s < kProjMaxSplit; ++s) sum += s < KS ? v[s] : vec_t(0.f);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+        float f = sum[j];
+        if (bias) f += bf16_bits_to_f32(bias[n + j]);
+        y[(int64_t)m * y_pitch + n + j] = f32_to_bf16_bits(f);
     }
 }
 
@@ -904,9 +949,18 @@ int decode_impl(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* s
     return check_launch();
 }
 
-// Where vsp_attn_decode_proj keeps the merged heads x [B][Hq*D] inside its workspace: in front of the split-K
-// partials, 4 bytes an element whatever the dtype, rounded up to 256 bytes.
+// vsp_attn_decode_proj's workspace: the merged heads x [B][Hq*D] (4 bytes an element whatever the dtype), the
+// projection's split-K partials [kProjMaxSplit][B][N] fp32, then the attention step's own partials; each part
+// rounded up to 256 bytes.
 size_t proj_x_bytes(int64_t B, int64_t Hq, int64_t D) { return (size_t)((B * Hq * D * 4 + 255) / 256 * 256); }
+size_t proj_part_bytes(int64_t B, int64_t N) { return (size_t)((kProjMaxSplit * B * N * 4 + 255) / 256 * 256); }
+
+// Equal ranges of K per workgroup row: as many as kProjMaxSplit while each stays a whole number of 32-wide slices.
+int proj_split(int64_t K) {
+    int ks = kProjMaxSplit;
+    while (ks > 1 && K % (32 * ks) != 0) ks >>= 1;
+    return ks;
+}
 
 }  // namespace
 
@@ -928,9 +982,9 @@ int vsp_attn_decode_noalloc(const vsp_tensor* q, const vsp_kv_cache* cache, cons
     return decode_impl(q, cache, seq_lens, max_len, out, scale, nullptr, 0, true, stream);
 }
 
-size_t vsp_attn_decode_proj_workspace_bytes(int32_t B, int32_t Hq, int32_t D, int32_t max_len) {
-    if (B <= 0 || Hq <= 0 || D <= 0) return 0;
-    return proj_x_bytes(B, Hq, D) + vsp_attn_decode_workspace_bytes(B, Hq, D, max_len);
+size_t vsp_attn_decode_proj_workspace_bytes(int32_t B, int32_t Hq, int32_t D, int32_t max_len, int32_t N) {
+    if (B <= 0 || Hq <= 0 || D <= 0 || N < 0) return 0;
+    return proj_x_bytes(B, Hq, D) + proj_part_bytes(B, N) + vsp_attn_decode_workspace_bytes(B, Hq, D, max_len);
 }
 
 int vsp_attn_decode_proj(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, int32_t max_len,
@@ -956,7 +1010,8 @@ int vsp_attn_decode_proj(const vsp_tensor* q, const vsp_kv_cache* cache, const i
         return decode_impl(q, cache, seq_lens, max_len, &none, scale, workspace, workspace_bytes, false, stream);
     }
     // the attention step writes the merged heads x [B][Hq][D] (= [B][K]) to the head of the workspace
-    const size_t xb = proj_x_bytes(B, Hq, D);
+    const size_t pb_bytes = proj_part_bytes(B, N);
+    const size_t xb = proj_x_bytes(B, Hq, D) + pb_bytes;
     if (!workspace || workspace_bytes < xb) return VSP_ERR_WORKSPACE;
     if (!is_aligned16(workspace)) return VSP_ERR_ALIGN;
     vsp_tensor x = *q;
@@ -974,17 +1029,32 @@ int vsp_attn_decode_proj(const vsp_tensor* q, const vsp_kv_cache* cache, const i
                            (float*)y->data, y->stride[0], (int)B, (int)N, (int)K);
     } else {
         // K = Hq * D with D 64 or 128 (the bf16 attention kernels' head sizes): a whole number of 32-wide slices
-        const dim3 grid((unsigned)ceil_div(N, 16));
-        const uint16_t* pb = bias ? (const uint16_t*)bias->data : nullptr;
-        if (B <= 16)
-            hipLaunchKernelGGL(proj_bf16_kernel<1>, grid, dim3(256), 0, st, (const uint16_t*)x.data, (const uint16_t*)wo->data,
-                               wo->stride[0], pb, (uint16_t*)y->data, y->stride[0], (int)B, (int)N, (int)K);
-        else if (B <= 32)
-            hipLaunchKernelGGL(proj_bf16_kernel<2>, grid, dim3(256), 0, st, (const uint16_t*)x.data, (const uint16_t*)wo->data,
-                               wo->stride[0], pb, (uint16_t*)y->data, y->stride[0], (int)B, (int)N, (int)K);
+        const int KS = proj_split(K);
+        float* part = (float*)((char*)workspace + proj_x_bytes(B, Hq, D));
+        const dim3 grid((unsigned)ceil_div(N, kProjCols), (unsigned)KS);
+        const uint16_t* px = (const uint16_t*)x.data;
+        const uint16_t* pw = (const uint16_t*)wo->data;
+        for (int64_t m0 = 0; m0 < B; m0 += 64) {  // 64 batch rows share a pass over W
+            const int64_t rows = B - m0;
+            if (rows <= 16)
+                hipLaunchKernelGGL(proj_bf16_partial_kernel<1>, grid, dim3(kProjThreads), 0, st, px, pw, wo->stride[0], part, (int)m0, (int)B,
+                                   (int)N, (int)K, (int)(K / KS));
+            else if (rows <= 32)
+                hipLaunchKernelGGL(proj_bf16_partial_kernel<2>, grid, dim3(kProjThreads), 0, st, px, pw, wo->stride[0], part, (int)m0, (int)B,
+                                   (int)N, (int)K, (int)(K / KS));
+            else
+                hipLaunchKernelGGL(proj_bf16_partial_kernel<4>, grid, dim3(kProjThreads), 0, st, px, pw, wo->stride[0], part, (int)m0, (int)B,
+                                   (int)N, (int)K, (int)(K / KS));
+        }
+        rc = check_launch();
+        if (rc != VSP_OK) return rc;
+        const uint16_t* pbias = bias ? (const uint16_t*)bias->data : nullptr;
+        if (N % 4 == 0)
+            hipLaunchKernelGGL(proj_reduce_kernel<4>, dim3((unsigned)ceil_div(B * N, 1024)), dim3(256), 0, st, part, pbias,
+                               (uint16_t*)y->data, y->stride[0], (int)B, (int)N, KS);
         else
-            hipLaunchKernelGGL(proj_bf16_kernel<4>, grid, dim3(256), 0, st, (const uint16_t*)x.data, (const uint16_t*)wo->data,
-                               wo->stride[0], pb, (uint16_t*)y->data, y->stride[0], (int)B, (int)N, (int)K);
+            hipLaunchKernelGGL(proj_reduce_kernel<1>, dim3((unsigned)ceil_div(B * N, 256)), dim3(256), 0, st, part, pbias,
+                               (uint16_t*)y->data, y->stride[0], (int)B, (int)N, KS);
     }
     return check_launch();
 }
