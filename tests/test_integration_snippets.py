@@ -17,6 +17,8 @@ BLOCKS = [
     ("KVCache::update / reset", "member", ""),
     ("decode inside scaled_dot_product_attention", "function",
      f"{_T} query, vesper::Tensor output, vsp_kv_cache* cache_desc, vsp_tensor dq, vsp_tensor dout, int32_t B, int32_t Hq, int32_t D, void* stream"),
+    ("decode through wo_", "function",
+     f"{_T} wo_weight, vesper::Tensor y, vsp_kv_cache* cache_desc, vsp_tensor dq, int64_t T, int32_t B, int32_t Hq, int32_t D, void* stream"),
     ("RoPE + cache write", "function",
      f"int32_t max_seq_len, int32_t head_dim_, float rope_base_, const float*& rope_table_, const float* (*upload)(const std::vector<float>&), "
      f"{_T} q_view, {_T} k_view, {_T} v_view, {_T} q_rot, vsp_kv_cache cache_desc, int64_t start_pos, void* stream"),
