@@ -292,7 +292,10 @@ def cpu_baseline(key):
 # cannot be collected inside a timed run, so these are properties of the workload shapes, not live values.
 PROFILE_OF = {
     "c2": ("prefill_bf16_config2.txt", "prefill_bf16", 96 * 2**20 + 65 * 2**20),
+    "p4k": ("prefill_bf16_4k.txt", "prefill_bf16", 96 * 2**20 + 65 * 2**20),
     "c3": ("prefill_bf16_config3.txt", "prefill_bf16", 96 * 2**20 + 65 * 2**20),
+    "c2c": ("prefill_bf16_cache_planes_config2.txt", "prefill_bf16_pipe_kernel<true>", 96 * 2**20 + 65 * 2**20),
+    "r2": ("rope_append_bf16_config2.txt", "append_bf16_tile_kernel<unsigned short, true", 202375168),
     "c4": ("decode_bf16_config4.txt", "decode_bf16_kernel", 2614935552),
     "c5": ("decode_q8_0_config5.txt", "decode_q8_kernel", 2282225664),
 }
