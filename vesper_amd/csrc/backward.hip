@@ -5,15 +5,16 @@
 // (src/ops/flash_attention.cpp:366-482): with P = exp(scale q.k - lse) recomputed from the forward's
 // log-sum-exp,  Di = rowsum(dO * O),  dV = P^T dO,  dP = dO V^T,  dS = P * (dP - Di),
 // dQ = scale dS K,  dK = scale dS^T Q.  Differences from the reference's HIP kernel: matrix cores
-// (fp32 MFMA 32x32x2) instead of scalar FMAs, any D in {64, 128}, grouped-query heads folded in
+// instead of scalar FMAs, D in {64, 128} (and 32 for fp32 operands), grouped-query heads folded in
 // (dK / dV of a kv head sum over its query heads, the gradient of ops::repeat_kv), and no atomics:
 // dQ is produced by one pass that owns query rows, dK / dV by a second pass that owns key rows, so the
 // result is bitwise reproducible (the reference accumulates dQ with atomicAdd).
 //
 // fp32 operands: fp32 MFMA (32x32x2) throughout.  bf16 operands: bf16 MFMA (32x32x16) with fp32 accumulation
 // and fp32 softmax algebra; P and dS are rounded to bf16 (round-to-nearest-even) between the products, as P is
-// in the forward kernel, and the gradients are rounded to bf16 on store.  This is the training-side companion of
-// the inference path: plain LDS tiles filled by ordinary loads, no direct-to-LDS pipeline.
+// in the forward kernel, and the gradients are rounded to bf16 on store.  The fp32 kernels use plain padded LDS
+// tiles filled by ordinary loads; the bf16 kernels use dense XOR-swizzled tiles filled by direct-to-LDS loads
+// through a ring of slots (see the comments at bwd_dq_bf16_kernel and bwd_dkdv_bf16_kernel).
 #include <math.h>
 
 #include <type_traits>

@@ -6,21 +6,25 @@
 // (src/ops/flash_attention.cpp:218-364): online softmax over key tiles, O = acc / l,
 // LSE = m + log l; the arithmetic is bf16 MFMA with fp32 accumulation (or fp32 MFMA for fp32 inputs).
 //
-// bf16 kernel.  A workgroup of 4 wavefronts owns 128 consecutive queries of one (batch, query head);
+// Two bf16 kernels share the tiles and the fragment layouts described here; prefill_bf16_pipe_kernel (D = 128,
+// further down) reorders the work of a wavefront into a three-stage software pipeline and is the one the
+// benchmark shapes run, prefill_bf16_kernel serves D = 64 and dense inputs with per-row lengths.
+//
+// A workgroup of 4 wavefronts owns 128 consecutive queries of one (batch, query head);
 // each wavefront owns 32 of them.  Key tiles of 32 go from global memory straight into LDS (buffer
-// loads with the LDS modifier, two ring slots, the next tile in flight while the current one is
+// loads with the LDS modifier, a ring of slots, later tiles in flight while the current one is
 // consumed, one barrier per tile).  LDS rows are unpadded; 16-byte chunks are XOR-swizzled so that
 // both the ds_read_b128 of K and the transposing reads of V are bank-conflict free.  The vector ALU,
-// not the matrix pipe, is what this kernel runs out of first (VALU and MFMA issue from one SIMD
-// overlap only partly), so the loop is written to keep VALU instructions per MFMA minimal: addresses
-// live in scalar registers, the row sum is a packed dot product, the mask and the rescale are rare
+// not the matrix pipe, is what these kernels run out of first (vector-ALU work of one wavefront hardly
+// overlaps with MFMAs of another wavefront on the same SIMD), so the loops are written to keep VALU
+// instructions per MFMA minimal: addresses live in scalar registers, the mask and the rescale are rare
 // branches.  Both GEMMs are computed transposed so that the softmax statistics of a query live in one
 // lane (and its partner 32 lanes away):
 //   S^T[key][q] = K[key][:] . Q^T[:][q]     32x32x16 MFMA, A = K rows from LDS, B = Q^T held in registers
 //   O^T[d][q]  += V^T[d][key] . P^T[key][q]  A = V^T read from the row-major V tile with the
 //                                            transposing LDS read, B = P^T straight from the S^T registers
 // The exponent uses a per-row reference maximum that is only raised (and the accumulators rescaled)
-// when the true running maximum outgrows it by more than 2^8; the result is mathematically the same
+// when the row has outgrown it by a wide margin; the result is mathematically the same
 // softmax, without a rescale per tile.  Key tiles entirely above the causal diagonal are skipped;
 // the mask is evaluated only on tiles that straddle it.
 #include <math.h>
@@ -466,7 +470,7 @@ constexpr int kLead = 6;  // LDS operand reads run this many MFMA slots ahead
 // MFMA slot order of a step: Q = a QK^T MFMA (k-step index), P = a PV MFMA (index p: key half p / 4, d block p % 4).
 // The QK chain finishes at slot 10, so that the row maximum of the new scores is taken under the last PV MFMAs.
 constexpr int kSlotIsQ[16] = {1, 1, 0, 1, 1, 0, 1, 1, 0, 1, 1, 0, 0, 0, 0, 0};
-constexpr int kSlotIdx[16] = {0, 1, 0, 2, 3, 1, 4, 5, 2, 6, 7, 3, 4, 5, 6, 7};
+[[maybe_unused]] constexpr int kSlotIdx[16] = {0, 1, 0, 2, 3, 1, 4, 5, 2, 6, 7, 3, 4, 5, 6, 7};
 // LDS read instructions per operand: one ds_read_b128 for K rows and for V^T taken from a token-blocked plane, two
 // transposing reads for V^T taken from row-major V
 template <bool VBLK>
