@@ -106,7 +106,7 @@ class Runner:
             self.o, self.lse = va.flash_attention(self.q, self.k, self.v, self.scale, True, return_lse=True)
             self.work = 2.5 * prefill_flops(w)
             self.unit, self.peak, self.bound = "TFLOP/s", MFMA_BF16_PEAK_TFLOPS, "mfma"
-            self.kernel = "bwd_delta + bwd_dq_bf16_kernel<128> + bwd_dkdv_bf16_kernel<128> (the three launches of one step)"
+            self.kernel = "bwd_dq_bf16_kernel<128> + bwd_dkdv_bf16_kernel<128> (the two launches of one step)"
         elif w["kind"] == "rope":
             B, Hq, Hkv, D, N = w["B"], w["Hq"], w["Hkv"], w["D"], w["N"]
             fused = (torch.randn(B, N, (Hq + 2 * Hkv) * D, device=dev, generator=g) * 0.5).to(torch.bfloat16)

@@ -347,34 +347,6 @@ __device__ inline uint32_t cvt_pk_bf16(float a, float b) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
-// Di = rowsum(dO * O) and lse * log2(e) (the softmax is recomputed with exp2); D / 8 lanes share a row, 16 bytes each.
-template <int D>
-__global__ void __launch_bounds__(256) bwd_delta_bf16_kernel(BwdArgs a) {
-    constexpr int LPR = D / 8, RPB = 256 / LPR;
-    const int sub = threadIdx.x % LPR;
-    const int64_t rows = (int64_t)a.B * a.Hq * a.N;
-    const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / LPR;
-    const int64_t rr = row < rows ? row : rows - 1;   // every lane takes part in the shuffles
-    const int i = (int)(rr % a.N);
-    const int64_t bh = rr / a.N;
-    const int h = (int)(bh % a.Hq), b = (int)(bh / a.Hq);
-    const uint4 wo = *(const uint4*)((const uint16_t*)a.out + (int64_t)b * a.s_o[0] + (int64_t)h * a.s_o[1] + (int64_t)i * a.s_o[2] + 8 * sub);
-    const uint4 wd = *(const uint4*)((const uint16_t*)a.dout + (int64_t)b * a.s_do[0] + (int64_t)h * a.s_do[1] + (int64_t)i * a.s_do[2] + 8 * sub);
-    const uint32_t o4[4] = {wo.x, wo.y, wo.z, wo.w}, d4[4] = {wd.x, wd.y, wd.z, wd.w};
-    float s = 0.f;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        s += __uint_as_float(o4[j] << 16) * __uint_as_float(d4[j] << 16);
-        s += __uint_as_float(o4[j] & 0xffff0000u) * __uint_as_float(d4[j] & 0xffff0000u);
-    }
-#pragma unroll
-    for (int o = LPR / 2; o > 0; o >>= 1) s += __shfl_xor(s, o);
-    if (sub == 0 && row < rows) {
-        a.delta[row] = s;
-        a.lse2[row] = kLog2e * a.lse[(int64_t)b * a.s_l[0] + (int64_t)h * a.s_l[1] + (int64_t)i * a.s_l[2]];
-    }
-}
-
 // ---- dQ (bf16): the structure of bwd_dq_kernel; K serves both as rows (S^T) and transposed (dQ^T) ----
 template <int D>
 __global__ void __launch_bounds__(256, 2) bwd_dq_bf16_kernel(BwdArgs a) {
@@ -404,8 +376,30 @@ __global__ void __launch_bounds__(256, 2) bwd_dq_bf16_kernel(BwdArgs a) {
         qf[ks] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(Qp + 16 * ks + 8 * h));
         dof[ks] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(Op + 16 * ks + 8 * h));
     }
-    const float lse_q = a.lse2[((int64_t)b * a.Hq + hq) * a.N + qrow];
-    const float di_q = a.delta[((int64_t)b * a.Hq + hq) * a.N + qrow];
+    // Di = rowsum(dO * O) of this lane's query: each lane holds half of the row of dO (the operand above) and reads the
+    // same half of O; the two halves meet across lane ^ 32.  Every query row belongs to exactly one wavefront of this
+    // launch, which also leaves Di and lse * log2(e) in the workspace for the dK/dV pass that follows.
+    float di_q = 0.f;
+    {
+        const uint16_t* Orow = (const uint16_t*)a.out + (int64_t)b * a.s_o[0] + (int64_t)hq * a.s_o[1] + (int64_t)qrow * a.s_o[2];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const uint4 wo = *(const uint4*)(Orow + 16 * ks + 8 * h);
+            const uint4 wd = __builtin_bit_cast(uint4, dof[ks]);
+            const uint32_t o4[4] = {wo.x, wo.y, wo.z, wo.w}, d4[4] = {wd.x, wd.y, wd.z, wd.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                di_q += __uint_as_float(o4[j] << 16) * __uint_as_float(d4[j] << 16);
+                di_q += __uint_as_float(o4[j] & 0xffff0000u) * __uint_as_float(d4[j] & 0xffff0000u);
+            }
+        }
+        di_q += __shfl_xor(di_q, 32);
+    }
+    const float lse_q = kLog2e * a.lse[(int64_t)b * a.s_l[0] + (int64_t)hq * a.s_l[1] + (int64_t)qrow * a.s_l[2]];
+    if (h == 0 && qi < a.N) {
+        a.delta[((int64_t)b * a.Hq + hq) * a.N + qi] = di_q;
+        a.lse2[((int64_t)b * a.Hq + hq) * a.N + qi] = lse_q;
+    }
     const float scale_log2 = a.scale * kLog2e;
 
     const int wg_qmax = min(qt * kBQ + kBQ - 1, a.N - 1);
@@ -695,8 +689,6 @@ template __global__ void bwd_dkdv_bf16_kernel<128>(BwdArgs);
 template __global__ void bwd_dkdv_bf16_kernel<64>(BwdArgs);
 template __global__ void bwd_dq_bf16_kernel<128>(BwdArgs);
 template __global__ void bwd_dq_bf16_kernel<64>(BwdArgs);
-template __global__ void bwd_delta_bf16_kernel<128>(BwdArgs);
-template __global__ void bwd_delta_bf16_kernel<64>(BwdArgs);
 
 int check4(const vsp_tensor* t, int64_t B, int64_t H, int64_t N, int64_t D, int dtype) {
     if (!t) return VSP_ERR_NULL;
@@ -711,14 +703,11 @@ int check4(const vsp_tensor* t, int64_t B, int64_t H, int64_t N, int64_t D, int 
 template <typename T>
 int launch_backward(const BwdArgs& a, int64_t D, hipStream_t st) {
     const int64_t rows = (int64_t)a.B * a.Hq * a.N;
-    if constexpr (sizeof(T) == 2) {
-        if (D == 128) hipLaunchKernelGGL(bwd_delta_bf16_kernel<128>, dim3((unsigned)ceil_div(rows, 16)), dim3(256), 0, st, a);
-        else hipLaunchKernelGGL(bwd_delta_bf16_kernel<64>, dim3((unsigned)ceil_div(rows, 32)), dim3(256), 0, st, a);
-    } else {
+    if constexpr (sizeof(T) != 2) {  // the bf16 dQ pass computes Di itself, in its prologue
         hipLaunchKernelGGL(bwd_delta_kernel<T>, dim3((unsigned)ceil_div(rows, 4)), dim3(256), 0, st, a, (int)D);
+        int rc = check_launch();
+        if (rc != VSP_OK) return rc;
     }
-    int rc = check_launch();
-    if (rc != VSP_OK) return rc;
     const int64_t tiles = ceil_div(a.N, kBQ);
     const dim3 gq((unsigned)(tiles * a.B * a.Hq)), gk((unsigned)(tiles * a.B * a.Hkv));
     if constexpr (sizeof(T) == 2) {
