@@ -124,3 +124,29 @@ def test_argument_errors(va):
     wide = torch.zeros(N, Hq * D + 4, dtype=torch.bfloat16, device=G.dev())
     assert code(wo=wide[:, :Hq * D]) == _ffi.ERR_ALIGN                # row pitch not a multiple of 16 bytes
     assert code(workspace=torch.zeros(256, dtype=torch.uint8, device=G.dev())) == _ffi.ERR_WORKSPACE
+
+
+def test_config4_shape_against_an_independent_gemm_and_linearity(va):
+    # config 4's heads and width (32 / 8 heads, D 128, C 4096, B 32) over a shorter context: the projection of the very
+    # activations vsp_attn_decode produced, against torch's fp32 matmul, and linearity in the weight
+    B, Hq, Hkv, S, D = 32, 32, 8, 1024, 128
+    C_ = Hq * D
+    g = torch.Generator(device="cuda").manual_seed(71)
+    dev = G.dev()
+    cache = va.KVCache(B, Hkv, S, D, fmt="bf16")
+    cache.update(torch.randn(B, Hkv, S, D, device=dev, generator=g).to(torch.bfloat16),
+                 torch.randn(B, Hkv, S, D, device=dev, generator=g).to(torch.bfloat16), 0, return_views=False)
+    lens = torch.randint(1, S + 1, (B,), device=dev, generator=g, dtype=torch.int32)
+    q = torch.randn(B, Hq, 1, D, device=dev, generator=g).to(torch.bfloat16)
+    w1 = (torch.randn(C_, C_, device=dev, generator=g) / 64).to(torch.bfloat16)
+    w2 = (torch.randn(C_, C_, device=dev, generator=g) / 64).to(torch.bfloat16)
+    x = va.decode_attention(q, cache, seq_lens=lens).transpose(1, 2).reshape(B, 1, C_).float()
+    y1 = va.decode_attention_proj(q, cache, w1, seq_lens=lens).float()
+    y2 = va.decode_attention_proj(q, cache, w2, seq_lens=lens).float()
+    ref1 = x @ w1.float().t()
+    err = (y1 - ref1).abs()
+    assert float(err.max()) <= 2.0**-8 * float(ref1.abs().max()) + 1e-3, float(err.max())
+    # w1 + w2 is not a bf16 tensor in general, so compare in fp32: y(w1) + y(w2) against x (w1 + w2)^T
+    ref12 = x @ (w1.float() + w2.float()).t()
+    assert float((y1 + y2 - ref12).abs().max()) <= 2.0**-7 * float(ref12.abs().max()) + 2e-3
+    assert torch.equal(va.decode_attention_proj(q, cache, w1, seq_lens=lens).float(), y1)  # bitwise run to run
