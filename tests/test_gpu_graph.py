@@ -97,3 +97,33 @@ def test_forward_backward_replays_bit_identically(va):
         torch.cuda.synchronize()
         for got, want in zip([o] + list(grads), eager[i]):
             assert torch.equal(got, want), f"replay {i}"
+
+
+def test_decode_through_the_output_projection_replays_bit_identically(va):
+    # the four launches of vsp_attn_decode_proj (split-K decode, combine, projection partials, reduce) in one graph;
+    # the workspace, which also carries the merged heads between the launches, belongs to the caller
+    B, Hq, Hkv, D, S = 3, 8, 2, 128, 300
+    C_ = Hq * D
+    dev = G.dev()
+    c = va.KVCache(B, Hkv, S, D, fmt="bf16")
+    c.update(G.to_bf16_dev(I.normal(21, (B, Hkv, S, D))), G.to_bf16_dev(I.normal(22, (B, Hkv, S, D))), 0, return_views=False)
+    lens = torch.tensor([300, 17, 128], dtype=torch.int32, device=dev)
+    wo = G.to_bf16_dev(I.normal(23, (C_, C_), scale=1.0 / 32))
+    bias = G.to_bf16_dev(I.normal(24, (C_,), scale=0.5))
+    qs = [G.to_bf16_dev(I.normal(30 + i, (B, Hq, 1, D))) for i in range(3)]
+    eager = [va.decode_attention_proj(q, c, wo, bias, seq_lens=lens).clone() for q in qs]
+    torch.cuda.synchronize()
+    sq = torch.empty_like(qs[0])
+    y = torch.empty(B, 1, C_, dtype=torch.bfloat16, device=dev)
+    ws = torch.empty(va._ffi.lib.vsp_attn_decode_proj_workspace_bytes(B, Hq, D, S, C_), dtype=torch.uint8, device=dev)
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            va.decode_attention_proj(sq, c, wo, bias, seq_lens=lens, max_len=S, out=y, workspace=ws)
+    torch.cuda.synchronize()
+    for i, q in enumerate(qs):
+        sq.copy_(q)          # eager work between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, eager[i]), f"replay {i}"
