@@ -282,8 +282,9 @@ int vsp_attn_decode_noalloc(const vsp_tensor* q, const vsp_kv_cache* cache, cons
  * bias: [N] or NULL; y: [B, 1, N]; all of q's dtype (bf16 over VSP_KV_BF16 / VSP_KV_Q8_0 caches, fp32 over
  * VSP_KV_F32).  The merged heads never become a caller tensor: the combine kernel leaves them, rounded to q's dtype
  * exactly as vsp_attn_decode's `out` would hold them, at the head of `workspace`, and a projection kernel streams
- * W over them once (bf16: 16x16x32 MFMA with fp32 accumulation, K split over up to eight workgroups whose partial
- * tiles a second kernel adds in index order before the bias and the rounding; bitwise run-to-run deterministic).
+ * W over them once (bf16: 16x16x32 MFMA with fp32 accumulation; up to 16 batch rows in one launch, K split over the
+ * eight wavefronts of a workgroup; more rows with K split over up to eight workgroups whose partial tiles a second
+ * kernel adds in index order before the bias and the rounding; bitwise run-to-run deterministic either way).
  * workspace >= vsp_attn_decode_proj_workspace_bytes(B, Hq, D, max_len, N), 16-byte aligned. */
 size_t vsp_attn_decode_proj_workspace_bytes(int32_t B, int32_t Hq, int32_t D, int32_t max_len, int32_t N);
 int vsp_attn_decode_proj(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, int32_t max_len,

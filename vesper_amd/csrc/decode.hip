@@ -723,6 +723,49 @@ __global__ void __launch_bounds__(kProjThreads) proj_bf16_partial_kernel(const u
     }
 }
 
+// Up to 16 batch rows: one launch.  A workgroup owns 16 output columns; its eight wavefronts take the 32-wide slices of K
+// round-robin (slice c goes to wavefront c % 8), x^T comes straight from L2 (16 rows at most: no staging pays), and the
+// eight partial tiles meet in LDS, where they are added in wavefront order.  No partial buffer, no second launch.
+__global__ void __launch_bounds__(512) proj_bf16_small_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
+                                                              int64_t w_pitch, const uint16_t* __restrict__ bias,
+                                                              uint16_t* __restrict__ y, int64_t y_pitch, int32_t M, int32_t N,
+                                                              int32_t K) {
+    __shared__ float part[8][16][17];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 15, g = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+    const uint16_t* pw = w + (int64_t)min(n0 + r, N - 1) * w_pitch + g * 8;  // rows past N: computed, never stored
+    const uint16_t* px = x + (int64_t)min(r, M - 1) * K + g * 8;             // likewise for batch rows past M
+    const int n_slices = K / 32;
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    for (int c0 = wave; c0 < n_slices; c0 += 8 * 16) {  // sixteen slices of W (and of x) in flight per lane
+        bf16x8_t a[16], b[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u)
+            if (c0 + 8 * u < n_slices) a[u] = *(const bf16x8_t*)(pw + (int64_t)(c0 + 8 * u) * 32);
+#pragma unroll
+        for (int u = 0; u < 16; ++u)
+            if (c0 + 8 * u < n_slices) b[u] = *(const bf16x8_t*)(px + (int64_t)(c0 + 8 * u) * 32);
+#pragma unroll
+        for (int u = 0; u < 16; ++u)
+            if (c0 + 8 * u < n_slices) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[u], acc, 0, 0, 0);
+    }
+    // the tile a lane holds: batch row r, output columns 4 g + i
+#pragma unroll
+    for (int i = 0; i < 4; ++i) part[wave][r][4 * g + i] = acc[i];
+    __syncthreads();
+    if (threadIdx.x < 256) {
+        const int m = threadIdx.x >> 4, n = threadIdx.x & 15;
+        if (m < M && n0 + n < N) {
+            float sum = part[0][m][n];
+#pragma unroll
+            for (int wv = 1; wv < 8; ++wv) sum += part[wv][m][n];
+            if (bias) sum += bf16_bits_to_f32(bias[n0 + n]);
+            y[(int64_t)m * y_pitch + n0 + n] = f32_to_bf16_bits(sum);
+        }
+    }
+}
+
 // y[m][n] = round(sum_ks P[ks][m][n] + bias[n]), the partials added in index order.  VEC consecutive outputs per thread
 // (4 when N is a multiple of 4, so that a group never straddles two rows).
 template <int VEC>
@@ -1029,6 +1072,12 @@ int vsp_attn_decode_proj(const vsp_tensor* q, const vsp_kv_cache* cache, const i
                            (float*)y->data, y->stride[0], (int)B, (int)N, (int)K);
     } else {
         // K = Hq * D with D 64 or 128 (the bf16 attention kernels' head sizes): a whole number of 32-wide slices
+        if (B <= 16) {
+            hipLaunchKernelGGL(proj_bf16_small_kernel, dim3((unsigned)ceil_div(N, 16)), dim3(512), 0, st, (const uint16_t*)x.data,
+                               (const uint16_t*)wo->data, wo->stride[0], bias ? (const uint16_t*)bias->data : nullptr,
+                               (uint16_t*)y->data, y->stride[0], (int)B, (int)N, (int)K);
+            return check_launch();
+        }
         const int KS = proj_split(K);
         float* part = (float*)((char*)workspace + proj_x_bytes(B, Hq, D));
         const dim3 grid((unsigned)ceil_div(N, kProjCols), (unsigned)KS);
