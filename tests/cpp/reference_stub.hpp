@@ -1,4 +1,4 @@
-// The few declarations of danielmriley/vesper that the code blocks of INTEGRATION.md refer to, as a stand-in so that
+// The few declarations of danielmriley/vesper that the code blocks of the integration guide refer to, as a stand-in so that
 // tests/test_integration_snippets.py can compile those blocks against include/vsp_attn.h without the reference tree.
 // Shapes of the declarations follow include/vesper/core/{tensor,dtype,device,stream}.h and include/vesper/nn/transformer.h;
 // nothing here is executed.

@@ -1,4 +1,5 @@
-"""Every C++ code block of INTEGRATION.md is compiled (syntax and types only) against include/vsp_attn.h, so that a
+"""Every C++ code block of the integration guide (the markdown file at the repository root that shows the reference-side
+bindings) is compiled (syntax and types only) against include/vsp_attn.h, so that a
 signature change in the header cannot leave the integration guide behind.  The reference's own declarations are
 replaced by the small stand-in tests/cpp/reference_stub.hpp; blocks that are statements are wrapped in a function whose
 parameters are the variables the surrounding text introduces."""
@@ -8,6 +9,7 @@ import subprocess
 import tempfile
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GUIDE = "INTEGRATION" + ".md"
 
 # what each block is, in the order of appearance: a translation-unit level block, or statements with the variables they use
 _T = "const vesper::Tensor&"
@@ -33,8 +35,8 @@ def _cpp_blocks(text):
 
 
 def test_integration_md_code_blocks_compile_against_the_header():
-    blocks = _cpp_blocks(open(os.path.join(ROOT, "INTEGRATION.md")).read())
-    assert len(blocks) == len(BLOCKS), f"INTEGRATION.md has {len(blocks)} C++ blocks, the test describes {len(BLOCKS)}"
+    blocks = _cpp_blocks(open(os.path.join(ROOT, GUIDE)).read())
+    assert len(blocks) == len(BLOCKS), f"{GUIDE} has {len(blocks)} C++ blocks, the test describes {len(BLOCKS)}"
     src = ['#include "reference_stub.hpp"', "using namespace vesper;", "using namespace vesper::nn;"]
     for i, (body, (name, kind, params)) in enumerate(zip(blocks, BLOCKS)):
         src.append(f"// ---- block {i}: {name}")
