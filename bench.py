@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on ONE MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|p4k|c3|c4|c5|c4p|c4w|c2c|c3c|r2|b2|b3] [--no-cpu] [--no-extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|p4k|c3|c2f|c4|c5|c4p|c4w|c2c|c3c|r2|b2|b3] [--no-cpu] [--no-extra]
 
 A "step" is one pass of the hot path over one batch of synthetic input that is already resident in
 HBM: one prefill launch (c2, p4k, c3) or one decode call = split-K kernel + combine kernel (c4, c5).
@@ -32,6 +32,10 @@ WORKLOADS = {
                 name="4k-context point: causal GQA prefill bf16, B2, 32 q / 8 kv heads, D128, N4096"),
     "c3": dict(kind="prefill", B=1, Hq=32, Hkv=8, D=128, N=8192,
                name="BASELINE config 3: causal GQA prefill bf16, B1, 32 q / 8 kv heads, D128, N8192"),
+    "c2f": dict(kind="prefill_split", B=4, Hq=32, Hkv=8, D=128, N=2048,
+                name="config 2's shape with fp32 tensors through the bf16 matrix cores (operands as two bf16 terms, three MFMAs "
+                     "per product, within the fp32 bar of 1e-4): causal GQA prefill, B4, 32 q / 8 kv heads, D128, N2048; "
+                     "algorithmic FLOPs, against the bf16 MFMA peak"),
     "c4": dict(kind="decode", fmt="bf16", B=32, Hq=32, Hkv=8, D=128, S=32768, lens=(1024, 32768, 4004),
                name="BASELINE config 4: batched decode bf16 KV cache, B32, 32 q / 8 kv heads, D128, L~U[1024,32768]"),
     "c5": dict(kind="decode", fmt="q8_0", B=16, Hq=64, Hkv=8, D=128, S=65536, lens=None,
@@ -89,6 +93,15 @@ class Runner:
             self.work = prefill_flops(w)
             self.unit, self.peak, self.bound = "TFLOP/s", MFMA_BF16_PEAK_TFLOPS, "mfma"
             self.kernel = "prefill_bf16_pipe_kernel"
+        elif w["kind"] == "prefill_split":
+            B, Hq, Hkv, D, N = w["B"], w["Hq"], w["Hkv"], w["D"], w["N"]
+            mk = lambda h: torch.randn(B, h, N, D, device=dev, generator=g) * 0.5
+            self.q, self.k, self.v = mk(Hq), mk(Hkv), mk(Hkv)
+            self.scale = 1.0 / math.sqrt(D)
+            self.ws = torch.empty(va._ffi.lib.vsp_attn_prefill_split_workspace_bytes(B, Hq, Hkv, N, N, D), dtype=torch.uint8, device=dev)
+            self.work = prefill_flops(w)
+            self.unit, self.peak, self.bound = "TFLOP/s", MFMA_BF16_PEAK_TFLOPS, "mfma"
+            self.kernel = "split_f32_kernel + prefill_split_kernel<128>"
         elif w["kind"] == "prefill_cached":
             B, Hq, Hkv, D, N = w["B"], w["Hq"], w["Hkv"], w["D"], w["N"]
             mk = lambda h: (torch.randn(B, h, N, D, device=dev, generator=g) * 0.5).to(torch.bfloat16)
@@ -182,6 +195,8 @@ class Runner:
     def step(self):
         if self.w["kind"] == "prefill":
             return self.va.flash_attention(self.q, self.k, self.v, self.scale, True)
+        if self.w["kind"] == "prefill_split":
+            return self.va.flash_attention_split(self.q, self.k, self.v, self.scale, True, workspace=self.ws)
         if self.w["kind"] == "backward":
             return self.va.flash_attention_backward(self.dout, self.q, self.k, self.v, self.o, self.lse, self.scale, True)
         if self.w["kind"] == "prefill_cached":
@@ -383,7 +398,8 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": ("bf16" if primary.w.get("fmt", "bf16") == "bf16" else "q8_0 (int8 payload, fp16 MFMA)"),
+        "dtype": ("f32 operands as two bf16 terms (bf16 MFMA, fp32 accumulation)" if primary.w["kind"] == "prefill_split"
+                  else "bf16" if primary.w.get("fmt", "bf16") == "bf16" else "q8_0 (int8 payload, fp16 MFMA)"),
         "data": "synthetic",
         "config": {"workload": primary.w["name"], "key": args.workload,
                    "algorithmic_work_per_step": primary.work,
@@ -404,7 +420,7 @@ def main():
 
     if not args.no_extra:
         others = {}
-        for key in ("c2", "p4k", "c3", "c4", "c5", "c4p", "c4w", "c2c", "c3c", "r2", "b2", "b3"):
+        for key in ("c2", "p4k", "c3", "c2f", "c4", "c5", "c4p", "c4w", "c2c", "c3c", "r2", "b2", "b3"):
             if key == args.workload:
                 continue
             r = Runner(key, torch, va)

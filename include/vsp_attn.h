@@ -199,6 +199,18 @@ int vsp_kv_view_f32(const vsp_kv_cache* cache, vsp_tensor* k_view, vsp_tensor* v
 int vsp_attn_prefill(const vsp_tensor* q, const vsp_tensor* k, const vsp_tensor* v, vsp_tensor* out, vsp_tensor* lse,
                      float scale, int is_causal, float dropout_p, int training, void* stream);
 
+/* vsp_attn_prefill for fp32 tensors at matrix-core speed (the reference computes this op in fp32,
+ * src/ops/flash_attention.cpp:218-364, and its modules hold fp32 tensors).  Same arguments and semantics as
+ * vsp_attn_prefill with q, k, v, out fp32 and D in {64, 128} (else VSP_ERR_UNSUPPORTED), plus a workspace of
+ * vsp_attn_prefill_split_workspace_bytes() bytes (16-byte aligned; else VSP_ERR_WORKSPACE).  A pre-pass writes every
+ * operand as two bf16 planes x = hi + lo (hi = bf16(x), lo = bf16(x - hi): 16 significant bits) into the workspace; the
+ * attention kernel takes each product as hi hi + hi lo + lo hi on the bf16 MFMAs with fp32 accumulation, and splits P the
+ * same way after the fp32 exponential.  Results agree with the reference's fp32 arithmetic within its 1e-4 bar
+ * (observed below 2e-5 of the output's magnitude) at several times the rate of the fp32-MFMA kernel. */
+size_t vsp_attn_prefill_split_workspace_bytes(int32_t B, int32_t Hq, int32_t Hkv, int32_t T, int32_t L, int32_t D);
+int vsp_attn_prefill_split(const vsp_tensor* q, const vsp_tensor* k, const vsp_tensor* v, vsp_tensor* out, vsp_tensor* lse,
+                           float scale, int is_causal, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ops::flash_attention_backward (include/vesper/ops/flash_attention.h:61-66, src/ops/flash_attention.cpp:165-216)
  * = flash_attention_backward_hip_dispatch (header :80-92, src/ops/hip/flash_attention.hip:183-299), the
  * training-side companion of vsp_attn_prefill; mathematics of the CPU backward, src/ops/flash_attention.cpp:366-482,

@@ -137,6 +137,11 @@ static void test_flash_attention_against_oracle() {
         Tensor out = ops::flash_attention(to_dev(q, {B, H, N, D}, DType::Float32), to_dev(k, {B, H, N, D}, DType::Float32),
                                           to_dev(v, {B, H, N, D}, DType::Float32), scale, causal != 0);
         CHECK(max_abs_diff(to_host(out), want.data(), want.size()) < 1e-4);
+        // the same fp32 tensors through the bf16 matrix cores (two bf16 terms per operand): inside the same bar, with room
+        Tensor outs = ops::flash_attention_split(to_dev(q, {B, H, N, D}, DType::Float32), to_dev(k, {B, H, N, D}, DType::Float32),
+                                                 to_dev(v, {B, H, N, D}, DType::Float32), scale, causal != 0);
+        CHECK(max_abs_diff(to_host(outs), want.data(), want.size()) < 1e-4);
+        CHECK(max_abs_diff(to_host(outs), to_host(out).data(), want.size()) < 5e-5);
         auto qb = bf16_round(q), kb = bf16_round(k), vb = bf16_round(v);
         orc_flash_attention_f32(qb.data(), kb.data(), vb.data(), want.data(), lse.data(), B, H, N, D, scale, causal);
         Tensor outb = ops::flash_attention(to_dev(qb, {B, H, N, D}, DType::BFloat16), to_dev(kb, {B, H, N, D}, DType::BFloat16),

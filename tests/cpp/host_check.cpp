@@ -197,6 +197,18 @@ static void test_validation() {
     bad = c;
     bad.k = nullptr;
     CHECK(vsp_kv_cache_reset(&bad, nullptr) == VSP_ERR_NULL);
+    // fp32 prefill through split bf16 operands: fp32 only, head_dim 64 / 128, workspace for the K and V planes
+    {
+        vsp_tensor qf = tensor4(mem, VSP_F32, 1, 4, 8, 64), kf = tensor4(mem, VSP_F32, 1, 2, 8, 64), of = qf;
+        CHECK(vsp_attn_prefill_split(&qf, &kf, &kf, &of, nullptr, 0.1f, 1, nullptr, 0, nullptr) == VSP_ERR_WORKSPACE);
+        CHECK(vsp_attn_prefill_split(&qf, &kf, &kf, &of, nullptr, 0.1f, 1, mem, 64, nullptr) == VSP_ERR_WORKSPACE);
+        CHECK(vsp_attn_prefill_split(&q, &k, &k, &out, nullptr, 0.1f, 1, mem, 1 << 16, nullptr) == VSP_ERR_UNSUPPORTED);   // bf16 tensors
+        vsp_tensor q32 = tensor4(mem, VSP_F32, 1, 4, 8, 32), k32 = tensor4(mem, VSP_F32, 1, 2, 8, 32), o32 = q32;
+        CHECK(vsp_attn_prefill_split(&q32, &k32, &k32, &o32, nullptr, 0.1f, 1, mem, 1 << 16, nullptr) == VSP_ERR_UNSUPPORTED);
+        CHECK(vsp_attn_prefill_split(&qf, &kf, &kf, &of, nullptr, 0.0f, 1, mem, 1 << 16, nullptr) == VSP_ERR_ARG);
+        CHECK(vsp_attn_prefill_split_workspace_bytes(1, 4, 2, 8, 8, 64) == (size_t)4 * 2048);   // 2 * 8 * 64 elements * 2 bytes, four planes
+        CHECK(vsp_attn_prefill_split_workspace_bytes(1, 4, 2, 8, 0, 64) == 0);
+    }
     // decode: shapes, head ratio, bounds, workspace
     vsp_tensor dq = tensor4(mem, VSP_BF16, 1, 4, 1, 64), dout = dq;
     c.len = 40;

@@ -44,6 +44,8 @@ SYMBOLS = {
     "vsp_kv_read_q8_0": (C.c_int, [_KP, C.c_int32, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]),
     "vsp_kv_view_f32": (C.c_int, [_KP, _TP, _TP]),
     "vsp_attn_prefill": (C.c_int, [_TP, _TP, _TP, _TP, _TP, C.c_float, C.c_int, C.c_float, C.c_int, C.c_void_p]),
+    "vsp_attn_prefill_split_workspace_bytes": (C.c_size_t, [C.c_int32] * 6),
+    "vsp_attn_prefill_split": (C.c_int, [_TP] * 5 + [C.c_float, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]),
     "vsp_attn_backward_workspace_bytes": (C.c_size_t, [C.c_int32] * 3),
     "vsp_attn_prefill_backward": (C.c_int, [_TP] * 9 + [C.c_float, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]),
     "vsp_attn_prefill_cached_workspace_bytes": (C.c_size_t, [_KP, C.c_int]),

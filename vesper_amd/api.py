@@ -60,6 +60,23 @@ def flash_attention(q, k, v, scale, is_causal=True, dropout_p=0.0, training=Fals
     return (out, lse) if return_lse else out
 
 
+def flash_attention_split(q, k, v, scale, is_causal=True, return_lse=False, workspace=None):
+    """ops::flash_attention for fp32 tensors through the bf16 matrix cores (vsp_attn_prefill_split): every operand as two
+    bf16 terms, three MFMAs per product, fp32 accumulation; within the reference's 1e-4 of its fp32 result."""
+    out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    lse = torch.empty(q.shape[:3], dtype=torch.float32, device=q.device) if (return_lse and q.dim() == 4) else None
+    if workspace is None:
+        nws = lib.vsp_attn_prefill_split_workspace_bytes(q.shape[0], q.shape[1], k.shape[1], q.shape[2], k.shape[2], q.shape[3]) \
+            if q.dim() == 4 and k.dim() == 4 else 0
+        workspace = torch.empty(max(nws, 16), dtype=torch.uint8, device=q.device)
+    dq, dk, dv, do = _desc(q), _desc(k), _desc(v), _desc(out)
+    dl = _desc(lse) if lse is not None else None
+    check(lib.vsp_attn_prefill_split(C.byref(dq), C.byref(dk), C.byref(dv), C.byref(do),
+                                     C.byref(dl) if dl is not None else None, float(scale), int(bool(is_causal)),
+                                     C.c_void_p(workspace.data_ptr()), workspace.numel(), _stream(q)))
+    return (out, lse) if return_lse else out
+
+
 def flash_attention_backward(grad_output, q, k, v, output, lse, scale, is_causal=True):
     """ops::flash_attention_backward: (dq, dk, dv); k, v may have fewer heads than q (their gradients then sum over
     the query heads of each group)."""

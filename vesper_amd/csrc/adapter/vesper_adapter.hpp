@@ -421,6 +421,25 @@ inline Tensor flash_attention(const Tensor& q, const Tensor& k, const Tensor& v,
     return output;
 }
 
+// The same op for fp32 tensors at matrix-core speed: every operand taken as two bf16 terms, three MFMAs per product, fp32
+// accumulation (vsp_attn_prefill_split); within the reference's 1e-4 of its fp32 result, not bit-close to it.  A caller
+// switches a model over by calling this where it called flash_attention with fp32 tensors of head_dim 64 or 128.
+inline Tensor flash_attention_split(const Tensor& q, const Tensor& k, const Tensor& v, float scale, bool is_causal = true,
+                                    Tensor* lse_out = nullptr) {
+    if (q.ndim() != 4 || k.ndim() != 4 || v.ndim() != 4) throw_status(VSP_ERR_NDIM);
+    Tensor kk = nn::materialize(k, q.dtype()), vv = nn::materialize(v, q.dtype());
+    if (kk.shape()[1] * kk.head_rep != q.shape()[1] || vv.shape()[1] * vv.head_rep != q.shape()[1]) throw_status(VSP_ERR_SHAPE);
+    Tensor output = empty(q.shape(), q.dtype());
+    Tensor lse = empty({q.shape()[0], q.shape()[1], q.shape()[2]}, DType::Float32);
+    const size_t ws_bytes = vsp_attn_prefill_split_workspace_bytes((int32_t)q.shape()[0], (int32_t)q.shape()[1], (int32_t)kk.shape()[1],
+                                                                   (int32_t)q.shape()[2], (int32_t)kk.shape()[2], (int32_t)q.shape()[3]);
+    Storage ws(ws_bytes > 0 ? ws_bytes : 16);
+    vsp_tensor dq = q.desc(), dk = kk.desc(), dv = vv.desc(), dout = output.desc(), dl = lse.desc();
+    throw_status(vsp_attn_prefill_split(&dq, &dk, &dv, &dout, &dl, scale, is_causal ? 1 : 0, ws.data(), ws_bytes, current_stream()));
+    if (lse_out) *lse_out = lse;
+    return output;
+}
+
 // include/vesper/ops/flash_attention.h:80-92 (defined src/ops/hip/flash_attention.hip:183-299): the gradients are
 // caller-allocated.  A dropout mask can only come from a training forward with dropout_p > 0, which this path
 // rejects, so a non-null mask with dropout_p > 0 is VSP_ERR_UNSUPPORTED here too.

@@ -55,6 +55,10 @@ struct PrefillArgs {
     const int32_t* page_table;  // cache-plane mode, paged cache: [B][pages_per_seq] page indices (device) or nullptr
     int32_t page_tokens, pages_per_seq;
     float scale_log2;  // |scale| * log2(e) for bf16; scale * log2(e) for fp32
+    // split-bf16 kernel (fp32 tensors as hi + lo bf16 terms): k / v above are the hi planes, these the lo planes; q is
+    // the caller's fp32 tensor
+    const void* k_lo;
+    const void* v_lo;
 };
 
 constexpr int kBM = 128;       // queries per workgroup
@@ -438,6 +442,276 @@ __global__ void __launch_bounds__(256, 3) prefill_bf16_kernel(PrefillArgs a) {
             }
         if (a.lse && h == 0)
             a.lse[(int64_t)b * a.sl[0] + (int64_t)hq * a.sl[1] + (int64_t)qi * a.sl[2]] = (m_ref + __builtin_amdgcn_logf(l)) * 0.6931471805599453f;
+    }
+#endif
+}
+
+// ---------------------------------------------------------------------------------------------
+// fp32 tensors on the bf16 matrix cores.  Every operand x is split into two bf16 terms, x = hi + lo with hi = bf16(x)
+// and lo = bf16(x - hi) (16 significant bits between them), and every product is taken as
+//     a b  ~  hi_a hi_b + hi_a lo_b + lo_a hi_b          (fp32 accumulation; the dropped lo_a lo_b is 2^-16 of a b)
+// for Q K^T and, with P split the same way after the exponential, for P V.  Three bf16 MFMAs per product at 16 times the
+// fp32 MFMA rate, against the reference's fp32 arithmetic (src/ops/flash_attention.cpp:218-364) within its 1e-4 bar
+// (observed: below 2e-5 of the output's magnitude).  A pre-pass writes the hi / lo planes of K and V, dense, into a
+// caller workspace (Q is split by the wavefront that owns the rows); the attention kernel is prefill_bf16_kernel's
+// structure over twice the tiles.
+// ---------------------------------------------------------------------------------------------
+struct SplitPlan {  // K and V
+    const float* src[2];
+    uint16_t* hi[2];
+    uint16_t* lo[2];
+    int64_t s0[2], s1[2], s2[2];  // source strides of dims 0..2 (elements)
+    int32_t H, N;
+    int64_t groups;               // 8-element groups per tensor
+    int32_t D;
+};
+
+__global__ void __launch_bounds__(256) split_f32_kernel(SplitPlan p) {
+    const int t = blockIdx.y;
+    const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (g >= p.groups) return;
+    const int per_row = p.D / 8;
+    const int d8 = (int)(g % per_row);
+    const int64_t row = g / per_row;
+    const int n = (int)(row % p.N);
+    const int64_t bh = row / p.N;
+    const int h = (int)(bh % p.H);
+    const int64_t b = bh / p.H;
+    const float* src = p.src[t] + b * p.s0[t] + (int64_t)h * p.s1[t] + (int64_t)n * p.s2[t] + 8 * d8;
+    const float4 x0 = *(const float4*)src, x1 = *(const float4*)(src + 4);
+    const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+    uint32_t hw[4], lw[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        hw[i] = cvt_pk_bf16(x[2 * i], x[2 * i + 1]);
+        const float r0 = x[2 * i] - __uint_as_float(hw[i] << 16), r1 = x[2 * i + 1] - __uint_as_float(hw[i] & 0xffff0000u);
+        lw[i] = cvt_pk_bf16(r0, r1);
+    }
+    *(uint4*)(p.hi[t] + g * 8) = uint4{hw[0], hw[1], hw[2], hw[3]};
+    *(uint4*)(p.lo[t] + g * 8) = uint4{lw[0], lw[1], lw[2], lw[3]};
+}
+
+template <int D>
+__global__ void __launch_bounds__(256, 2) prefill_split_kernel(PrefillArgs a) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the body uses device-only builtins
+    constexpr int KS = D / 16;
+    constexpr int DB = D / 32;
+    constexpr int CPR = D / 8;
+    constexpr int RP = 256 / (2 * D);
+    constexpr int NR = 1024 / (2 * D);
+    constexpr int NGRP = kUnit / NR;
+    constexpr int NLD = (NGRP + 3) / 4;
+    constexpr int SLOT = kUnit * D;
+    constexpr int NJ = kUnit / 16;
+    constexpr int SLOTB = 2 * SLOT;  // bytes per tile
+    // ring slot r holds four tiles: K hi | K lo | V hi | V lo
+    __shared__ __attribute__((aligned(1024))) uint16_t smem[8 * SLOT];
+    const uint32_t lds0 = lds_addr(smem);
+
+    const int bid = blockIdx.x;
+    const int nbh = a.B * a.Hq;
+    const int qt = a.n_qtiles - 1 - bid / nbh;  // heaviest query tiles first
+    const int bh = bid % nbh;
+    const int b = bh / a.Hq, hq = bh % a.Hq, kvh = hq / a.n_rep;
+    const int L = a.L;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ql = lane & 31, h = lane >> 5;
+    const int q0 = qt * kBM + wave * 32;
+    const int off = L - a.T;
+    const int qrow = min(q0 + ql, a.T - 1);
+
+    const int64_t ko = (int64_t)b * a.sk[0] + (int64_t)kvh * a.sk[1];
+    const int64_t vo = (int64_t)b * a.sv[0] + (int64_t)kvh * a.sv[1];
+    // Q comes as the caller's fp32 tensor (any strides) and is split here: each row is read by exactly one wavefront
+    const float* qp = (const float*)a.q + (int64_t)b * a.sq[0] + (int64_t)hq * a.sq[1] + (int64_t)qrow * a.sq[2];
+    bf16x8_t qh[KS], qlo[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        const float4 x0 = *(const float4*)(qp + 16 * ks + 8 * h), x1 = *(const float4*)(qp + 16 * ks + 8 * h + 4);
+        float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+        uint32_t hw[4], lw[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float f0 = a.negate_q ? -x[2 * i] : x[2 * i], f1 = a.negate_q ? -x[2 * i + 1] : x[2 * i + 1];  // exact
+            hw[i] = cvt_pk_bf16(f0, f1);
+            lw[i] = cvt_pk_bf16(f0 - __uint_as_float(hw[i] << 16), f1 - __uint_as_float(hw[i] & 0xffff0000u));
+        }
+        qh[ks] = __builtin_bit_cast(bf16x8_t, uint4{hw[0], hw[1], hw[2], hw[3]});
+        qlo[ks] = __builtin_bit_cast(bf16x8_t, uint4{lw[0], lw[1], lw[2], lw[3]});
+    }
+
+    const int wg_qmax = min(qt * kBM + kBM - 1, a.T - 1);
+    const int kv_end_wg = a.causal ? min(L, wg_qmax + off + 1) : L;
+    const int n_tiles = (kv_end_wg + kUnit - 1) / kUnit;
+    const int wave_qmax = min(q0 + 31, a.T - 1);
+    const int kv_end_wave = (q0 < a.T) ? (a.causal ? min(L, wave_qmax + off + 1) : L) : 0;
+
+    f32x16_t acc[DB];
+#pragma unroll
+    for (int i = 0; i < DB; ++i)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) acc[i][j] = 0.f;
+    float m_ref = -INFINITY;
+    float l = 0.f;
+
+    // global -> LDS as in prefill_bf16_kernel; the planes are dense, so K and V rows have the same pitch
+    const int ld_row = lane / CPR, ld_pos = lane % CPR;
+    uint32_t voffK[NLD], voffV[NLD];
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+        const int r = NR * (wave + 4 * i) + ld_row;
+        voffK[i] = (uint32_t)r * (uint32_t)(2 * D) + 16u * (uint32_t)(ld_pos ^ ((r / RP) % CPR));
+        voffV[i] = (uint32_t)r * (uint32_t)(2 * D) + 16u * (uint32_t)(ld_pos ^ (((r / RP) % (CPR / 4)) << 2));
+    }
+    auto load_tile = [&](int t, int slot) {
+        const int key0 = t * kUnit;
+        const int bytes = (L - key0) * 2 * D;  // rows past the context read as zeros
+        const char* bases[4] = {(const char*)((const uint16_t*)a.k + ko), (const char*)((const uint16_t*)a.k_lo + ko),
+                                (const char*)((const uint16_t*)a.v + vo), (const char*)((const uint16_t*)a.v_lo + vo)};
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)(bases[x] + (int64_t)key0 * 2 * D), 0, bytes, 0x00020000);
+            uint16_t* dst = smem + (4 * slot + x) * SLOT;
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) {
+                const int grp = wave + 4 * i;
+                if (NGRP % 4 != 0 && grp >= NGRP) break;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(dst + grp * 512), 16, x < 2 ? voffK[i] : voffV[i], 0, 0, 0);
+            }
+        }
+    };
+
+    const int kswz = (ql / RP) % CPR;
+    uint32_t kaddr[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) kaddr[ks] = lds0 + 2u * (uint32_t)(ql * D + 8 * ((2 * ks + h) ^ kswz));
+    const int i16 = lane & 15;
+    const int vswz = ((i16 >> 2) / RP) % (CPR / 4);
+    const int v_lane_off = (4 * h + (i16 >> 2)) * D + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+    uint32_t va[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) va[db] = lds0 + 2u * (uint32_t)v_lane_off + 64u * (uint32_t)(db ^ vswz);
+
+    auto tile_step = [&](int t, auto slot_c) {
+        constexpr int slot = decltype(slot_c)::value;
+        constexpr int KH = (4 * slot) * SLOTB, KL = (4 * slot + 1) * SLOTB, VH = (4 * slot + 2) * SLOTB, VL = (4 * slot + 3) * SLOTB;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (t + 1 < n_tiles) load_tile(t + 1, slot ^ 1);
+        const int k0 = t * kUnit;
+        if (k0 >= kv_end_wave) return;
+
+        // S^T = K_hi Q_hi^T + K_hi Q_lo^T + K_lo Q_hi^T; the operands of k-step ks + 1 are requested before those of ks are used
+        f32x16_t s;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) s[j] = 0.f;
+        u32x4_t kh[KS], kl[KS];
+        kh[0] = lds_read_b128_asm<KH>(kaddr[0]);
+        kl[0] = lds_read_b128_asm<KL>(kaddr[0]);
+        static_for<KS>([&](auto i) {
+            constexpr int ks = i.value;
+            if constexpr (ks + 1 < KS) {
+                kh[ks + 1] = lds_read_b128_asm<KH>(kaddr[ks + 1]);
+                kl[ks + 1] = lds_read_b128_asm<KL>(kaddr[ks + 1]);
+                lds_wait<3>(kh[ks]);
+                lds_wait<2>(kl[ks]);
+            } else {
+                lds_wait<1>(kh[ks]);
+                lds_wait<0>(kl[ks]);
+            }
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kh[ks]), qh[ks], s, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kh[ks]), qlo[ks], s, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kl[ks]), qh[ks], s, 0, 0, 0);
+        });
+        const bool need_mask = (a.causal && k0 + kUnit - 1 > q0 + off) || (k0 + kUnit > L);
+        if (need_mask) {
+            const int q_abs = q0 + ql + off;
+            const int lim = a.causal ? min(q_abs, L - 1) : L - 1;
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+                if (k0 + 8 * (v >> 2) + 4 * h + (v & 3) > lim) s[v] = -INFINITY;
+        }
+        float mx = s[0];
+#pragma unroll
+        for (int v = 1; v < 16; ++v) mx = fmaxf(mx, s[v]);
+        mx = half_swap_max(mx) * a.scale_log2;
+        if (__any(mx > m_ref + kRescaleThreshold)) {  // P stays below 2^8 between raises: nothing to lose in fp32
+            const float m_new = fmaxf(m_ref, mx);
+            const float alpha = (m_new == -INFINITY || m_ref == -INFINITY) ? (m_ref == -INFINITY ? 0.f : 1.f) : __builtin_amdgcn_exp2f(m_ref - m_new);
+            l *= alpha;
+#pragma unroll
+            for (int i = 0; i < DB; ++i)
+#pragma unroll
+                for (int j = 0; j < 16; ++j) acc[i][j] *= alpha;
+            m_ref = m_new;
+        }
+        const float neg_m = (m_ref == -INFINITY) ? 0.f : -m_ref;
+        // P = exp2(s scale - m) in fp32, summed in fp32, then split like the inputs
+        uint32_t ph[NJ][4], pl[NJ][4];
+        float lsum = 0.f;
+#pragma unroll
+        for (int v = 0; v < 16; v += 2) {
+            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v], a.scale_log2, neg_m));
+            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[v + 1], a.scale_log2, neg_m));
+            lsum += p0 + p1;
+            const uint32_t hw = cvt_pk_bf16(p0, p1);
+            ph[v >> 3][(v & 7) >> 1] = hw;
+            pl[v >> 3][(v & 7) >> 1] = cvt_pk_bf16(p0 - __uint_as_float(hw << 16), p1 - __uint_as_float(hw & 0xffff0000u));
+        }
+        l += lsum;
+        // O^T += V_hi^T P_hi + V_hi^T P_lo + V_lo^T P_hi, one (key half, d block) at a time, the next operands in flight
+        uint2 vh[2], vl[2], nh[2], nl[2];
+        vh[0] = lds_read_tr16_b64_asm<VH>(va[0]);
+        vh[1] = lds_read_tr16_b64_asm<VH + 8 * D * 2>(va[0]);
+        vl[0] = lds_read_tr16_b64_asm<VL>(va[0]);
+        vl[1] = lds_read_tr16_b64_asm<VL + 8 * D * 2>(va[0]);
+        static_for<NJ * DB>([&](auto ic) {
+            constexpr int idx = ic.value, j = idx / DB, db = idx % DB;
+            if constexpr (idx + 1 < NJ * DB) {
+                constexpr int j2 = (idx + 1) / DB, db2 = (idx + 1) % DB;
+                nh[0] = lds_read_tr16_b64_asm<VH + (16 * j2) * D * 2>(va[db2]);
+                nh[1] = lds_read_tr16_b64_asm<VH + (16 * j2 + 8) * D * 2>(va[db2]);
+                nl[0] = lds_read_tr16_b64_asm<VL + (16 * j2) * D * 2>(va[db2]);
+                nl[1] = lds_read_tr16_b64_asm<VL + (16 * j2 + 8) * D * 2>(va[db2]);
+                asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(vh[0]), "+v"(vh[1]), "+v"(vl[0]), "+v"(vl[1]));
+            } else {
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(vh[0]), "+v"(vh[1]), "+v"(vl[0]), "+v"(vl[1]));
+            }
+            const bf16x8_t pfh = __builtin_bit_cast(bf16x8_t, uint4{ph[j][0], ph[j][1], ph[j][2], ph[j][3]});
+            const bf16x8_t pfl = __builtin_bit_cast(bf16x8_t, uint4{pl[j][0], pl[j][1], pl[j][2], pl[j][3]});
+            const bf16x8_t vfh = __builtin_bit_cast(bf16x8_t, uint4{vh[0].x, vh[0].y, vh[1].x, vh[1].y});
+            const bf16x8_t vfl = __builtin_bit_cast(bf16x8_t, uint4{vl[0].x, vl[0].y, vl[1].x, vl[1].y});
+            acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfh, pfh, acc[db], 0, 0, 0);
+            acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfh, pfl, acc[db], 0, 0, 0);
+            acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfl, pfh, acc[db], 0, 0, 0);
+            if constexpr (idx + 1 < NJ * DB) {
+                vh[0] = nh[0];
+                vh[1] = nh[1];
+                vl[0] = nl[0];
+                vl[1] = nl[1];
+            }
+        });
+    };
+
+    if (n_tiles > 0) load_tile(0, 0);
+    for (int t = 0; t < n_tiles; t += 2) {
+        tile_step(t, std::integral_constant<int, 0>{});
+        if (t + 1 < n_tiles) tile_step(t + 1, std::integral_constant<int, 1>{});
+    }
+
+    l = half_swap_sum(l);
+    const int qi = q0 + ql;
+    if (qi < a.T) {
+        const float inv_l = l > 0.f ? 1.0f / l : 0.f;
+        float* op = (float*)a.out + (int64_t)b * a.so[0] + (int64_t)hq * a.so[1] + (int64_t)qi * a.so[2];
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int vq = 0; vq < 4; ++vq)
+                *(float4*)(op + 32 * db + 8 * vq + 4 * h) = float4{acc[db][4 * vq] * inv_l, acc[db][4 * vq + 1] * inv_l, acc[db][4 * vq + 2] * inv_l, acc[db][4 * vq + 3] * inv_l};
+        if (a.lse && h == 0)
+            a.lse[(int64_t)b * a.sl[0] + (int64_t)hq * a.sl[1] + (int64_t)qi * a.sl[2]] = (m_ref + log2f(l)) * 0.6931471805599453f;
     }
 #endif
 }
@@ -1153,9 +1427,34 @@ extern "C" int vsp_attn_prefill_cached(const vsp_tensor* q, const vsp_kv_cache* 
     return launch_prefill(a, q->dtype, D, cache->format == VSP_KV_BF16, stream);
 }
 
+namespace {
+// Bytes of the hi / lo bf16 planes of Q, K and V (dense [B,H,N,D] each, 256-byte aligned starts).
+size_t split_plane_bytes(int64_t elems) { return (size_t)((elems * 2 + 255) / 256 * 256); }
+
+int prefill_entry(const vsp_tensor* q, const vsp_tensor* k, const vsp_tensor* v, vsp_tensor* out, vsp_tensor* lse, float scale,
+                  int is_causal, float dropout_p, int training, bool split, void* workspace, size_t workspace_bytes, void* stream);
+}  // namespace
+
 extern "C" int vsp_attn_prefill(const vsp_tensor* q, const vsp_tensor* k, const vsp_tensor* v, vsp_tensor* out,
                                 vsp_tensor* lse, float scale, int is_causal, float dropout_p, int training,
                                 void* stream) {
+    return prefill_entry(q, k, v, out, lse, scale, is_causal, dropout_p, training, false, nullptr, 0, stream);
+}
+
+extern "C" size_t vsp_attn_prefill_split_workspace_bytes(int32_t B, int32_t Hq, int32_t Hkv, int32_t T, int32_t L, int32_t D) {
+    if (B <= 0 || Hq <= 0 || Hkv <= 0 || T <= 0 || L <= 0 || D <= 0) return 0;
+    return 4 * split_plane_bytes((int64_t)B * Hkv * L * D);  // hi and lo planes of K and of V
+}
+
+extern "C" int vsp_attn_prefill_split(const vsp_tensor* q, const vsp_tensor* k, const vsp_tensor* v, vsp_tensor* out,
+                                      vsp_tensor* lse, float scale, int is_causal, void* workspace, size_t workspace_bytes,
+                                      void* stream) {
+    return prefill_entry(q, k, v, out, lse, scale, is_causal, 0.0f, 0, true, workspace, workspace_bytes, stream);
+}
+
+namespace {
+int prefill_entry(const vsp_tensor* q, const vsp_tensor* k, const vsp_tensor* v, vsp_tensor* out, vsp_tensor* lse, float scale,
+                  int is_causal, float dropout_p, int training, bool split, void* workspace, size_t workspace_bytes, void* stream) {
     if (!q || !k || !v || !out) return VSP_ERR_NULL;
     // validation in the reference's order, src/ops/flash_attention.cpp:45-59
     if (q->ndim != 4 || k->ndim != 4 || v->ndim != 4) return VSP_ERR_NDIM;
@@ -1217,5 +1516,47 @@ extern "C" int vsp_attn_prefill(const vsp_tensor* q, const vsp_tensor* k, const 
     a.n_qtiles = (int)ceil_div(T, kBM);
     a.negate_q = (q->dtype == VSP_BF16 && scale < 0.0f) ? 1 : 0;
     a.scale_log2 = (q->dtype == VSP_BF16 ? fabsf(scale) : scale) * kLog2e;
+    if (split) {
+        // fp32 tensors through the bf16 matrix cores: split planes in the workspace, then the attention kernel over them
+        if (q->dtype != VSP_F32 || (D != 64 && D != 128)) return VSP_ERR_UNSUPPORTED;
+        const int64_t nk = B * Hkv * L * D;
+        if (L * D * 2 > INT32_MAX || nk / 8 > INT32_MAX * 256LL) return VSP_ERR_ARG;
+        const size_t need = 4 * split_plane_bytes(nk);
+        if (!workspace || workspace_bytes < need) return VSP_ERR_WORKSPACE;
+        if (!is_aligned16(workspace)) return VSP_ERR_ALIGN;
+        uint16_t* planes[4];
+        for (int i = 0; i < 4; ++i) planes[i] = (uint16_t*)((char*)workspace + i * split_plane_bytes(nk));
+        SplitPlan sp{};
+        const vsp_tensor* src[2] = {k, v};
+        for (int t = 0; t < 2; ++t) {
+            sp.src[t] = (const float*)src[t]->data;
+            sp.hi[t] = planes[2 * t];
+            sp.lo[t] = planes[2 * t + 1];
+            sp.s0[t] = src[t]->stride[0];
+            sp.s1[t] = src[t]->stride[1];
+            sp.s2[t] = src[t]->stride[2];
+        }
+        sp.H = (int)Hkv;
+        sp.N = (int)L;
+        sp.groups = nk / 8;
+        sp.D = (int)D;
+        hipStream_t st = (hipStream_t)stream;
+        hipLaunchKernelGGL(split_f32_kernel, dim3((unsigned)ceil_div(nk / 8, 256), 2), dim3(256), 0, st, sp);
+        rc = check_launch();
+        if (rc != VSP_OK) return rc;
+        a.k = planes[0];
+        a.k_lo = planes[1];
+        a.v = planes[2];
+        a.v_lo = planes[3];
+        a.sk[0] = Hkv * L * D, a.sk[1] = L * D, a.sk[2] = D;
+        a.sv[0] = a.sk[0], a.sv[1] = a.sk[1], a.sv[2] = D;
+        a.negate_q = scale < 0.0f ? 1 : 0;
+        a.scale_log2 = fabsf(scale) * kLog2e;
+        const dim3 grid((unsigned)((int64_t)a.n_qtiles * B * Hq));
+        if (D == 128) hipLaunchKernelGGL(prefill_split_kernel<128>, grid, dim3(256), 0, st, a);
+        else hipLaunchKernelGGL(prefill_split_kernel<64>, grid, dim3(256), 0, st, a);
+        return check_launch();
+    }
     return launch_prefill(a, q->dtype, D, false, stream);
 }
+}  // namespace
