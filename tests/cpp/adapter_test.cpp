@@ -142,6 +142,12 @@ static void test_flash_attention_against_oracle() {
                                                  to_dev(v, {B, H, N, D}, DType::Float32), scale, causal != 0);
         CHECK(max_abs_diff(to_host(outs), want.data(), want.size()) < 1e-4);
         CHECK(max_abs_diff(to_host(outs), to_host(out).data(), want.size()) < 5e-5);
+        // and the process-wide switch that sends the reference-shaped call the same way
+        ops::fp32_on_bf16_matrix_cores() = true;
+        Tensor outw = ops::flash_attention(to_dev(q, {B, H, N, D}, DType::Float32), to_dev(k, {B, H, N, D}, DType::Float32),
+                                           to_dev(v, {B, H, N, D}, DType::Float32), scale, causal != 0);
+        ops::fp32_on_bf16_matrix_cores() = false;
+        CHECK(max_abs_diff(to_host(outw), to_host(outs).data(), want.size()) == 0.0);
         auto qb = bf16_round(q), kb = bf16_round(k), vb = bf16_round(v);
         orc_flash_attention_f32(qb.data(), kb.data(), vb.data(), want.data(), lse.data(), B, H, N, D, scale, causal);
         Tensor outb = ops::flash_attention(to_dev(qb, {B, H, N, D}, DType::BFloat16), to_dev(kb, {B, H, N, D}, DType::BFloat16),

@@ -397,6 +397,14 @@ inline Tensor repeat_kv(const Tensor& x, int64_t n_rep) {
     return r;
 }
 
+// Process-wide choice for fp32 tensors of head_dim 64 / 128 in flash_attention_hip_dispatch: false (default) = fp32 matrix
+// cores, bit-level properties of the fp32 algorithm kept; true = bf16 matrix cores with every operand as two bf16 terms
+// (vsp_attn_prefill_split), several times faster and inside the reference's 1e-4 tolerance.
+inline bool& fp32_on_bf16_matrix_cores() {
+    static bool on = false;
+    return on;
+}
+
 // include/vesper/ops/flash_attention.h:74-78.  output/lse are caller-allocated; lse may be undefined.
 inline void flash_attention_hip_dispatch(const Tensor& q, const Tensor& k, const Tensor& v, Tensor& output, Tensor& lse,
                                          float scale, bool is_causal, float dropout_p, bool training,
@@ -407,6 +415,16 @@ inline void flash_attention_hip_dispatch(const Tensor& q, const Tensor& k, const
     // a repeat_kv'ed operand must expand to exactly q's head count
     if (q.ndim() == 4 && kk.ndim() == 4 && (kk.shape()[1] * kk.head_rep != q.shape()[1] || vv.shape()[1] * vv.head_rep != q.shape()[1]))
         throw_status(VSP_ERR_SHAPE);
+    if (fp32_on_bf16_matrix_cores() && q.ndim() == 4 && kk.ndim() == 4 && q.dtype() == DType::Float32 && kk.dtype() == DType::Float32 &&
+        vv.dtype() == DType::Float32 && (q.shape()[3] == 64 || q.shape()[3] == 128) && !(training && dropout_p > 0.0f) &&
+        q.shape()[2] > 0 && kk.shape()[2] > 0) {
+        const size_t ws_bytes = vsp_attn_prefill_split_workspace_bytes((int32_t)q.shape()[0], (int32_t)q.shape()[1], (int32_t)kk.shape()[1],
+                                                                       (int32_t)q.shape()[2], (int32_t)kk.shape()[2], (int32_t)q.shape()[3]);
+        Storage ws(ws_bytes > 0 ? ws_bytes : 16);
+        throw_status(vsp_attn_prefill_split(&dq, &dk, &dv, &dout, lse.defined() ? &dl : nullptr, scale, is_causal ? 1 : 0, ws.data(),
+                                            ws_bytes, current_stream()));
+        return;
+    }
     throw_status(vsp_attn_prefill(&dq, &dk, &dv, &dout, lse.defined() ? &dl : nullptr, scale, is_causal ? 1 : 0, dropout_p,
                                   training ? 1 : 0, current_stream()));
 }
