@@ -505,82 +505,110 @@ __global__ void __launch_bounds__(256, 2) decode_q8_kernel(DecodeArgs a) {
 // fp32 cache in the reference's own layout: plain fp32 arithmetic, one workgroup per
 // (batch row, query head, split).  Correctness path for callers that keep the reference's fp32 cache.
 // ---------------------------------------------------------------------------------------------
-template <int MAXD>
+// NH query heads of one kv head per workgroup (NH divides n_rep), so that K and V are read n_rep / NH times instead of
+// n_rep times; a thread owns a key in the score phase and a (d, key residue) pair in the output phase.
+template <int MAXD, int NH>
 __global__ void __launch_bounds__(256) decode_f32_kernel(DecodeArgs a, int D) {
     const int tid = threadIdx.x;
-    const int hq = blockIdx.y;
+    const int hq0 = blockIdx.y * NH;
     int b, split, L;
     if (!locate_work(a, blockIdx.x, tid & 63, b, split, L)) return;
     const int chunk_start = split * a.chunk;
     const int chunk_end = min(L, chunk_start + a.chunk);
     const int n = chunk_end - chunk_start;
-    const int kvh = hq / a.n_rep;
+    const int kvh = hq0 / a.n_rep;
 
     extern __shared__ float smem[];
-    float* sq = smem;              // [MAXD]
-    float* sp = smem + MAXD;       // [chunk]
-    float* red = sp + a.chunk;     // [256]
-    const float* qrow = (const float*)a.q + (int64_t)b * a.sq_b + (int64_t)hq * a.sq_h;
-    for (int d = tid; d < D; d += 256) sq[d] = qrow[d];
+    float* sq = smem;                    // [NH][MAXD]
+    float* sp = smem + NH * MAXD;        // [NH][chunk]
+    float* red = sp + NH * a.chunk;      // [256]
+    for (int i = tid; i < NH * D; i += 256) {
+        const int r = i / D, d = i - r * D;
+        sq[r * MAXD + d] = ((const float*)a.q + (int64_t)b * a.sq_b + (int64_t)(hq0 + r) * a.sq_h)[d];
+    }
     __syncthreads();
     const float* Kp = (const float*)a.k + (((int64_t)b * a.Hkv + kvh) * a.S + chunk_start) * D;
     const float* Vp = (const float*)a.v + (((int64_t)b * a.Hkv + kvh) * a.S + chunk_start) * D;
-    float mloc = -INFINITY;
+    float mloc[NH];
+#pragma unroll
+    for (int r = 0; r < NH; ++r) mloc[r] = -INFINITY;
     for (int j = tid; j < n; j += 256) {
         const float4* kr = (const float4*)(Kp + (int64_t)j * D);
-        float s = 0.f;
+        float s[NH];
+#pragma unroll
+        for (int r = 0; r < NH; ++r) s[r] = 0.f;
         for (int d4 = 0; d4 < D / 4; ++d4) {
             const float4 kk = kr[d4];
-            s = fmaf(sq[4 * d4], kk.x, s);
-            s = fmaf(sq[4 * d4 + 1], kk.y, s);
-            s = fmaf(sq[4 * d4 + 2], kk.z, s);
-            s = fmaf(sq[4 * d4 + 3], kk.w, s);
+#pragma unroll
+            for (int r = 0; r < NH; ++r) {
+                const float* qr = sq + r * MAXD + 4 * d4;
+                s[r] = fmaf(qr[0], kk.x, s[r]);
+                s[r] = fmaf(qr[1], kk.y, s[r]);
+                s[r] = fmaf(qr[2], kk.z, s[r]);
+                s[r] = fmaf(qr[3], kk.w, s[r]);
+            }
         }
-        s *= a.scale_log2;
-        sp[j] = s;
-        mloc = fmaxf(mloc, s);
+#pragma unroll
+        for (int r = 0; r < NH; ++r) {
+            const float t = s[r] * a.scale_log2;
+            sp[r * a.chunk + j] = t;
+            mloc[r] = fmaxf(mloc[r], t);
+        }
     }
-    red[tid] = mloc;
-    __syncthreads();
-    for (int st = 128; st > 0; st >>= 1) {
-        if (tid < st) red[tid] = fmaxf(red[tid], red[tid + st]);
+    float m[NH], l[NH];
+#pragma unroll
+    for (int r = 0; r < NH; ++r) {
+        red[tid] = mloc[r];
+        __syncthreads();
+        for (int st = 128; st > 0; st >>= 1) {
+            if (tid < st) red[tid] = fmaxf(red[tid], red[tid + st]);
+            __syncthreads();
+        }
+        m[r] = red[0];
+        __syncthreads();
+        float lloc = 0.f;
+        for (int j = tid; j < n; j += 256) {
+            const float p = exp2f(sp[r * a.chunk + j] - m[r]);
+            sp[r * a.chunk + j] = p;
+            lloc += p;
+        }
+        red[tid] = lloc;
+        __syncthreads();
+        for (int st = 128; st > 0; st >>= 1) {
+            if (tid < st) red[tid] += red[tid + st];
+            __syncthreads();
+        }
+        l[r] = red[0];
         __syncthreads();
     }
-    const float m = red[0];
-    __syncthreads();
-    float lloc = 0.f;
-    for (int j = tid; j < n; j += 256) {
-        const float p = exp2f(sp[j] - m);
-        sp[j] = p;
-        lloc += p;
-    }
-    red[tid] = lloc;
-    __syncthreads();
-    for (int st = 128; st > 0; st >>= 1) {
-        if (tid < st) red[tid] += red[tid + st];
-        __syncthreads();
-    }
-    const float l = red[0];
-    __syncthreads();
     // PV: thread (d, part) sums keys part, part+P, ...; P = 256 / D' where D' = D rounded up to a power of two
     int Dp = 1;
     while (Dp < D) Dp <<= 1;
     const int P = 256 / Dp > 0 ? 256 / Dp : 1;
     const int d = tid % Dp, part = tid / Dp;
-    float o = 0.f;
+    float o[NH];
+#pragma unroll
+    for (int r = 0; r < NH; ++r) o[r] = 0.f;
     if (d < D && part < P)
-        for (int j = part; j < n; j += P) o = fmaf(sp[j], Vp[(int64_t)j * D + d], o);
-    __syncthreads();
-    red[tid] = o;
-    __syncthreads();
-    if (tid < D && tid < Dp) {
-        float t = 0.f;
-        for (int p = 0; p < P; ++p) t += red[p * Dp + tid];
-        const int64_t row = ((int64_t)b * a.Hq + hq) * a.max_splits + split;
-        a.ws_o[row * D + tid] = t;
-        if (tid == 0) {
-            a.ws_ml[row * 2] = m;
-            a.ws_ml[row * 2 + 1] = l;
+        for (int j = part; j < n; j += P) {
+            const float vv = Vp[(int64_t)j * D + d];
+#pragma unroll
+            for (int r = 0; r < NH; ++r) o[r] = fmaf(sp[r * a.chunk + j], vv, o[r]);
+        }
+#pragma unroll
+    for (int r = 0; r < NH; ++r) {
+        __syncthreads();
+        red[tid] = o[r];
+        __syncthreads();
+        if (tid < D && tid < Dp) {
+            float t = 0.f;
+            for (int p = 0; p < P; ++p) t += red[p * Dp + tid];
+            const int64_t row = ((int64_t)b * a.Hq + hq0 + r) * a.max_splits + split;
+            a.ws_o[row * D + tid] = t;
+            if (tid == 0) {
+                a.ws_ml[row * 2] = m[r];
+                a.ws_ml[row * 2 + 1] = l[r];
+            }
         }
     }
 }
@@ -971,9 +999,13 @@ int decode_impl(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* s
                 else hipLaunchKernelGGL((decode_q8_kernel<64, false>), grid, dim3(256), 0, st, a);
             }
         } else {
-            dim3 grid((unsigned)(max_splits * B), (unsigned)Hq);
-            const size_t smem = (256 + chunk + 256) * sizeof(float);
-            hipLaunchKernelGGL(decode_f32_kernel<256>, grid, dim3(256), smem, st, a, (int)D);
+            // as many query heads of a kv head per workgroup as divide n_rep (up to four: 16 KB of scores each at chunk 1024)
+            const int nh = n_rep % 4 == 0 ? 4 : (n_rep % 2 == 0 ? 2 : 1);
+            dim3 grid((unsigned)(max_splits * B), (unsigned)(Hq / nh));
+            const size_t smem = ((size_t)nh * 256 + (size_t)nh * chunk + 256) * sizeof(float);
+            if (nh == 4) hipLaunchKernelGGL((decode_f32_kernel<256, 4>), grid, dim3(256), smem, st, a, (int)D);
+            else if (nh == 2) hipLaunchKernelGGL((decode_f32_kernel<256, 2>), grid, dim3(256), smem, st, a, (int)D);
+            else hipLaunchKernelGGL((decode_f32_kernel<256, 1>), grid, dim3(256), smem, st, a, (int)D);
         }
         rc = check_launch();
         if (rc != VSP_OK) return rc;
