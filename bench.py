@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on ONE MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|p4k|c3|c2f|c4|c5|c4p|c4w|c2c|c3c|r2|b2|b3] [--no-cpu] [--no-extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|p4k|c3|c2f|c4|c5|c4f|c4p|c4w|c2c|c3c|r2|b2|b3] [--no-cpu] [--no-extra]
 
 A "step" is one pass of the hot path over one batch of synthetic input that is already resident in
 HBM: one prefill launch (c2, p4k, c3) or one decode call = split-K kernel + combine kernel (c4, c5).
@@ -40,6 +40,9 @@ WORKLOADS = {
                name="BASELINE config 4: batched decode bf16 KV cache, B32, 32 q / 8 kv heads, D128, L~U[1024,32768]"),
     "c5": dict(kind="decode", fmt="q8_0", B=16, Hq=64, Hkv=8, D=128, S=65536, lens=None,
                name="BASELINE config 5: decode over Q8_0 KV cache, B16, 64 q / 8 kv heads, D128, L=65536"),
+    "c4f": dict(kind="decode", fmt="f32", B=32, Hq=32, Hkv=8, D=128, S=32768, lens=(1024, 32768, 4004),
+                name="config 4 with the reference's own fp32 cache layout (fp32 q, fp32 matrix instructions): B32, 32 q / 8 kv heads, "
+                     "D128, L~U[1024,32768]; algorithmic bytes = the fp32 K and V rows"),
     "c4p": dict(kind="decode", fmt="bf16", B=32, Hq=32, Hkv=8, D=128, S=32768, lens=(1024, 32768, 4004), page=256,
                 name="config 4 over a paged cache: pages of 256 tokens in a shuffled page table, otherwise as config 4"),
     "c4w": dict(kind="decode", fmt="bf16", B=32, Hq=32, Hkv=8, D=128, S=32768, lens=(1024, 32768, 4004), proj=True,
@@ -73,8 +76,9 @@ def prefill_flops(w):
 
 
 def decode_bytes(w, lens):
-    row = 2 * w["D"] if w["fmt"] == "bf16" else (w["D"] + 2 * (w["D"] // 32))  # bytes per (token, kv head) per plane
-    return float(sum(2 * w["Hkv"] * int(L) * row for L in lens) + w["B"] * w["Hq"] * w["D"] * (2 + 2))
+    esz = {"bf16": 2, "f32": 4}.get(w["fmt"])
+    row = esz * w["D"] if esz else (w["D"] + 2 * (w["D"] // 32))  # bytes per (token, kv head) per plane
+    return float(sum(2 * w["Hkv"] * int(L) * row for L in lens) + w["B"] * w["Hq"] * w["D"] * 2 * (esz or 2))
 
 
 class Runner:
@@ -161,7 +165,7 @@ class Runner:
                     del kb, vb
             self.cache.set_len(S)
             self.seq_lens = torch.from_numpy(lens).to(dev)
-            self.q = torch.randn(B, Hq, 1, D, device=dev, generator=g).to(torch.bfloat16)
+            self.q = torch.randn(B, Hq, 1, D, device=dev, generator=g).to(torch.float32 if w["fmt"] == "f32" else torch.bfloat16)
             self.out = torch.empty_like(self.q)
             self.scale = 1.0 / math.sqrt(D)
             self.work = decode_bytes(w, lens)
@@ -171,7 +175,9 @@ class Runner:
                 self.y = torch.empty(B, 1, C_, device=dev, dtype=torch.bfloat16)
                 self.work += C_ * C_ * 2
             self.unit, self.peak, self.bound = "GB/s", HBM_PEAK_GBS, "hbm"
-            self.kernel = ("decode_bf16_kernel<128, %s>" if w["fmt"] == "bf16" else "decode_q8_kernel<128, %s>") % ("true" if w.get("page") else "false")
+            paged = "true" if w.get("page") else "false"
+            self.kernel = {"bf16": f"decode_bf16_kernel<128, {paged}>", "q8_0": f"decode_q8_kernel<128, {paged}>",
+                           "f32": "decode_f32_mfma_kernel<128>"}[w["fmt"]]
             self.max_len = int(lens.max())
 
     def _append_row(self, b, kb, vb):
@@ -313,6 +319,7 @@ PROFILE_OF = {
     "r2": ("rope_append_bf16_config2.txt", "append_bf16_tile_kernel<unsigned short, true", 202375168),
     "c4": ("decode_bf16_config4.txt", "decode_bf16_kernel", 2614935552),
     "c5": ("decode_q8_0_config5.txt", "decode_q8_kernel", 2282225664),
+    "c4f": ("decode_f32_config4.txt", "decode_f32_mfma_kernel", 5229871104),
 }
 CALIBRATION_KERNEL, CALIBRATION_KIB = "CUDAFunctorOnSelf_add<int>", 1048576.0
 
@@ -399,7 +406,7 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": ("f32 operands as two bf16 terms (bf16 MFMA, fp32 accumulation)" if primary.w["kind"] == "prefill_split"
-                  else "bf16" if primary.w.get("fmt", "bf16") == "bf16" else "q8_0 (int8 payload, fp16 MFMA)"),
+                  else {"bf16": "bf16", "f32": "f32", "q8_0": "q8_0 (int8 payload, fp16 MFMA)"}[primary.w.get("fmt", "bf16")]),
         "data": "synthetic",
         "config": {"workload": primary.w["name"], "key": args.workload,
                    "algorithmic_work_per_step": primary.work,
@@ -420,7 +427,7 @@ def main():
 
     if not args.no_extra:
         others = {}
-        for key in ("c2", "p4k", "c3", "c2f", "c4", "c5", "c4p", "c4w", "c2c", "c3c", "r2", "b2", "b3"):
+        for key in ("c2", "p4k", "c3", "c2f", "c4", "c5", "c4f", "c4p", "c4w", "c2c", "c3c", "r2", "b2", "b3"):
             if key == args.workload:
                 continue
             r = Runner(key, torch, va)

@@ -65,13 +65,37 @@ def test_q8_0_decode_against_oracle_over_dequantised_cache(va, B, Hq, Hkv, S, D,
     G.assert_bf16_close(G.bf16_to_np(out), oracle_decode(q, kd, vd, lens), f"q8_0 lens={lens}")
 
 
-@pytest.mark.parametrize("B,Hq,Hkv,S,D,lens", [(2, 8, 2, 300, 64, [300, 41]), (1, 4, 4, 1200, 128, [1111]), (1, 2, 1, 40, 32, [40])])
+# D 64 / 128 with up to 16 query heads per kv head run on the fp32 matrix instructions, everything else (D 32: the
+# reference's own test shapes; 32 query heads on one kv head) on the plain-FMA kernel
+@pytest.mark.parametrize("B,Hq,Hkv,S,D,lens", [
+    (2, 8, 2, 300, 64, [300, 41]), (1, 4, 4, 1200, 128, [1111]), (1, 2, 1, 40, 32, [40]),
+    (3, 16, 1, 2500, 128, [2500, 1, 1025]), (2, 6, 2, 777, 64, [0, 777]), (2, 12, 4, 130, 128, [31, 33]),
+    (1, 32, 1, 200, 64, [200]), (4, 8, 8, 96, 128, [16, 17, 32, 96])])
 def test_f32_decode_against_oracle(va, B, Hq, Hkv, S, D, lens):
     q, k, v = I.qkv(43, B, Hq, Hkv, 1, S, D)
     c = fill_cache(va, "f32", k, v)
     sl = torch.tensor(lens, dtype=torch.int32, device=G.dev())
     out = va.decode_attention(G.f32_dev(q), c, seq_lens=sl)
     G.assert_f32_close(out.cpu().numpy(), oracle_decode(q, k, v, lens), "f32 decode")
+    assert torch.equal(out, va.decode_attention(G.f32_dev(q), c, seq_lens=sl))  # fixed split order
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_f32_decode_ignores_rows_past_the_length(va, D):
+    # the fp32 planes are the reference's layout, unpadded: rows past a sequence's length may hold anything (here NaN
+    # and infinities), and the last row of the last head is the end of the allocation
+    B, Hq, Hkv, S = 2, 8, 2, 300
+    lens = [173, 300]
+    q, k, v = I.qkv(47, B, Hq, Hkv, 1, S, D)
+    c = fill_cache(va, "f32", k, v)
+    sl = torch.tensor(lens, dtype=torch.int32, device=G.dev())
+    a = va.decode_attention(G.f32_dev(q), c, seq_lens=sl)
+    G.assert_f32_close(a.cpu().numpy(), oracle_decode(q, k, v, lens), "before poisoning")
+    kp = c.raw_plane(0).view(torch.float32).view(B, Hkv, S, D)
+    vp = c.raw_plane(1).view(torch.float32).view(B, Hkv, S, D)
+    kp[0, :, lens[0]:] = float("nan")
+    vp[0, :, lens[0]:] = float("inf")
+    assert torch.equal(a, va.decode_attention(G.f32_dev(q), c, seq_lens=sl))
 
 
 def test_decode_after_token_by_token_appends_matches_causal_prefill(va):

@@ -502,8 +502,9 @@ __global__ void __launch_bounds__(256, 2) decode_q8_kernel(DecodeArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// fp32 cache in the reference's own layout: plain fp32 arithmetic, one workgroup per
-// (batch row, query head, split).  Correctness path for callers that keep the reference's fp32 cache.
+// fp32 cache in the reference's own layout, any head size: plain fp32 arithmetic, one workgroup per
+// (batch row, group of query heads, split).  Serves what decode_f32_mfma_kernel does not take (D other than 64 / 128,
+// more than 16 query heads per kv head).
 // ---------------------------------------------------------------------------------------------
 // NH query heads of one kv head per workgroup (NH divides n_rep), so that K and V are read n_rep / NH times instead of
 // n_rep times; a thread owns a key in the score phase and a (d, key residue) pair in the output phase.
@@ -609,6 +610,175 @@ __global__ void __launch_bounds__(256) decode_f32_kernel(DecodeArgs a, int D) {
                 a.ws_ml[row * 2] = m[r];
                 a.ws_ml[row * 2 + 1] = l[r];
             }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// fp32 cache, D = 64 or 128, n_rep <= 16: the bf16 kernel's structure on fp32 matrix instructions
+// (v_mfma_f32_16x16x4_f32), so that the reference's own cache layout is also read once per kv head and at the
+// rate HBM delivers it.  One workgroup (4 wavefronts) per (batch row, kv head, context split); a wavefront
+// consumes 32 keys per iteration as two 16-key tiles.
+//   S^T[key][head] = K[key][:] . Q^T[:][head]: lane (row i, k-slot kk) of the A operand loads the 16 bytes
+//     K[key i][16 cc + 4 kk .. + 3] and feeds its four floats to four MFMAs; MFMA (cc, e) contracts over
+//     d = 16 cc + 4 kk + e, and the Q^T operand is laid out to match (scale * log2(e) folded in).
+//   O^T[d][head] += V^T[d][key] . P^T[key][head]: the S^T result of a lane holds keys 4 g + v of the tile, so
+//     k-step v of the PV product takes the keys {4 kk + v}: P needs no cross-lane movement and stays fp32.
+//     Lane (row i, kk) loads the 16 bytes V[key 4 kk + v][64 vc + 4 i .. + 3] and feeds them to four MFMAs;
+//     tile (vc, e) therefore holds the rows d = 64 vc + 4 i + e.
+// Keys past the end of the split are read from the split's last valid row instead (the planes are not padded, and
+// rows that were never written may hold anything) and masked in S.
+// ---------------------------------------------------------------------------------------------
+template <int D>
+__global__ void __launch_bounds__(256, 2) decode_f32_mfma_kernel(DecodeArgs a) {
+    constexpr int C4 = D / 16;  // 16-byte pieces of a K row per lane
+    constexpr int VC = D / 64;  // 16-byte pieces of a V row per lane
+    constexpr int KT = 2;       // 16-key tiles per wavefront iteration
+    constexpr int GROUP = 16 * KT;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kvh = blockIdx.y;
+    int b, split, L;
+    if (!locate_work(a, blockIdx.x, lane, b, split, L)) return;
+    const int chunk_start = split * a.chunk;
+    const int chunk_end = min(L, chunk_start + a.chunk);
+    const int c = lane & 15, g = lane >> 4;
+
+    float qf[C4][4];
+    {
+        const float* qrow = (const float*)a.q + (int64_t)b * a.sq_b + (int64_t)(kvh * a.n_rep + min(c, a.n_rep - 1)) * a.sq_h;
+#pragma unroll
+        for (int cc = 0; cc < C4; ++cc) {
+            const float4 w = *(const float4*)(qrow + 16 * cc + 4 * g);
+            const float f = c < a.n_rep ? a.scale_log2 : 0.f;
+            qf[cc][0] = w.x * f, qf[cc][1] = w.y * f, qf[cc][2] = w.z * f, qf[cc][3] = w.w * f;
+        }
+    }
+    const float* Kp = (const float*)a.k + ((int64_t)b * a.Hkv + kvh) * a.S * D;
+    const float* Vp = (const float*)a.v + ((int64_t)b * a.Hkv + kvh) * a.S * D;
+
+    f32x4_t acc[VC][4];
+#pragma unroll
+    for (int i = 0; i < VC; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[i][e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+
+    float4 kf[KT][C4];
+    float4 vf[KT][4][VC];
+    const int last = chunk_end - 1;
+    auto load_k = [&](int kbase) {
+#pragma unroll
+        for (int t = 0; t < KT; ++t) {
+            const float* kr = Kp + (int64_t)min(kbase + 16 * t + c, last) * D + 4 * g;
+#pragma unroll
+            for (int cc = 0; cc < C4; ++cc) kf[t][cc] = *(const float4*)(kr + 16 * cc);
+        }
+    };
+    auto load_v = [&](int kbase) {
+#pragma unroll
+        for (int t = 0; t < KT; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const float* vr = Vp + (int64_t)min(kbase + 16 * t + 4 * g + v, last) * D + 4 * c;
+#pragma unroll
+                for (int vc = 0; vc < VC; ++vc) vf[t][v][vc] = *(const float4*)(vr + 64 * vc);
+            }
+    };
+    const int kfirst = chunk_start + wave * GROUP;
+    if (kfirst < chunk_end) {
+        load_k(kfirst);
+        load_v(kfirst);
+    }
+    for (int kbase = kfirst; kbase < chunk_end; kbase += kWaves * GROUP) {
+        const int knext = kbase + kWaves * GROUP;
+        f32x4_t s[KT];
+#pragma unroll
+        for (int t = 0; t < KT; ++t) {
+            s[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int cc = 0; cc < C4; ++cc) {
+                const float kk[4] = {kf[t][cc].x, kf[t][cc].y, kf[t][cc].z, kf[t][cc].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) s[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kk[e], qf[cc][e], s[t], 0, 0, 0);
+            }
+        }
+        if (knext < chunk_end) load_k(knext);
+        const bool tail = kbase + GROUP > chunk_end;
+        float mloc = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < KT; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                float x = s[t][v];
+                if (tail && kbase + 16 * t + 4 * g + v >= chunk_end) x = -INFINITY;
+                s[t][v] = x;
+                mloc = fmaxf(mloc, x);
+            }
+        mloc = wave_max_over_groups(mloc);
+        const float m_new = fmaxf(m, mloc);  // finite: the group holds at least one valid key
+        const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+        float lsum = 0.f;
+#pragma unroll
+        for (int t = 0; t < KT; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                s[t][v] = __builtin_amdgcn_exp2f(s[t][v] - m_new);
+                lsum += s[t][v];
+            }
+        l = l * alpha + lsum;
+        m = m_new;
+#pragma unroll
+        for (int vc = 0; vc < VC; ++vc)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[vc][e] *= alpha;
+#pragma unroll
+        for (int t = 0; t < KT; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+#pragma unroll
+                for (int vc = 0; vc < VC; ++vc) {
+                    const float vv[4] = {vf[t][v][vc].x, vf[t][v][vc].y, vf[t][v][vc].z, vf[t][v][vc].w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[vc][e] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv[e], s[t][v], acc[vc][e], 0, 0, 0);
+                }
+        if (knext < chunk_end) load_v(knext);
+    }
+    l = wave_sum_over_groups(l);
+
+    // ---- combine the four wavefronts through LDS, write one partial per (b, head, split)
+    __shared__ float sm_o[kWaves][16][D + 4];
+    __shared__ float sm_m[kWaves][16], sm_l[kWaves][16];
+    if (c < a.n_rep) {
+#pragma unroll
+        for (int vc = 0; vc < VC; ++vc)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) sm_o[wave][c][64 * vc + 4 * (4 * g + v) + e] = acc[vc][e][v];
+        if (g == 0) {
+            sm_m[wave][c] = m;
+            sm_l[wave][c] = l;
+        }
+    }
+    __syncthreads();
+    for (int i = tid; i < a.n_rep * D; i += 256) {
+        const int hc = i / D, d = i % D;
+        float mm = sm_m[0][hc];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) mm = fmaxf(mm, sm_m[w][hc]);
+        float o = 0.f, ll = 0.f;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            // a wavefront that saw no key of a short split carries m = -inf, l = 0 and zero sums
+            const float f = sm_m[w][hc] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(sm_m[w][hc] - mm);
+            o += f * sm_o[w][hc][d];
+            ll += f * sm_l[w][hc];
+        }
+        const int64_t row = ((int64_t)b * a.Hq + kvh * a.n_rep + hc) * a.max_splits + split;
+        a.ws_o[row * D + d] = o;
+        if (d == 0) {
+            a.ws_ml[row * 2] = mm;
+            a.ws_ml[row * 2 + 1] = ll;
         }
     }
 }
@@ -998,6 +1168,10 @@ int decode_impl(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* s
                 if (D == 128) hipLaunchKernelGGL((decode_q8_kernel<128, false>), grid, dim3(256), 0, st, a);
                 else hipLaunchKernelGGL((decode_q8_kernel<64, false>), grid, dim3(256), 0, st, a);
             }
+        } else if ((D == 64 || D == 128) && n_rep <= 16) {
+            dim3 grid((unsigned)(max_splits * B), cache->Hkv);
+            if (D == 128) hipLaunchKernelGGL((decode_f32_mfma_kernel<128>), grid, dim3(256), 0, st, a);
+            else hipLaunchKernelGGL((decode_f32_mfma_kernel<64>), grid, dim3(256), 0, st, a);
         } else {
             // as many query heads of a kv head per workgroup as divide n_rep (up to four: 16 KB of scores each at chunk 1024)
             const int nh = n_rep % 4 == 0 ? 4 : (n_rep % 2 == 0 ? 2 : 1);
