@@ -146,6 +146,28 @@ def test_q8_0_cache(va):
     assert rc == _ffi.ERR_WORKSPACE
 
 
+@pytest.mark.parametrize("fmt", ["bf16", "q8_0"])
+def test_module_level_prefill_reads_the_planes_in_place(va, fmt, monkeypatch):
+    # GroupedQueryAttention::forward(x, cache, 0) with T > 1 (src/nn/gqa_attention.cpp:128-148) on a bf16 / Q8_0
+    # cache: the attention core goes through vsp_attn_prefill_cached, not through a read-back of the context
+    B, Hq, Hkv, T, D = 2, 8, 2, 70, 128
+    q, k, v = [O.bf16_round(x * np.float32(0.5)) for x in I.qkv(3500, B, Hq, Hkv, T, T, D)]
+    c = va.KVCache(B, Hkv, 96, D, fmt=fmt)
+
+    def no_read(*a, **kw):
+        raise AssertionError("attention_core materialised the cache")
+    monkeypatch.setattr(va.KVCache, "read", no_read)
+    out = va.attention_core(G.to_bf16_dev(q), G.to_bf16_dev(k), G.to_bf16_dev(v), c, 0)
+    assert c.current_seq_len() == T
+    assert torch.equal(out, c.prefill(G.to_bf16_dev(q)))
+    if fmt == "q8_0":
+        k, v = O.q8_0_dequantize(*O.q8_0_quantize(k)), O.q8_0_dequantize(*O.q8_0_quantize(v))
+    G.assert_bf16_close(G.bf16_to_np(out), _expected(q, k, v, T, T), fmt)
+    # the reference cannot add its [T, T] mask to [T, L] scores: a second multi-token call is an error there too
+    with pytest.raises(va.VspError):
+        va.attention_core(G.to_bf16_dev(q), G.to_bf16_dev(k), G.to_bf16_dev(v), va.KVCache(B, Hkv, 200, D, fmt=fmt), 5)
+
+
 def test_argument_errors(va):
     q = torch.zeros(1, 4, 8, 64, device=G.dev(), dtype=torch.bfloat16)
     c = va.KVCache(1, 2, 64, 64, fmt="bf16")

@@ -359,11 +359,12 @@ def attention_core(q, new_k, new_v, cache=None, start_pos=0, rope=None, q_dtype=
         cache.update(new_k, new_v, start_pos, return_views=False)
     if T == 1:
         return decode_attention(q, cache)
-    if cache.fmt == "f32":
-        k, v = cache.views()
-    else:
-        k, v = cache.views(dtype=q.dtype)
-    L = k.shape[2]
-    if L != T:
+    if cache.current_seq_len() != T:
         raise VspError(_ffi.ERR_BROADCAST)  # the reference's [T,T] mask cannot be added to [T,L] scores
+    if cache.fmt == "f32":
+        k, v = cache.views()  # true views of the fp32 planes, as in the reference
+        return flash_attention(q, k, v, 1.0 / math.sqrt(q.shape[-1]), is_causal=True)
+    if q.dtype == torch.bfloat16:
+        return cache.prefill(q, is_causal=True)  # bf16 / Q8_0 planes are read in place, nothing is materialised
+    k, v = cache.views(dtype=q.dtype)  # fp32 queries over a narrower cache: the context is widened once
     return flash_attention(q, k, v, 1.0 / math.sqrt(q.shape[-1]), is_causal=True)
