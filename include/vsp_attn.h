@@ -228,6 +228,22 @@ int vsp_attn_prefill_backward(const vsp_tensor* dout, const vsp_tensor* q, const
                               vsp_tensor* dv, float scale, int is_causal, void* workspace, size_t workspace_bytes,
                               void* stream);
 
+/* vsp_attn_prefill_backward for fp32 tensors at matrix-core speed: the backward companion of vsp_attn_prefill_split
+ * (the reference computes this op in fp32, src/ops/flash_attention.cpp:366-482, and its modules hold fp32 tensors).
+ * Same arguments and semantics as vsp_attn_prefill_backward with every tensor fp32 and D in {64, 128} (else
+ * VSP_ERR_UNSUPPORTED).  A pre-pass writes Q, K, V and dO as two bf16 planes each
+ * (x = hi + lo) and Di = rowsum(dO * O) in fp32 into the workspace; the two passes of the bf16 path then take every
+ * product as hi hi + hi lo + lo hi with fp32 accumulation, with P and dS split the same way after the fp32 algebra,
+ * and store fp32 gradients.  Inputs: base pointers 8-byte aligned, even strides; dq/dk/dv: 16-byte aligned, strides
+ * multiples of 4 elements (VSP_ERR_ALIGN).  workspace: vsp_attn_backward_split_workspace_bytes() bytes, 16-byte aligned.
+ * Results agree with the reference's fp32 gradients within its 1e-4 bar at several times the rate of the fp32-MFMA path;
+ * bitwise reproducible like the other paths. */
+size_t vsp_attn_backward_split_workspace_bytes(int32_t B, int32_t Hq, int32_t Hkv, int32_t N, int32_t D);
+int vsp_attn_prefill_backward_split(const vsp_tensor* dout, const vsp_tensor* q, const vsp_tensor* k, const vsp_tensor* v,
+                                    const vsp_tensor* out, const vsp_tensor* lse, vsp_tensor* dq, vsp_tensor* dk,
+                                    vsp_tensor* dv, float scale, int is_causal, void* workspace, size_t workspace_bytes,
+                                    void* stream);
+
 /* Chunked / offset prefill straight over the cache planes (no counterpart in the reference, whose causal mask is
  * [T,T] and cannot be added to [T,L] scores, src/nn/functional.cpp:406-410; the semantics are the rows
  * [L-T, L) of the reference's full causal forward over L tokens, src/ops/flash_attention.cpp:218-364):

@@ -169,6 +169,14 @@ static void test_flash_attention_against_oracle() {
         CHECK(max_abs_diff(to_host(std::get<0>(g)), wq.data(), wq.size()) < 2e-4);
         CHECK(max_abs_diff(to_host(std::get<1>(g)), wk.data(), wk.size()) < 2e-4);
         CHECK(max_abs_diff(to_host(std::get<2>(g)), wv.data(), wv.size()) < 2e-4);
+        // the process-wide switch sends the same call through the split-operand backward (fp32 tensors, bf16 matrix cores)
+        ops::fp32_on_bf16_matrix_cores() = true;
+        auto gs = ops::flash_attention_backward(tdo, tq, tk, tv, out, l, scale, true);
+        ops::fp32_on_bf16_matrix_cores() = false;
+        CHECK(max_abs_diff(to_host(std::get<0>(gs)), wq.data(), wq.size()) < 2e-4);
+        CHECK(max_abs_diff(to_host(std::get<1>(gs)), wk.data(), wk.size()) < 2e-4);
+        CHECK(max_abs_diff(to_host(std::get<2>(gs)), wv.data(), wv.size()) < 2e-4);
+        CHECK(max_abs_diff(to_host(std::get<0>(gs)), to_host(std::get<0>(g)).data(), wq.size()) > 0.0);   // it is the other kernel
     }
     // the reference's validation messages (src/ops/flash_attention.cpp:45-59)
     Tensor a = empty({1, 2, 4, 64}, DType::Float32), b = empty({1, 2, 5, 64}, DType::Float32), c3 = empty({2, 4, 64}, DType::Float32);

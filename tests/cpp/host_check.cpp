@@ -264,6 +264,22 @@ static void test_validation() {
     CHECK(vsp_attn_prefill_backward(&q, &q, &k, &k, &q, &lse, &q, &k, &k, 0.1f, 1, nullptr, 0, nullptr) == VSP_ERR_WORKSPACE);
     CHECK(vsp_attn_prefill_backward(&q, &q, &k5, &k5, &q, &lse, &q, &k5, &k5, 0.1f, 1, mem, 1 << 16, nullptr) == VSP_ERR_SHAPE);
     CHECK(vsp_attn_backward_workspace_bytes(1, 4, 8) == 2u * 4 * 8 * 4);
+    // backward with split operands: fp32 only, head_dim 64 / 128, workspace for Di, lse and the eight planes
+    {
+        vsp_tensor qf = tensor4(mem, VSP_F32, 1, 4, 8, 64), kf = tensor4(mem, VSP_F32, 1, 2, 8, 64), k3 = tensor4(mem, VSP_F32, 1, 3, 8, 64);
+        CHECK(vsp_attn_prefill_backward_split(&qf, &qf, &kf, &kf, &qf, &lse, &qf, &kf, &kf, 0.1f, 1, nullptr, 0, nullptr) == VSP_ERR_WORKSPACE);
+        CHECK(vsp_attn_prefill_backward_split(&qf, &qf, &kf, &kf, &qf, &lse, &qf, &kf, &kf, 0.1f, 1, mem, 64, nullptr) == VSP_ERR_WORKSPACE);
+        CHECK(vsp_attn_prefill_backward_split(&q, &q, &k, &k, &q, &lse, &q, &k, &k, 0.1f, 1, mem, 1 << 16, nullptr) == VSP_ERR_UNSUPPORTED);   // bf16
+        CHECK(vsp_attn_prefill_backward_split(&qf, &qf, &k3, &k3, &qf, &lse, &qf, &k3, &k3, 0.1f, 1, mem, 1 << 16, nullptr) == VSP_ERR_SHAPE);
+        CHECK(vsp_attn_prefill_backward_split(&qf, &qf, &kf, &kf, &qf, &lse, &qf, &kf, &q, 0.1f, 1, mem, 1 << 16, nullptr) == VSP_ERR_SHAPE);   // dv of q's shape
+        vsp_tensor q32 = tensor4(mem, VSP_F32, 1, 4, 8, 32), k32 = tensor4(mem, VSP_F32, 1, 2, 8, 32);
+        CHECK(vsp_attn_prefill_backward_split(&q32, &q32, &k32, &k32, &q32, &lse, &q32, &k32, &k32, 0.1f, 1, mem, 1 << 16, nullptr) == VSP_ERR_UNSUPPORTED);
+        vsp_tensor odd = qf;
+        odd.data = (char*)mem + 4;   // rows are read in 8-byte pieces
+        CHECK(vsp_attn_prefill_backward_split(&odd, &qf, &kf, &kf, &qf, &lse, &qf, &kf, &kf, 0.1f, 1, mem, 1 << 16, nullptr) == VSP_ERR_ALIGN);
+        CHECK(vsp_attn_backward_split_workspace_bytes(1, 4, 2, 8, 64) == 2u * 4 * 8 * 4 + 4u * (4 + 2) * 8 * 64 * 2);
+        CHECK(vsp_attn_backward_split_workspace_bytes(1, 4, 0, 8, 64) == 0);
+    }
     // cached prefill: the chunk is part of the context, so T = 8 over a context of 4 is a shape error
     c.len = 4;
     CHECK(vsp_attn_prefill_cached(&q, &c, nullptr, nullptr, &out, nullptr, 0.1f, 1, nullptr, 0, nullptr) == VSP_ERR_SHAPE);

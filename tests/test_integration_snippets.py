@@ -27,6 +27,9 @@ BLOCKS = [
     ("chunked prefill over the cache", "function",
      "vsp_tensor dq_rot, vsp_tensor dout, vsp_kv_cache cache_desc, int D, void* workspace, void* stream"),
     ("flash_attention_backward_hip_dispatch", "global", ""),
+    ("the same body for fp32 tensors with split operands", "function",
+     f"{_T} q, {_T} k, vsp_tensor d_dout, vsp_tensor dq_, vsp_tensor dk_, vsp_tensor dv_, vsp_tensor d_out, vsp_tensor d_lse, "
+     "vsp_tensor d_gq, vsp_tensor d_gk, vsp_tensor d_gv, float scale, bool is_causal"),
 ]
 
 

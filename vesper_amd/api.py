@@ -89,6 +89,20 @@ def flash_attention_backward(grad_output, q, k, v, output, lse, scale, is_causal
     return dq, dk, dv
 
 
+def flash_attention_backward_split(grad_output, q, k, v, output, lse, scale, is_causal=True, workspace=None):
+    """ops::flash_attention_backward for fp32 tensors through the bf16 matrix cores (vsp_attn_prefill_backward_split):
+    every operand as two bf16 terms, three MFMAs per product, fp32 accumulation and fp32 gradients."""
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    descs = [_desc(t) for t in (grad_output, q, k, v, output, lse, dq, dk, dv)]
+    if workspace is None:
+        nws = lib.vsp_attn_backward_split_workspace_bytes(q.shape[0], q.shape[1], k.shape[1], q.shape[2], q.shape[3]) \
+            if q.dim() == 4 and k.dim() == 4 else 0
+        workspace = torch.empty(max(nws, 16), dtype=torch.uint8, device=q.device)
+    check(lib.vsp_attn_prefill_backward_split(*[C.byref(d) for d in descs], float(scale), int(bool(is_causal)),
+                                              C.c_void_p(workspace.data_ptr()), workspace.numel(), _stream(q)))
+    return dq, dk, dv
+
+
 class RopeTable:
     """{cos, sin} of the angles of functional::compute_rope_frequencies (src/nn/functional.cpp:424-443) for
     absolute positions [0, length): computed once on the host by the library, kept on the device."""

@@ -397,9 +397,10 @@ inline Tensor repeat_kv(const Tensor& x, int64_t n_rep) {
     return r;
 }
 
-// Process-wide choice for fp32 tensors of head_dim 64 / 128 in flash_attention_hip_dispatch: false (default) = fp32 matrix
-// cores, bit-level properties of the fp32 algorithm kept; true = bf16 matrix cores with every operand as two bf16 terms
-// (vsp_attn_prefill_split), several times faster and inside the reference's 1e-4 tolerance.
+// Process-wide choice for fp32 tensors of head_dim 64 / 128 in flash_attention_hip_dispatch and
+// flash_attention_backward_hip_dispatch: false (default) = fp32 matrix cores, bit-level properties of the fp32 algorithm
+// kept; true = bf16 matrix cores with every operand as two bf16 terms (vsp_attn_prefill_split,
+// vsp_attn_prefill_backward_split), several times faster and inside the reference's 1e-4 tolerance.
 inline bool& fp32_on_bf16_matrix_cores() {
     static bool on = false;
     return on;
@@ -469,6 +470,15 @@ inline void flash_attention_backward_hip_dispatch(const Tensor& grad_output, con
     if (dropout_p > 0.0f) throw_status(VSP_ERR_UNSUPPORTED);
     vsp_tensor d0 = grad_output.desc(), d1 = q.desc(), d2 = k.desc(), d3 = v.desc(), d4 = output.desc(), d5 = lse.desc();
     vsp_tensor o0 = grad_q.desc(), o1 = grad_k.desc(), o2 = grad_v.desc();
+    if (fp32_on_bf16_matrix_cores() && q.ndim() == 4 && k.ndim() == 4 && q.dtype() == DType::Float32 &&
+        (q.shape()[3] == 64 || q.shape()[3] == 128) && q.shape()[2] > 0) {   // the switch covers the backward of the same tensors
+        const size_t split_bytes = vsp_attn_backward_split_workspace_bytes((int32_t)q.shape()[0], (int32_t)q.shape()[1], (int32_t)k.shape()[1],
+                                                                           (int32_t)q.shape()[2], (int32_t)q.shape()[3]);
+        Storage split_ws(split_bytes ? split_bytes : 16);
+        throw_status(vsp_attn_prefill_backward_split(&d0, &d1, &d2, &d3, &d4, &d5, &o0, &o1, &o2, scale, is_causal ? 1 : 0, split_ws.data(),
+                                                     split_bytes, current_stream()));
+        return;
+    }
     const size_t ws_bytes = q.ndim() == 4 ? vsp_attn_backward_workspace_bytes((int32_t)q.shape()[0], (int32_t)q.shape()[1], (int32_t)q.shape()[2]) : 0;
     Storage ws(ws_bytes ? ws_bytes : 4);
     throw_status(vsp_attn_prefill_backward(&d0, &d1, &d2, &d3, &d4, &d5, &o0, &o1, &o2, scale, is_causal ? 1 : 0, ws.data(), ws_bytes,

@@ -34,6 +34,7 @@ struct BwdArgs {
     int32_t B, Hq, Hkv, n_rep, N;
     int32_t causal;
     float scale;
+    int64_t lo_q, lo_kv;                   // split operands: elements from a hi plane to its lo plane (q-shaped, kv-shaped)
 };
 
 template <typename T>
@@ -347,14 +348,32 @@ __device__ inline uint32_t cvt_pk_bf16(float a, float b) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
+// four consecutive gradient elements from accumulator registers v .. v + 3: bf16 (rounded to nearest even) or fp32
+template <bool F32>
+__device__ inline void store4(void* base, int64_t elem, float f, const f32x16_t& acc, int v) {
+    if constexpr (F32) {
+        *(float4*)((float*)base + elem) = float4{f * acc[v], f * acc[v + 1], f * acc[v + 2], f * acc[v + 3]};
+    } else {
+        uint2 w;
+        w.x = cvt_pk_bf16(f * acc[v], f * acc[v + 1]);
+        w.y = cvt_pk_bf16(f * acc[v + 2], f * acc[v + 3]);
+        *(uint2*)((uint16_t*)base + elem) = w;
+    }
+}
+
 // ---- dQ (bf16): the structure of bwd_dq_kernel; K serves both as rows (S^T) and transposed (dQ^T) ----
-template <int D>
-__global__ void __launch_bounds__(256, 2) bwd_dq_bf16_kernel(BwdArgs a) {
+// SPLIT: fp32 tensors taken as two bf16 terms each (x = hi + lo, planes written by bwd_split_kernel); every product
+// is hi hi + hi lo + lo hi, dS is split the same way after the fp32 algebra, Di and lse * log2(e) come from the
+// pre-pass, and dQ is stored as fp32.
+template <int D, bool SPLIT = false>
+__global__ void __launch_bounds__(256, SPLIT ? 1 : 2) bwd_dq_bf16_kernel(BwdArgs a) {
     constexpr int KS = D / 16, DB = D / 32;
     // One variable per ring slot: the compiler then knows that a read of one slot does not touch the slot a
     // direct-to-LDS load in flight is filling, and does not wait for that load.
     __shared__ __attribute__((aligned(1024))) uint16_t sK0[kBT * D], sK1[kBT * D];
     __shared__ __attribute__((aligned(1024))) uint16_t sV0[kBT * D], sV1[kBT * D];
+    __shared__ __attribute__((aligned(1024))) uint16_t sKl0[SPLIT ? kBT * D : 8], sKl1[SPLIT ? kBT * D : 8];   // the lo planes' tiles
+    __shared__ __attribute__((aligned(1024))) uint16_t sVl0[SPLIT ? kBT * D : 8], sVl1[SPLIT ? kBT * D : 8];
     const int n_qtiles = (a.N + kBQ - 1) / kBQ;
     const int bid = blockIdx.x;
     const int qt = n_qtiles - 1 - bid / (a.B * a.Hq);
@@ -370,17 +389,23 @@ __global__ void __launch_bounds__(256, 2) bwd_dq_bf16_kernel(BwdArgs a) {
     const uint16_t* Op = (const uint16_t*)a.dout + (int64_t)b * a.s_do[0] + (int64_t)hq * a.s_do[1] + (int64_t)qrow * a.s_do[2];
     const uint16_t* Kp = (const uint16_t*)a.k + (int64_t)b * a.s_k[0] + (int64_t)kvh * a.s_k[1];
     const uint16_t* Vp = (const uint16_t*)a.v + (int64_t)b * a.s_v[0] + (int64_t)kvh * a.s_v[1];
-    bf16x8_t qf[KS], dof[KS];
+    bf16x8_t qf[KS], dof[KS], qfl[SPLIT ? KS : 1], dofl[SPLIT ? KS : 1];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
         qf[ks] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(Qp + 16 * ks + 8 * h));
         dof[ks] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(Op + 16 * ks + 8 * h));
+        if constexpr (SPLIT) {
+            qfl[ks] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(Qp + a.lo_q + 16 * ks + 8 * h));
+            dofl[ks] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(Op + a.lo_q + 16 * ks + 8 * h));
+        }
     }
     // Di = rowsum(dO * O) of this lane's query: each lane holds half of the row of dO (the operand above) and reads the
     // same half of O; the two halves meet across lane ^ 32.  Every query row belongs to exactly one wavefront of this
     // launch, which also leaves Di and lse * log2(e) in the workspace for the dK/dV pass that follows.
     float di_q = 0.f;
-    {
+    if constexpr (SPLIT) {
+        di_q = a.delta[((int64_t)b * a.Hq + hq) * a.N + qrow];
+    } else {
         const uint16_t* Orow = (const uint16_t*)a.out + (int64_t)b * a.s_o[0] + (int64_t)hq * a.s_o[1] + (int64_t)qrow * a.s_o[2];
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
@@ -395,8 +420,9 @@ __global__ void __launch_bounds__(256, 2) bwd_dq_bf16_kernel(BwdArgs a) {
         }
         di_q += __shfl_xor(di_q, 32);
     }
-    const float lse_q = kLog2e * a.lse[(int64_t)b * a.s_l[0] + (int64_t)hq * a.s_l[1] + (int64_t)qrow * a.s_l[2]];
-    if (h == 0 && qi < a.N) {
+    const float lse_q = SPLIT ? a.lse2[((int64_t)b * a.Hq + hq) * a.N + qrow]
+                              : kLog2e * a.lse[(int64_t)b * a.s_l[0] + (int64_t)hq * a.s_l[1] + (int64_t)qrow * a.s_l[2]];
+    if (!SPLIT && h == 0 && qi < a.N) {
         a.delta[((int64_t)b * a.Hq + hq) * a.N + qi] = di_q;
         a.lse2[((int64_t)b * a.Hq + hq) * a.N + qi] = lse_q;
     }
@@ -420,6 +446,10 @@ __global__ void __launch_bounds__(256, 2) bwd_dq_bf16_kernel(BwdArgs a) {
     auto load = [&](int kt, auto slot) {
         dk_.load(slot.value ? sK1 : sK0, Kp + (int64_t)kt * kBT * a.s_k[2], a.N - kt * kBT, a.s_k[2], wave);
         dv_.load(slot.value ? sV1 : sV0, Vp + (int64_t)kt * kBT * a.s_v[2], a.N - kt * kBT, a.s_v[2], wave);
+        if constexpr (SPLIT) {
+            dk_.load(slot.value ? sKl1 : sKl0, Kp + a.lo_kv + (int64_t)kt * kBT * a.s_k[2], a.N - kt * kBT, a.s_k[2], wave);
+            dv_.load(slot.value ? sVl1 : sVl0, Vp + a.lo_kv + (int64_t)kt * kBT * a.s_v[2], a.N - kt * kBT, a.s_v[2], wave);
+        }
     };
     auto step = [&](int kt, auto slot) {
         dma_wait_all();
@@ -427,6 +457,8 @@ __global__ void __launch_bounds__(256, 2) bwd_dq_bf16_kernel(BwdArgs a) {
         if (kt + 1 < n_tiles) load(kt + 1, std::integral_constant<int, 1 - slot.value>{});
         const uint16_t* tK = slot.value ? sK1 : sK0;
         const uint16_t* tV = slot.value ? sV1 : sV0;
+        const uint16_t* tKl = slot.value ? sKl1 : sKl0;
+        const uint16_t* tVl = slot.value ? sVl1 : sVl0;
         const int k0 = kt * kBT;
         if (k0 >= kv_end_wave) return;
         f32x16_t s, dp;
@@ -434,16 +466,29 @@ __global__ void __launch_bounds__(256, 2) bwd_dq_bf16_kernel(BwdArgs a) {
         for (int j = 0; j < 16; ++j) s[j] = dp[j] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_row<D>(tK, ks, lane), qf[ks], s, 0, 0, 0);
-            dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_row<D>(tV, ks, lane), dof[ks], dp, 0, 0, 0);
+            const bf16x8_t kh = load_row<D>(tK, ks, lane), vh = load_row<D>(tV, ks, lane);
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kh, qf[ks], s, 0, 0, 0);
+            dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vh, dof[ks], dp, 0, 0, 0);
+            if constexpr (SPLIT) {
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kh, qfl[ks], s, 0, 0, 0);
+                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vh, dofl[ks], dp, 0, 0, 0);
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_row<D>(tKl, ks, lane), qf[ks], s, 0, 0, 0);
+                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_row<D>(tVl, ks, lane), dof[ks], dp, 0, 0, 0);
+            }
         }
-        uint32_t dsw[2][4];
+        uint32_t dsw[2][4], dsl[SPLIT ? 2 : 1][4];
+        // dS as bf16 pairs; SPLIT: the rounding remainders as a second set of pairs
+        auto pack = [&](int v, float d0, float d1) {
+            const uint32_t w = cvt_pk_bf16(d0, d1);
+            dsw[v >> 3][(v & 7) >> 1] = w;
+            if constexpr (SPLIT) dsl[v >> 3][(v & 7) >> 1] = cvt_pk_bf16(d0 - __uint_as_float(w << 16), d1 - __uint_as_float(w & 0xffff0000u));
+        };
         if (k0 + kBT - 1 <= min(q0, a.N - 1) || (!a.causal && k0 + kBT <= a.N)) {   // no position of the tile is masked
 #pragma unroll
             for (int v = 0; v < 16; v += 2) {
                 const float p0 = __builtin_amdgcn_exp2f(fmaf(s[v], scale_log2, -lse_q));
                 const float p1 = __builtin_amdgcn_exp2f(fmaf(s[v + 1], scale_log2, -lse_q));
-                dsw[v >> 3][(v & 7) >> 1] = cvt_pk_bf16(p0 * (dp[v] - di_q), p1 * (dp[v + 1] - di_q));
+                pack(v, p0 * (dp[v] - di_q), p1 * (dp[v + 1] - di_q));
             }
         } else {
 #pragma unroll
@@ -455,15 +500,22 @@ __global__ void __launch_bounds__(256, 2) bwd_dq_bf16_kernel(BwdArgs a) {
                     const float p = __builtin_amdgcn_exp2f(key <= lim ? fmaf(s[v + u], scale_log2, -lse_q) : -INFINITY);
                     d2[u] = p * (dp[v + u] - di_q);
                 }
-                dsw[v >> 3][(v & 7) >> 1] = cvt_pk_bf16(d2[0], d2[1]);
+                pack(v, d2[0], d2[1]);
             }
         }
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const bf16x8_t dsf = __builtin_bit_cast(bf16x8_t, uint4{dsw[j][0], dsw[j][1], dsw[j][2], dsw[j][3]});
 #pragma unroll
-            for (int db = 0; db < DB; ++db)
-                acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_transposed<D>(tK, j, db, lane), dsf, acc[db], 0, 0, 0);
+            for (int db = 0; db < DB; ++db) {
+                const bf16x8_t kt_h = load_transposed<D>(tK, j, db, lane);
+                acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kt_h, dsf, acc[db], 0, 0, 0);
+                if constexpr (SPLIT) {
+                    const bf16x8_t dsfl = __builtin_bit_cast(bf16x8_t, uint4{dsl[j][0], dsl[j][1], dsl[j][2], dsl[j][3]});
+                    acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kt_h, dsfl, acc[db], 0, 0, 0);
+                    acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_transposed<D>(tKl, j, db, lane), dsf, acc[db], 0, 0, 0);
+                }
+            }
         }
     };
     load(0, std::integral_constant<int, 0>{});
@@ -472,16 +524,11 @@ __global__ void __launch_bounds__(256, 2) bwd_dq_bf16_kernel(BwdArgs a) {
         if (kt + 1 < n_tiles) step(kt + 1, std::integral_constant<int, 1>{});
     }
     if (qi < a.N) {
-        uint16_t* op = (uint16_t*)a.dq + (int64_t)b * a.s_dq[0] + (int64_t)hq * a.s_dq[1] + (int64_t)qi * a.s_dq[2];
+        const int64_t row = (int64_t)b * a.s_dq[0] + (int64_t)hq * a.s_dq[1] + (int64_t)qi * a.s_dq[2];
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll
-            for (int vq = 0; vq < 4; ++vq) {
-                uint2 w;
-                w.x = cvt_pk_bf16(a.scale * acc[db][4 * vq], a.scale * acc[db][4 * vq + 1]);
-                w.y = cvt_pk_bf16(a.scale * acc[db][4 * vq + 2], a.scale * acc[db][4 * vq + 3]);
-                *(uint2*)(op + 32 * db + 8 * vq + 4 * h) = w;
-            }
+            for (int vq = 0; vq < 4; ++vq) store4<SPLIT>(a.dq, row + 32 * db + 8 * vq + 4 * h, a.scale, acc[db], 4 * vq);
     }
 }
 
@@ -497,8 +544,10 @@ __global__ void __launch_bounds__(256, 2) bwd_dq_bf16_kernel(BwdArgs a) {
 // therefore live for two iterations and the ring holds three.
 constexpr int kBK = 64;   // key rows per workgroup in the bf16 dK / dV pass
 
-template <int D>
-__global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
+// SPLIT: as in bwd_dq_bf16_kernel; P crosses to the partner as fp32, and each wavefront splits what it feeds to its
+// own second product (P or dS) into two bf16 terms.
+template <int D, bool SPLIT = false>
+__global__ void __launch_bounds__(256, SPLIT ? 1 : 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
     constexpr int KS = D / 16, DB = D / 32;
     // One variable per ring slot: the compiler then knows that a read of one slot does not touch the slot a
     // direct-to-LDS load in flight is filling, and does not wait for that load.
@@ -506,7 +555,11 @@ __global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
     __shared__ __attribute__((aligned(1024))) uint16_t sO0[kBT * D], sO1[kBT * D], sO2[kBT * D];
     __shared__ __attribute__((aligned(256))) float sL0[64], sL1[64], sL2[64];   // lse and Di of the tile's rows (32 used; a
     __shared__ __attribute__((aligned(256))) float sD0[64], sD1[64], sD2[64];   // wavefront instruction fills 64 words)
-    __shared__ __attribute__((aligned(16))) uint32_t sP[3][2][8][64];            // [ring slot][key block][word][lane]
+    __shared__ __attribute__((aligned(16))) uint32_t sP[3][2][SPLIT ? 16 : 8][64];   // [ring slot][key block][word][lane]
+    __shared__ __attribute__((aligned(1024))) uint16_t sQl0[SPLIT ? kBT * D : 8], sQl1[SPLIT ? kBT * D : 8], sQl2[SPLIT ? kBT * D : 8];   // lo planes
+    __shared__ __attribute__((aligned(1024))) uint16_t sOl0[SPLIT ? kBT * D : 8], sOl1[SPLIT ? kBT * D : 8], sOl2[SPLIT ? kBT * D : 8];
+    auto tql = [&](auto s) -> uint16_t* { if constexpr (s.value == 0) return sQl0; else if constexpr (s.value == 1) return sQl1; else return sQl2; };
+    auto tol = [&](auto s) -> uint16_t* { if constexpr (s.value == 0) return sOl0; else if constexpr (s.value == 1) return sOl1; else return sOl2; };
     auto tq = [&](auto s) -> uint16_t* { if constexpr (s.value == 0) return sQ0; else if constexpr (s.value == 1) return sQ1; else return sQ2; };
     auto to = [&](auto s) -> uint16_t* { if constexpr (s.value == 0) return sO0; else if constexpr (s.value == 1) return sO1; else return sO2; };
     auto tl = [&](auto s) -> float* { if constexpr (s.value == 0) return sL0; else if constexpr (s.value == 1) return sL1; else return sL2; };
@@ -528,9 +581,12 @@ __global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
     // the stationary operand: K rows for the P wavefront, V rows for the D wavefront
     const uint16_t* Xp = role_d ? (const uint16_t*)a.v + (int64_t)b * a.s_v[0] + (int64_t)kvh * a.s_v[1] + (int64_t)krow * a.s_v[2]
                                 : (const uint16_t*)a.k + (int64_t)b * a.s_k[0] + (int64_t)kvh * a.s_k[1] + (int64_t)krow * a.s_k[2];
-    bf16x8_t xf[KS];
+    bf16x8_t xf[KS], xfl[SPLIT ? KS : 1];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) xf[ks] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(Xp + 16 * ks + 8 * h));
+    for (int ks = 0; ks < KS; ++ks) {
+        xf[ks] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(Xp + 16 * ks + 8 * h));
+        if constexpr (SPLIT) xfl[ks] = __builtin_bit_cast(bf16x8_t, *(const uint4*)(Xp + a.lo_kv + 16 * ks + 8 * h));
+    }
     f32x16_t acc[DB];
 #pragma unroll
     for (int i = 0; i < DB; ++i)
@@ -561,6 +617,12 @@ __global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
                  a.s_q[2], wave);
         do_.load(to(buf), (const uint16_t*)a.dout + (int64_t)b * a.s_do[0] + (int64_t)hq * a.s_do[1] + (int64_t)qb * a.s_do[2],
                  a.N - qb, a.s_do[2], wave);
+        if constexpr (SPLIT) {
+            dq_.load(tql(buf), (const uint16_t*)a.q + a.lo_q + (int64_t)b * a.s_q[0] + (int64_t)hq * a.s_q[1] + (int64_t)qb * a.s_q[2],
+                     a.N - qb, a.s_q[2], wave);
+            do_.load(tol(buf), (const uint16_t*)a.dout + a.lo_q + (int64_t)b * a.s_do[0] + (int64_t)hq * a.s_do[1] + (int64_t)qb * a.s_do[2],
+                     a.N - qb, a.s_do[2], wave);
+        }
         if (wave == 0)
             row_dma(tl(buf), a.lse2 + ((int64_t)b * a.Hq + hq) * a.N + qb, min(a.N - qb, kBT), 1, lane);
         else if (wave == 1)
@@ -572,26 +634,41 @@ __global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
     // first products of tile t: S (P wavefront) or dP (D wavefront) into s; the P wavefront goes on to P(t),
     // packed into pw and posted for its partner.  Masked or out-of-range positions get P = 0, so a tile that lies
     // wholly above the diagonal or past the end costs its MFMAs and contributes nothing.
-    auto first = [&](int t, auto buf, f32x16_t& s, uint32_t (&pw)[2][4]) {
-        const uint16_t* rows;
-        if constexpr (RD) rows = to(buf);
-        else rows = tq(buf);
+    auto first = [&](int t, auto buf, f32x16_t& s, uint32_t (&pw)[2][4], uint32_t (&pl)[2][4]) {
+        const uint16_t *rows, *rows_lo;
+        if constexpr (RD) rows = to(buf), rows_lo = tol(buf);
+        else rows = tq(buf), rows_lo = tql(buf);
 #pragma unroll
         for (int j = 0; j < 16; ++j) s[j] = 0.f;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
-            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_row<D>(rows, ks, lane), xf[ks], s, 0, 0, 0);
+        for (int ks = 0; ks < KS; ++ks) {
+            const bf16x8_t rh = load_row<D>(rows, ks, lane);
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(rh, xf[ks], s, 0, 0, 0);
+            if constexpr (SPLIT) {
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(rh, xfl[ks], s, 0, 0, 0);
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_row<D>(rows_lo, ks, lane), xf[ks], s, 0, 0, 0);
+            }
+        }
         if constexpr (!RD) {
             const int qb = (qt_begin + fi_t) * kBT;
             float lq[16];
 #pragma unroll
             for (int g = 0; g < 4; ++g) *(float4*)&lq[4 * g] = *(const float4*)&tl(buf)[8 * g + 4 * h];
             const bool edge = (a.causal && qb < key0 + 31) || qb + kBT > a.N || key0 + 32 > a.N;   // same for the wavefront
+            // P as bf16 pairs (SPLIT: the rounding remainders as a second set, and fp32 P posted for the partner)
+            auto pack = [&](int v, float p0, float p1) {
+                const uint32_t w = cvt_pk_bf16(p0, p1);
+                pw[v >> 3][(v & 7) >> 1] = w;
+                if constexpr (SPLIT) {
+                    pl[v >> 3][(v & 7) >> 1] = cvt_pk_bf16(p0 - __uint_as_float(w << 16), p1 - __uint_as_float(w & 0xffff0000u));
+                    sP[buf.value][kb][v][lane] = __float_as_uint(p0);
+                    sP[buf.value][kb][v + 1][lane] = __float_as_uint(p1);
+                }
+            };
             if (!edge) {
 #pragma unroll
                 for (int v = 0; v < 16; v += 2)
-                    pw[v >> 3][(v & 7) >> 1] = cvt_pk_bf16(__builtin_amdgcn_exp2f(fmaf(s[v], scale_log2, -lq[v])),
-                                                           __builtin_amdgcn_exp2f(fmaf(s[v + 1], scale_log2, -lq[v + 1])));
+                    pack(v, __builtin_amdgcn_exp2f(fmaf(s[v], scale_log2, -lq[v])), __builtin_amdgcn_exp2f(fmaf(s[v + 1], scale_log2, -lq[v + 1])));
             } else {
 #pragma unroll
                 for (int v = 0; v < 16; v += 2) {
@@ -602,44 +679,61 @@ __global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
                         const bool ok = qi < a.N && ki < a.N && (!a.causal || ki <= qi);
                         p2[u] = __builtin_amdgcn_exp2f(ok ? fmaf(s[v + u], scale_log2, -lq[v + u]) : -INFINITY);
                     }
-                    pw[v >> 3][(v & 7) >> 1] = cvt_pk_bf16(p2[0], p2[1]);
+                    pack(v, p2[0], p2[1]);
                 }
             }
+            if constexpr (!SPLIT) {
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
+                for (int j = 0; j < 2; ++j)
 #pragma unroll
-                for (int w = 0; w < 4; ++w) sP[buf.value][kb][4 * j + w][lane] = pw[j][w];
+                    for (int w = 0; w < 4; ++w) sP[buf.value][kb][4 * j + w][lane] = pw[j][w];
+            }
             advance(fi_r, fi_t);
         }
     };
     // second products of tile t: dV^T += dO^T P (P wavefront, P from its own registers) or
     // dS = P (dP - Di), dK^T += Q^T dS (D wavefront, P from its partner)
-    auto second = [&](int t, auto buf, const f32x16_t& s, uint32_t (&pw)[2][4]) {
+    auto second = [&](int t, auto buf, const f32x16_t& s, uint32_t (&pw)[2][4], uint32_t (&pl)[2][4]) {
         if constexpr (RD) {
             float di[16];
 #pragma unroll
             for (int g = 0; g < 4; ++g) *(float4*)&di[4 * g] = *(const float4*)&td(buf)[8 * g + 4 * h];
 #pragma unroll
             for (int v = 0; v < 16; v += 2) {
-                const uint32_t w = sP[buf.value][kb][v >> 1][lane];
-                const float p0 = __uint_as_float(w << 16), p1 = __uint_as_float(w & 0xffff0000u);
-                pw[v >> 3][(v & 7) >> 1] = cvt_pk_bf16(p0 * (s[v] - di[v]), p1 * (s[v + 1] - di[v + 1]));
+                float p0, p1;
+                if constexpr (SPLIT) {
+                    p0 = __uint_as_float(sP[buf.value][kb][v][lane]), p1 = __uint_as_float(sP[buf.value][kb][v + 1][lane]);
+                } else {
+                    const uint32_t w = sP[buf.value][kb][v >> 1][lane];
+                    p0 = __uint_as_float(w << 16), p1 = __uint_as_float(w & 0xffff0000u);
+                }
+                const float d0 = p0 * (s[v] - di[v]), d1 = p1 * (s[v + 1] - di[v + 1]);
+                const uint32_t w2 = cvt_pk_bf16(d0, d1);
+                pw[v >> 3][(v & 7) >> 1] = w2;
+                if constexpr (SPLIT) pl[v >> 3][(v & 7) >> 1] = cvt_pk_bf16(d0 - __uint_as_float(w2 << 16), d1 - __uint_as_float(w2 & 0xffff0000u));
             }
         }
-        const uint16_t* cols;
-        if constexpr (RD) cols = tq(buf);
-        else cols = to(buf);
+        const uint16_t *cols, *cols_lo;
+        if constexpr (RD) cols = tq(buf), cols_lo = tql(buf);
+        else cols = to(buf), cols_lo = tol(buf);
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const bf16x8_t bf = __builtin_bit_cast(bf16x8_t, uint4{pw[j][0], pw[j][1], pw[j][2], pw[j][3]});
 #pragma unroll
-            for (int db = 0; db < DB; ++db)
-                acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_transposed<D>(cols, j, db, lane), bf, acc[db], 0, 0, 0);
+            for (int db = 0; db < DB; ++db) {
+                const bf16x8_t ch = load_transposed<D>(cols, j, db, lane);
+                acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ch, bf, acc[db], 0, 0, 0);
+                if constexpr (SPLIT) {
+                    const bf16x8_t bl = __builtin_bit_cast(bf16x8_t, uint4{pl[j][0], pl[j][1], pl[j][2], pl[j][3]});
+                    acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ch, bl, acc[db], 0, 0, 0);
+                    acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_transposed<D>(cols_lo, j, db, lane), bf, acc[db], 0, 0, 0);
+                }
+            }
         }
     };
 
     f32x16_t s_cur;
-    uint32_t pw_cur[2][4];
+    uint32_t pw_cur[2][4], pl_cur[2][4];
     using S0 = std::integral_constant<int, 0>;
     using S1 = std::integral_constant<int, 1>;
     using S2 = std::integral_constant<int, 2>;
@@ -647,7 +741,7 @@ __global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
     if (n_it > 1) load(1, S1{});
     dma_wait_all();
     __syncthreads();
-    first(0, S0{}, s_cur, pw_cur);
+    first(0, S0{}, s_cur, pw_cur, pl_cur);
     // one iteration, for tile `it` in ring slot `buf`
     auto step = [&](int it, auto buf) {
         using B1 = std::integral_constant<int, (buf.value + 1) % 3>;
@@ -657,8 +751,8 @@ __global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
         __syncthreads();
         if (it + 2 < n_it) load(it + 2, B2{});
         // the second products consume s / pw of this tile, then the first products of the next tile refill them
-        second(it, buf, s_cur, pw_cur);
-        if (it + 1 < n_it) first(it + 1, B1{}, s_cur, pw_cur);
+        second(it, buf, s_cur, pw_cur, pl_cur);
+        if (it + 1 < n_it) first(it + 1, B1{}, s_cur, pw_cur, pl_cur);
     };
     for (int it = 0; it < n_it; it += 3) {
         step(it, S0{});
@@ -670,25 +764,81 @@ __global__ void __launch_bounds__(256, 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
     else run(std::false_type{});
     if (ki < a.N) {
         const float f = role_d ? a.scale : 1.f;
-        uint16_t* po = role_d ? (uint16_t*)a.dk + (int64_t)b * a.s_dk[0] + (int64_t)kvh * a.s_dk[1] + (int64_t)ki * a.s_dk[2]
-                              : (uint16_t*)a.dv + (int64_t)b * a.s_dv[0] + (int64_t)kvh * a.s_dv[1] + (int64_t)ki * a.s_dv[2];
+        void* po = role_d ? a.dk : a.dv;
+        const int64_t row = role_d ? (int64_t)b * a.s_dk[0] + (int64_t)kvh * a.s_dk[1] + (int64_t)ki * a.s_dk[2]
+                                   : (int64_t)b * a.s_dv[0] + (int64_t)kvh * a.s_dv[1] + (int64_t)ki * a.s_dv[2];
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll
-            for (int vq = 0; vq < 4; ++vq) {
-                uint2 w;
-                w.x = cvt_pk_bf16(f * acc[db][4 * vq], f * acc[db][4 * vq + 1]);
-                w.y = cvt_pk_bf16(f * acc[db][4 * vq + 2], f * acc[db][4 * vq + 3]);
-                *(uint2*)(po + 32 * db + 8 * vq + 4 * h) = w;
-            }
+            for (int vq = 0; vq < 4; ++vq) store4<SPLIT>(po, row + 32 * db + 8 * vq + 4 * h, f, acc[db], 4 * vq);
     }
 }
 
 // Instantiated explicitly: the host pass of this compiler drops the implicit instantiation of the launch stubs.
-template __global__ void bwd_dkdv_bf16_kernel<128>(BwdArgs);
-template __global__ void bwd_dkdv_bf16_kernel<64>(BwdArgs);
-template __global__ void bwd_dq_bf16_kernel<128>(BwdArgs);
-template __global__ void bwd_dq_bf16_kernel<64>(BwdArgs);
+template __global__ void bwd_dkdv_bf16_kernel<128, false>(BwdArgs);
+template __global__ void bwd_dkdv_bf16_kernel<64, false>(BwdArgs);
+template __global__ void bwd_dq_bf16_kernel<128, false>(BwdArgs);
+template __global__ void bwd_dq_bf16_kernel<64, false>(BwdArgs);
+template __global__ void bwd_dkdv_bf16_kernel<128, true>(BwdArgs);
+template __global__ void bwd_dkdv_bf16_kernel<64, true>(BwdArgs);
+template __global__ void bwd_dq_bf16_kernel<128, true>(BwdArgs);
+template __global__ void bwd_dq_bf16_kernel<64, true>(BwdArgs);
+
+// ---- pre-pass of the split-operand path: every fp32 operand as two bf16 planes, Di and lse * log2(e) ----
+struct SplitArgs {
+    const float *q, *dout, *out, *k, *v, *lse;
+    int64_t s_q[3], s_do[3], s_o[3], s_k[3], s_v[3], s_l[3];
+    uint16_t *qh, *doh, *kh, *vh;          // hi planes, dense [B][H][N][D]; the lo plane follows at lo_q / lo_kv elements
+    int64_t lo_q, lo_kv;
+    float *delta, *lse2;
+    int32_t B, Hq, Hkv, N, D;
+};
+__device__ inline void split_pair(float x0, float x1, uint16_t* hi, uint16_t* lo) {
+    const uint32_t h = cvt_pk_bf16(x0, x1);
+    *(uint32_t*)hi = h;
+    *(uint32_t*)lo = cvt_pk_bf16(x0 - __uint_as_float(h << 16), x1 - __uint_as_float(h & 0xffff0000u));
+}
+// One wavefront per row: rows [0, B Hq N) are query rows (Q, dO, and Di = rowsum(dO * O) in fp32,
+// src/ops/flash_attention.cpp:416-423), the rest are key rows (K, V).
+__global__ void __launch_bounds__(256) bwd_split_kernel(SplitArgs a) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t rows_q = (int64_t)a.B * a.Hq * a.N, rows_kv = (int64_t)a.B * a.Hkv * a.N;
+    if (row < rows_q) {
+        const int i = (int)(row % a.N);
+        const int64_t bh = row / a.N;
+        const int h = (int)(bh % a.Hq), b = (int)(bh / a.Hq);
+        const float* pq = a.q + (int64_t)b * a.s_q[0] + (int64_t)h * a.s_q[1] + (int64_t)i * a.s_q[2];
+        const float* pd = a.dout + (int64_t)b * a.s_do[0] + (int64_t)h * a.s_do[1] + (int64_t)i * a.s_do[2];
+        const float* po = a.out + (int64_t)b * a.s_o[0] + (int64_t)h * a.s_o[1] + (int64_t)i * a.s_o[2];
+        float di = 0.f;
+        for (int d = 2 * lane; d < a.D; d += 128) {
+            const float2 xq = *(const float2*)(pq + d), xd = *(const float2*)(pd + d), xo = *(const float2*)(po + d);
+            split_pair(xq.x, xq.y, a.qh + row * a.D + d, a.qh + a.lo_q + row * a.D + d);
+            split_pair(xd.x, xd.y, a.doh + row * a.D + d, a.doh + a.lo_q + row * a.D + d);
+            di += xd.x * xo.x;
+            di += xd.y * xo.y;
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) di += __shfl_xor(di, o);
+        if (lane == 0) {
+            a.delta[row] = di;
+            a.lse2[row] = kLog2e * a.lse[(int64_t)b * a.s_l[0] + (int64_t)h * a.s_l[1] + (int64_t)i * a.s_l[2]];
+        }
+    } else if (row < rows_q + rows_kv) {
+        const int64_t r = row - rows_q;
+        const int i = (int)(r % a.N);
+        const int64_t bh = r / a.N;
+        const int h = (int)(bh % a.Hkv), b = (int)(bh / a.Hkv);
+        const float* pk = a.k + (int64_t)b * a.s_k[0] + (int64_t)h * a.s_k[1] + (int64_t)i * a.s_k[2];
+        const float* pv = a.v + (int64_t)b * a.s_v[0] + (int64_t)h * a.s_v[1] + (int64_t)i * a.s_v[2];
+        for (int d = 2 * lane; d < a.D; d += 128) {
+            const float2 xk = *(const float2*)(pk + d), xv = *(const float2*)(pv + d);
+            split_pair(xk.x, xk.y, a.kh + r * a.D + d, a.kh + a.lo_kv + r * a.D + d);
+            split_pair(xv.x, xv.y, a.vh + r * a.D + d, a.vh + a.lo_kv + r * a.D + d);
+        }
+    }
+}
 
 int check4(const vsp_tensor* t, int64_t B, int64_t H, int64_t N, int64_t D, int dtype) {
     if (!t) return VSP_ERR_NULL;
@@ -713,11 +863,11 @@ int launch_backward(const BwdArgs& a, int64_t D, hipStream_t st) {
     if constexpr (sizeof(T) == 2) {
         const dim3 gk((unsigned)(ceil_div(a.N, kBK) * a.B * a.Hkv));
         if (D == 128) {
-            hipLaunchKernelGGL(bwd_dq_bf16_kernel<128>, gq, dim3(256), 0, st, a);
-            hipLaunchKernelGGL(bwd_dkdv_bf16_kernel<128>, gk, dim3(256), 0, st, a);
+            hipLaunchKernelGGL((bwd_dq_bf16_kernel<128, false>), gq, dim3(256), 0, st, a);
+            hipLaunchKernelGGL((bwd_dkdv_bf16_kernel<128, false>), gk, dim3(256), 0, st, a);
         } else {
-            hipLaunchKernelGGL(bwd_dq_bf16_kernel<64>, gq, dim3(256), 0, st, a);
-            hipLaunchKernelGGL(bwd_dkdv_bf16_kernel<64>, gk, dim3(256), 0, st, a);
+            hipLaunchKernelGGL((bwd_dq_bf16_kernel<64, false>), gq, dim3(256), 0, st, a);
+            hipLaunchKernelGGL((bwd_dkdv_bf16_kernel<64, false>), gk, dim3(256), 0, st, a);
         }
         return check_launch();
     }
@@ -733,6 +883,24 @@ int launch_backward(const BwdArgs& a, int64_t D, hipStream_t st) {
     }
     return check_launch();
 }
+
+int launch_backward_split(const SplitArgs& sa, const BwdArgs& a, int64_t D, hipStream_t st) {
+    const int64_t rows = (int64_t)a.B * (a.Hq + a.Hkv) * a.N;
+    hipLaunchKernelGGL(bwd_split_kernel, dim3((unsigned)ceil_div(rows, 4)), dim3(256), 0, st, sa);
+    int rc = check_launch();
+    if (rc != VSP_OK) return rc;
+    const dim3 gq((unsigned)(ceil_div(a.N, kBQ) * a.B * a.Hq)), gk((unsigned)(ceil_div(a.N, kBK) * a.B * a.Hkv));
+    if (D == 128) {
+        hipLaunchKernelGGL((bwd_dq_bf16_kernel<128, true>), gq, dim3(256), 0, st, a);
+        hipLaunchKernelGGL((bwd_dkdv_bf16_kernel<128, true>), gk, dim3(256), 0, st, a);
+    } else {
+        hipLaunchKernelGGL((bwd_dq_bf16_kernel<64, true>), gq, dim3(256), 0, st, a);
+        hipLaunchKernelGGL((bwd_dkdv_bf16_kernel<64, true>), gk, dim3(256), 0, st, a);
+    }
+    return check_launch();
+}
+
+size_t align16(size_t n) { return (n + 15) & ~(size_t)15; }
 
 }  // namespace
 }  // namespace vsp
@@ -811,4 +979,82 @@ extern "C" int vsp_attn_prefill_backward(const vsp_tensor* dout, const vsp_tenso
     a.causal = is_causal ? 1 : 0;
     a.scale = scale;
     return dt == VSP_F32 ? launch_backward<float>(a, D, (hipStream_t)stream) : launch_backward<uint16_t>(a, D, (hipStream_t)stream);
+}
+
+// fp32 tensors, the arithmetic on the bf16 matrix cores with every operand as two bf16 terms (see include/vsp_attn.h).
+extern "C" size_t vsp_attn_backward_split_workspace_bytes(int32_t B, int32_t Hq, int32_t Hkv, int32_t N, int32_t D) {
+    if (B <= 0 || Hq <= 0 || Hkv <= 0 || N <= 0 || D <= 0) return 0;
+    const size_t rows_q = (size_t)B * (size_t)Hq * (size_t)N, rows_kv = (size_t)B * (size_t)Hkv * (size_t)N;
+    return align16(2 * rows_q * sizeof(float)) + 4 * (rows_q + rows_kv) * (size_t)D * sizeof(uint16_t);   // Q, dO, K, V: hi and lo
+}
+
+extern "C" int vsp_attn_prefill_backward_split(const vsp_tensor* dout, const vsp_tensor* q, const vsp_tensor* k,
+                                               const vsp_tensor* v, const vsp_tensor* out, const vsp_tensor* lse,
+                                               vsp_tensor* dq, vsp_tensor* dk, vsp_tensor* dv, float scale, int is_causal,
+                                               void* workspace, size_t workspace_bytes, void* stream) {
+    if (!q || !k || !v) return VSP_ERR_NULL;
+    if (q->ndim != 4 || k->ndim != 4 || v->ndim != 4) return VSP_ERR_NDIM;
+    const int64_t B = q->shape[0], Hq = q->shape[1], N = q->shape[2], D = q->shape[3];
+    const int64_t Hkv = k->shape[1];
+    if (Hkv <= 0 ? Hq != 0 : (Hq % Hkv != 0)) return VSP_ERR_SHAPE;
+    if (q->dtype != VSP_F32) return VSP_ERR_UNSUPPORTED;
+    int rc;
+    if ((rc = check4(q, B, Hq, N, D, VSP_F32)) || (rc = check4(dout, B, Hq, N, D, VSP_F32)) || (rc = check4(out, B, Hq, N, D, VSP_F32)) ||
+        (rc = check4(dq, B, Hq, N, D, VSP_F32)) || (rc = check4(k, B, Hkv, N, D, VSP_F32)) || (rc = check4(v, B, Hkv, N, D, VSP_F32)) ||
+        (rc = check4(dk, B, Hkv, N, D, VSP_F32)) || (rc = check4(dv, B, Hkv, N, D, VSP_F32)))
+        return rc;
+    if (!lse) return VSP_ERR_NULL;
+    if (lse->ndim != 3 || lse->shape[0] != B || lse->shape[1] != Hq || lse->shape[2] != N) return VSP_ERR_SHAPE;
+    if (lse->dtype != VSP_F32) return VSP_ERR_DTYPE;
+    if (B * Hq * N * D == 0) return VSP_OK;
+    if (!lse->data) return VSP_ERR_NULL;
+    if (D != 64 && D != 128) return VSP_ERR_UNSUPPORTED;
+    if (!(fabsf(scale) < INFINITY)) return VSP_ERR_ARG;
+    if (N > INT32_MAX / 2 || (uint64_t)N * (uint64_t)D * 2u > 0x7fffffffull) return VSP_ERR_ARG;
+    if (!workspace || workspace_bytes < vsp_attn_backward_split_workspace_bytes((int32_t)B, (int32_t)Hq, (int32_t)Hkv, (int32_t)N, (int32_t)D))
+        return VSP_ERR_WORKSPACE;
+    if (!is_aligned16(workspace)) return VSP_ERR_ALIGN;
+    for (const vsp_tensor* t : {dout, q, k, v, out}) {   // rows are read in 8-byte pieces
+        if (((uintptr_t)t->data & 7) != 0) return VSP_ERR_ALIGN;
+        for (int i = 0; i < 3; ++i)
+            if (t->stride[i] % 2 != 0) return VSP_ERR_ALIGN;
+    }
+    for (const vsp_tensor* t : {(const vsp_tensor*)dq, (const vsp_tensor*)dk, (const vsp_tensor*)dv}) {   // and written in 16-byte ones
+        if (!is_aligned16(t->data)) return VSP_ERR_ALIGN;
+        for (int i = 0; i < 3; ++i)
+            if (t->stride[i] % 4 != 0) return VSP_ERR_ALIGN;
+    }
+
+    const int64_t rows_q = B * Hq * N, rows_kv = B * Hkv * N;
+    SplitArgs sa{};
+    sa.q = (const float*)q->data, sa.dout = (const float*)dout->data, sa.out = (const float*)out->data;
+    sa.k = (const float*)k->data, sa.v = (const float*)v->data, sa.lse = (const float*)lse->data;
+    for (int i = 0; i < 3; ++i) {
+        sa.s_q[i] = q->stride[i], sa.s_do[i] = dout->stride[i], sa.s_o[i] = out->stride[i];
+        sa.s_k[i] = k->stride[i], sa.s_v[i] = v->stride[i], sa.s_l[i] = lse->stride[i];
+    }
+    sa.delta = (float*)workspace;
+    sa.lse2 = sa.delta + rows_q;
+    sa.qh = (uint16_t*)((char*)workspace + align16(2 * (size_t)rows_q * sizeof(float)));
+    sa.doh = sa.qh + 2 * rows_q * D;
+    sa.kh = sa.doh + 2 * rows_q * D;
+    sa.vh = sa.kh + 2 * rows_kv * D;
+    sa.lo_q = rows_q * D, sa.lo_kv = rows_kv * D;
+    sa.B = (int)B, sa.Hq = (int)Hq, sa.Hkv = (int)Hkv, sa.N = (int)N, sa.D = (int)D;
+
+    BwdArgs a{};
+    a.dout = sa.doh, a.q = sa.qh, a.k = sa.kh, a.v = sa.vh;
+    a.dq = dq->data, a.dk = dk->data, a.dv = dv->data;
+    a.delta = sa.delta, a.lse2 = sa.lse2;
+    const int64_t sq[3] = {Hq * N * D, N * D, D}, skv[3] = {Hkv * N * D, N * D, D};
+    for (int i = 0; i < 3; ++i) {
+        a.s_do[i] = a.s_q[i] = sq[i];
+        a.s_k[i] = a.s_v[i] = skv[i];
+        a.s_dq[i] = dq->stride[i], a.s_dk[i] = dk->stride[i], a.s_dv[i] = dv->stride[i];
+    }
+    a.lo_q = sa.lo_q, a.lo_kv = sa.lo_kv;
+    a.B = (int)B, a.Hq = (int)Hq, a.Hkv = (int)Hkv, a.n_rep = (int)(Hq / Hkv), a.N = (int)N;
+    a.causal = is_causal ? 1 : 0;
+    a.scale = scale;
+    return launch_backward_split(sa, a, D, (hipStream_t)stream);
 }
