@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on ONE MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|p4k|c3|c2f|c4|c5|c4f|c4p|c4w|c2c|c3c|r2|b2|b3] [--no-cpu] [--no-extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|p4k|c3|c2f|c4|c5|c4f|c4p|c4w|c2c|c3c|r2|b2|b3|b2f] [--no-cpu] [--no-extra]
 
 A "step" is one pass of the hot path over one batch of synthetic input that is already resident in
 HBM: one prefill launch (c2, p4k, c3) or one decode call = split-K kernel + combine kernel (c4, c5).
@@ -60,6 +60,10 @@ WORKLOADS = {
     "b3": dict(kind="backward", B=1, Hq=32, Hkv=8, D=128, N=8192,
                name="attention backward at config 3's shape: causal GQA bf16 in/out, bf16 MFMA with fp32 accumulation, "
                     "B1, 32 q / 8 kv heads, D128, N8192 (dq, dk, dv; 2.5 x the forward's FLOPs)"),
+    "b2f": dict(kind="backward_split", B=4, Hq=32, Hkv=8, D=128, N=2048,
+                name="attention backward at config 2's shape with fp32 tensors through the bf16 matrix cores (operands as two "
+                     "bf16 terms, three MFMAs per product, fp32 gradients, within the fp32 bar of 1e-4): causal GQA, B4, "
+                     "32 q / 8 kv heads, D128, N2048; algorithmic FLOPs, against the bf16 MFMA peak"),
     "r2": dict(kind="rope", fmt="bf16", B=4, Hq=32, Hkv=8, D=128, N=2048,
                name="RoPE + KV append for config 2: q/k/v bf16 views of one fused projection buffer [B,T,(Hq+2Hkv)D], "
                     "rotated q out bf16, bf16 cache, B4, 32 q / 8 kv heads, D128, T2048"),
@@ -124,6 +128,17 @@ class Runner:
             self.work = 2.5 * prefill_flops(w)
             self.unit, self.peak, self.bound = "TFLOP/s", MFMA_BF16_PEAK_TFLOPS, "mfma"
             self.kernel = "bwd_dq_bf16_kernel<128> + bwd_dkdv_bf16_kernel<128> (the two launches of one step)"
+        elif w["kind"] == "backward_split":
+            B, Hq, Hkv, D, N = w["B"], w["Hq"], w["Hkv"], w["D"], w["N"]
+            mk = lambda h: torch.randn(B, h, N, D, device=dev, generator=g) * 0.5
+            self.q, self.k, self.v, self.dout = mk(Hq), mk(Hkv), mk(Hkv), mk(Hq)
+            self.scale = 1.0 / math.sqrt(D)
+            ws = torch.empty(va._ffi.lib.vsp_attn_prefill_split_workspace_bytes(B, Hq, Hkv, N, N, D), dtype=torch.uint8, device=dev)
+            self.o, self.lse = va.flash_attention_split(self.q, self.k, self.v, self.scale, True, return_lse=True, workspace=ws)
+            self.ws = torch.empty(va._ffi.lib.vsp_attn_backward_split_workspace_bytes(B, Hq, Hkv, N, D), dtype=torch.uint8, device=dev)
+            self.work = 2.5 * prefill_flops(w)
+            self.unit, self.peak, self.bound = "TFLOP/s", MFMA_BF16_PEAK_TFLOPS, "mfma"
+            self.kernel = "bwd_split_kernel + bwd_dq_bf16_kernel<128, true> + bwd_dkdv_bf16_kernel<128, true> (the three launches of one step)"
         elif w["kind"] == "rope":
             B, Hq, Hkv, D, N = w["B"], w["Hq"], w["Hkv"], w["D"], w["N"]
             fused = (torch.randn(B, N, (Hq + 2 * Hkv) * D, device=dev, generator=g) * 0.5).to(torch.bfloat16)
@@ -203,6 +218,9 @@ class Runner:
             return self.va.flash_attention(self.q, self.k, self.v, self.scale, True)
         if self.w["kind"] == "prefill_split":
             return self.va.flash_attention_split(self.q, self.k, self.v, self.scale, True, workspace=self.ws)
+        if self.w["kind"] == "backward_split":
+            return self.va.flash_attention_backward_split(self.dout, self.q, self.k, self.v, self.o, self.lse, self.scale, True,
+                                                          workspace=self.ws)
         if self.w["kind"] == "backward":
             return self.va.flash_attention_backward(self.dout, self.q, self.k, self.v, self.o, self.lse, self.scale, True)
         if self.w["kind"] == "prefill_cached":
@@ -405,7 +423,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": ("f32 operands as two bf16 terms (bf16 MFMA, fp32 accumulation)" if primary.w["kind"] == "prefill_split"
+        "dtype": ("f32 operands as two bf16 terms (bf16 MFMA, fp32 accumulation)" if primary.w["kind"] in ("prefill_split", "backward_split")
                   else {"bf16": "bf16", "f32": "f32", "q8_0": "q8_0 (int8 payload, fp16 MFMA)"}[primary.w.get("fmt", "bf16")]),
         "data": "synthetic",
         "config": {"workload": primary.w["name"], "key": args.workload,
@@ -427,7 +445,7 @@ def main():
 
     if not args.no_extra:
         others = {}
-        for key in ("c2", "p4k", "c3", "c2f", "c4", "c5", "c4f", "c4p", "c4w", "c2c", "c3c", "r2", "b2", "b3"):
+        for key in ("c2", "p4k", "c3", "c2f", "c4", "c5", "c4f", "c4p", "c4w", "c2c", "c3c", "r2", "b2", "b3", "b2f"):
             if key == args.workload:
                 continue
             r = Runner(key, torch, va)
