@@ -786,7 +786,7 @@ __global__ void __launch_bounds__(256, 2) decode_f32_mfma_kernel(DecodeArgs a) {
 // ---------------------------------------------------------------------------------------------
 // combine: out[b][h][:] = sum_s w_s O_s / sum_s w_s l_s, w_s = 2^(m_s - max m); fixed order.
 // ---------------------------------------------------------------------------------------------
-template <typename OutT>
+template <typename OutT, int BLK>
 __global__ void __launch_bounds__(256) decode_combine_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
                                                              const int32_t* __restrict__ seq_lens, int32_t len, int32_t chunk,
                                                              int32_t max_splits, int32_t Hq, int32_t D, OutT* __restrict__ out,
@@ -795,29 +795,35 @@ __global__ void __launch_bounds__(256) decode_combine_kernel(const float* __rest
     const int L = min(max(seq_lens ? seq_lens[b] : len, 0), L_cap);  // the producers' clamp (locate_work)
     const int ns = min((L + chunk - 1) / chunk, max_splits);
     const int64_t row0 = ((int64_t)b * Hq + hq) * max_splits;
-    float M = -INFINITY;
-    for (int s = 0; s < ns; ++s) M = fmaxf(M, ws_ml[(row0 + s) * 2]);
-    float o = 0.f, l = 0.f;
+    // One pass over blocks of BLK splits (8, 16 or 32, the smallest that covers the launch's split count): everything a block needs (maxima, sums, partial rows) is requested before any of
+    // it is used, so the workgroup pays one memory latency per block instead of one per dependent step; across blocks
+    // the reference point moves as in the online softmax.  Within a block and across blocks the sums run over the
+    // splits in ascending order: the result does not depend on anything but the inputs.
+    float M = -INFINITY, o = 0.f, l = 0.f;
     const float* po = ws_o + row0 * D + (d < D ? d : 0);
-    int s = 0;
-    for (; s + 4 <= ns; s += 4) {  // four independent loads in flight; the sums keep a fixed order
-        const float x0 = po[(int64_t)(s + 0) * D], x1 = po[(int64_t)(s + 1) * D];
-        const float x2 = po[(int64_t)(s + 2) * D], x3 = po[(int64_t)(s + 3) * D];
-        const float w0 = exp2f(ws_ml[(row0 + s + 0) * 2] - M), w1 = exp2f(ws_ml[(row0 + s + 1) * 2] - M);
-        const float w2 = exp2f(ws_ml[(row0 + s + 2) * 2] - M), w3 = exp2f(ws_ml[(row0 + s + 3) * 2] - M);
-        l += w0 * ws_ml[(row0 + s + 0) * 2 + 1];
-        l += w1 * ws_ml[(row0 + s + 1) * 2 + 1];
-        l += w2 * ws_ml[(row0 + s + 2) * 2 + 1];
-        l += w3 * ws_ml[(row0 + s + 3) * 2 + 1];
-        o += w0 * x0;
-        o += w1 * x1;
-        o += w2 * x2;
-        o += w3 * x3;
-    }
-    for (; s < ns; ++s) {
-        const float w = exp2f(ws_ml[(row0 + s) * 2] - M);
-        l += w * ws_ml[(row0 + s) * 2 + 1];
-        o += w * po[(int64_t)s * D];
+    for (int s0 = 0; s0 < ns; s0 += BLK) {
+        float x[BLK], ms[BLK], ls[BLK];
+#pragma unroll
+        for (int i = 0; i < BLK; ++i) {
+            const int64_t si = min(s0 + i, ns - 1);
+            x[i] = po[si * D];
+            ms[i] = ws_ml[(row0 + si) * 2];
+            ls[i] = ws_ml[(row0 + si) * 2 + 1];
+        }
+        float Mb = M;
+#pragma unroll
+        for (int i = 0; i < BLK; ++i) Mb = fmaxf(Mb, ms[i]);   // indices past the end repeat the last split: harmless in a maximum
+        const float keep = exp2f(M - Mb);                      // 0 for the first block (M = -inf, Mb finite)
+        o *= keep;
+        l *= keep;
+        M = Mb;
+#pragma unroll
+        for (int i = 0; i < BLK; ++i)
+            if (s0 + i < ns) {
+                const float w = exp2f(ms[i] - M);
+                l += w * ls[i];
+                o += w * x[i];
+            }
     }
     if (d < D) {
         const float r = ns > 0 ? o / l : 0.f;
@@ -1187,14 +1193,19 @@ int decode_impl(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* s
     // with max_len == 0 every row is empty: the combine kernel reads nothing and writes zeros
     dim3 cgrid((unsigned)Hq, (unsigned)B);
     const int cthreads = D <= 64 ? 64 : (D <= 128 ? 128 : 256);
-    if (out->dtype == VSP_F32)
-        hipLaunchKernelGGL(decode_combine_kernel<float>, cgrid, dim3(cthreads), 0, st, a.ws_o, a.ws_ml, seq_lens,
-                           max_len > 0 ? cache->len : 0, chunk, max_splits, (int)Hq, (int)D, (float*)out->data,
-                           out->stride[0], out->stride[1], a.L_cap);
-    else
-        hipLaunchKernelGGL(decode_combine_kernel<uint16_t>, cgrid, dim3(cthreads), 0, st, a.ws_o, a.ws_ml, seq_lens,
-                           max_len > 0 ? cache->len : 0, chunk, max_splits, (int)Hq, (int)D, (uint16_t*)out->data,
-                           out->stride[0], out->stride[1], a.L_cap);
+    auto combine = [&](auto out_tag, auto blk) {
+        using OutT = decltype(out_tag);
+        hipLaunchKernelGGL((decode_combine_kernel<OutT, decltype(blk)::value>), cgrid, dim3(cthreads), 0, st, a.ws_o, a.ws_ml, seq_lens,
+                           max_len > 0 ? cache->len : 0, chunk, max_splits, (int)Hq, (int)D, (OutT*)out->data, out->stride[0],
+                           out->stride[1], a.L_cap);
+    };
+    auto combine_blk = [&](auto out_tag) {
+        if (max_splits <= 8) combine(out_tag, std::integral_constant<int, 8>{});
+        else if (max_splits <= 16) combine(out_tag, std::integral_constant<int, 16>{});
+        else combine(out_tag, std::integral_constant<int, 32>{});
+    };
+    if (out->dtype == VSP_F32) combine_blk(float{});
+    else combine_blk(uint16_t{});
     return check_launch();
 }
 
