@@ -140,9 +140,11 @@ __global__ void __launch_bounds__(256, 2) decode_bf16_kernel(DecodeArgs a) {
     constexpr int KS = D / 32;   // MFMA k-steps over the head dim
     constexpr int DB = D / 16;   // 16-row tiles of O^T
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int kvh = blockIdx.y;
+    // kv head fastest: every item that exists comes before the first surplus workgroup of the grid (which is sized for
+    // the longest possible batch), so the surplus ones start, find nothing and exit under the tail of the real work
+    const int kvh = blockIdx.x % a.Hkv;
     int b, split, L;
-    if (!locate_work(a, blockIdx.x, lane, b, split, L)) return;
+    if (!locate_work(a, blockIdx.x / a.Hkv, lane, b, split, L)) return;
     const int chunk_start = split * a.chunk;
     const int chunk_end = min(L, chunk_start + a.chunk);
 
@@ -311,9 +313,11 @@ __global__ void __launch_bounds__(256, 2) decode_q8_kernel(DecodeArgs a) {
     constexpr int NH = D / 64;  // 16-byte K loads per row per lane
     constexpr int NQ = D / kQBlock;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int kvh = blockIdx.y;
+    // kv head fastest: every item that exists comes before the first surplus workgroup of the grid (which is sized for
+    // the longest possible batch), so the surplus ones start, find nothing and exit under the tail of the real work
+    const int kvh = blockIdx.x % a.Hkv;
     int b, split, L;
-    if (!locate_work(a, blockIdx.x, lane, b, split, L)) return;
+    if (!locate_work(a, blockIdx.x / a.Hkv, lane, b, split, L)) return;
     const int chunk_start = split * a.chunk;
     const int chunk_end = min(L, chunk_start + a.chunk);
 
@@ -636,9 +640,11 @@ __global__ void __launch_bounds__(256, 2) decode_f32_mfma_kernel(DecodeArgs a) {
     constexpr int KT = 2;       // 16-key tiles per wavefront iteration
     constexpr int GROUP = 16 * KT;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int kvh = blockIdx.y;
+    // kv head fastest: every item that exists comes before the first surplus workgroup of the grid (which is sized for
+    // the longest possible batch), so the surplus ones start, find nothing and exit under the tail of the real work
+    const int kvh = blockIdx.x % a.Hkv;
     int b, split, L;
-    if (!locate_work(a, blockIdx.x, lane, b, split, L)) return;
+    if (!locate_work(a, blockIdx.x / a.Hkv, lane, b, split, L)) return;
     const int chunk_start = split * a.chunk;
     const int chunk_end = min(L, chunk_start + a.chunk);
     const int c = lane & 15, g = lane >> 4;
@@ -1157,7 +1163,7 @@ int decode_impl(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* s
 
     if (max_len > 0) {
         if (cache->format == VSP_KV_BF16) {
-            dim3 grid((unsigned)(max_splits * B), cache->Hkv);
+            dim3 grid((unsigned)(max_splits * B * cache->Hkv));
             if (cache->page_table) {
                 if (D == 128) hipLaunchKernelGGL((decode_bf16_kernel<128, true>), grid, dim3(256), 0, st, a);
                 else hipLaunchKernelGGL((decode_bf16_kernel<64, true>), grid, dim3(256), 0, st, a);
@@ -1166,7 +1172,7 @@ int decode_impl(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* s
                 else hipLaunchKernelGGL((decode_bf16_kernel<64, false>), grid, dim3(256), 0, st, a);
             }
         } else if (cache->format == VSP_KV_Q8_0) {
-            dim3 grid((unsigned)(max_splits * B), cache->Hkv);
+            dim3 grid((unsigned)(max_splits * B * cache->Hkv));
             if (cache->page_table) {
                 if (D == 128) hipLaunchKernelGGL((decode_q8_kernel<128, true>), grid, dim3(256), 0, st, a);
                 else hipLaunchKernelGGL((decode_q8_kernel<64, true>), grid, dim3(256), 0, st, a);
@@ -1175,7 +1181,7 @@ int decode_impl(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* s
                 else hipLaunchKernelGGL((decode_q8_kernel<64, false>), grid, dim3(256), 0, st, a);
             }
         } else if ((D == 64 || D == 128) && n_rep <= 16) {
-            dim3 grid((unsigned)(max_splits * B), cache->Hkv);
+            dim3 grid((unsigned)(max_splits * B * cache->Hkv));
             if (D == 128) hipLaunchKernelGGL((decode_f32_mfma_kernel<128>), grid, dim3(256), 0, st, a);
             else hipLaunchKernelGGL((decode_f32_mfma_kernel<64>), grid, dim3(256), 0, st, a);
         } else {
