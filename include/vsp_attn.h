@@ -290,6 +290,19 @@ size_t vsp_attn_decode_workspace_bytes(int32_t B, int32_t Hq, int32_t D, int32_t
 int vsp_attn_decode(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, int32_t max_len,
                     vsp_tensor* out, float scale, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The decode step for a few tokens per sequence at once (the last T tokens of each context, already appended:
+ * speculative-decoding verification, multi-token prediction): what GroupedQueryAttention::forward(x, cache,
+ * start_pos) would compute for T > 1 and start_pos > 0 if its mask broadcast (src/nn/gqa_attention.cpp:128-148; the
+ * reference throws there), i.e. the rows vsp_attn_prefill_cached returns, at the decode kernels' rate.  q, out
+ * [B,Hq,T,D]: token t of sequence b sits at position L_b - T + t and attends keys [0, L_b - T + t].  The T tokens and the
+ * Hq/Hkv query heads of a kv head share the 16 columns of the matrix instructions, so K and V are still read once per kv
+ * head: T * Hq/Hkv <= 16 and D in {64, 128}, else VSP_ERR_UNSUPPORTED (use vsp_attn_prefill_cached).  T == 1 is
+ * vsp_attn_decode, bit for bit.  Everything else as vsp_attn_decode; workspace >=
+ * vsp_attn_decode_workspace_bytes(B * T, Hq, D, max_len).  A token placed before the start of its context
+ * (L_b < T - t) gets zeros. */
+int vsp_attn_decode_multi(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, int32_t max_len,
+                          vsp_tensor* out, float scale, void* workspace, size_t workspace_bytes, void* stream);
+
 /* vsp_attn_decode for callers that cannot allocate device memory (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments,
  * validation, kernels and results (bit for bit) as vsp_attn_decode, minus the workspace: the split-K

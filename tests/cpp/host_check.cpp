@@ -257,6 +257,19 @@ static void test_validation() {
     big.B = 64, big.Hkv = 8, big.S_max = 65536, big.D = 128, big.len = 65536;
     vsp_tensor bq = tensor4(mem, VSP_BF16, 64, 128, 1, 128);
     CHECK(vsp_attn_decode_noalloc(&bq, &big, nullptr, 0, &bq, 0.1f, nullptr) == VSP_ERR_WORKSPACE);
+    // several tokens per sequence through the decode kernels: tokens x heads per kv head <= 16, head_dim 64 / 128
+    {
+        vsp_tensor q4 = tensor4(mem, VSP_BF16, 1, 4, 4, 64), q9 = tensor4(mem, VSP_BF16, 1, 4, 9, 64);
+        const int32_t keep_len = c.len;
+        c.len = 8;
+        CHECK(vsp_attn_decode(&q4, &c, nullptr, 0, &q4, 0.1f, mem, 1 << 16, nullptr) == VSP_ERR_SHAPE);        // the plain step: T == 1
+        CHECK(vsp_attn_decode_multi(&q9, &c, nullptr, 0, &q9, 0.1f, mem, 1 << 16, nullptr) == VSP_ERR_UNSUPPORTED);   // 2 x 9 columns
+        CHECK(vsp_attn_decode_multi(&q4, &c, nullptr, 0, &q4, 0.1f, nullptr, 0, nullptr) == VSP_ERR_WORKSPACE);
+        vsp_tensor q4s = q4;
+        q4s.stride[2] = 68;   // token rows must stay 16-byte aligned
+        CHECK(vsp_attn_decode_multi(&q4s, &c, nullptr, 0, &q4, 0.1f, mem, 1 << 16, nullptr) == VSP_ERR_ALIGN);
+        c.len = keep_len;
+    }
     // backward
     vsp_tensor lse{};
     lse.data = mem, lse.dtype = VSP_F32, lse.ndim = 3, lse.shape[0] = 1, lse.shape[1] = 4, lse.shape[2] = 8;

@@ -26,6 +26,8 @@ BLOCKS = [
      f"{_T} q_view, {_T} k_view, {_T} v_view, {_T} q_rot, vsp_kv_cache cache_desc, int64_t start_pos, void* stream"),
     ("chunked prefill over the cache", "function",
      "vsp_tensor dq_rot, vsp_tensor dout, vsp_kv_cache cache_desc, int D, void* workspace, void* stream"),
+    ("a few tokens per sequence through the decode kernels", "function",
+     "vsp_tensor dq_rot, vsp_tensor dout, vsp_kv_cache cache_desc, int32_t B, int32_t T, int32_t Hq, int D, void* workspace, void* stream"),
     ("flash_attention_backward_hip_dispatch", "global", ""),
     ("the same body for fp32 tensors with split operands", "function",
      f"{_T} q, {_T} k, vsp_tensor d_dout, vsp_tensor dq_, vsp_tensor dk_, vsp_tensor dv_, vsp_tensor d_out, vsp_tensor d_lse, "

@@ -56,6 +56,7 @@ SYMBOLS = {
     "vsp_seq_lens_advance": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p]),
     "vsp_attn_decode_workspace_bytes": (C.c_size_t, [C.c_int32] * 4),
     "vsp_attn_decode": (C.c_int, [_TP, _KP, C.c_void_p, C.c_int32, _TP, C.c_float, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "vsp_attn_decode_multi": (C.c_int, [_TP, _KP, C.c_void_p, C.c_int32, _TP, C.c_float, C.c_void_p, C.c_size_t, C.c_void_p]),
     "vsp_attn_decode_noalloc": (C.c_int, [_TP, _KP, C.c_void_p, C.c_int32, _TP, C.c_float, C.c_void_p]),
     "vsp_attn_decode_proj_workspace_bytes": (C.c_size_t, [C.c_int32] * 5),
     "vsp_attn_decode_proj": (C.c_int, [_TP, _KP, C.c_void_p, C.c_int32, _TP, _TP, _TP, C.c_float, C.c_void_p, C.c_size_t,

@@ -312,6 +312,25 @@ def decode_attention(q, cache, seq_lens=None, max_len=0, scale=None, out=None, w
     return out
 
 
+def decode_attention_multi(q, cache, seq_lens=None, max_len=0, scale=None, out=None, workspace=None):
+    """The last T tokens of each sequence (already appended) attending to the cache at the decode kernels' rate:
+    q [B,Hq,T,D] -> [B,Hq,T,D], token t sees keys [0, L_b - T + t]; T * Hq/Hkv <= 16 (vsp_attn_decode_multi)."""
+    c = cache._c
+    if scale is None:
+        scale = 1.0 / math.sqrt(q.shape[-1])
+    if out is None:
+        out = torch.empty_like(q)
+    if workspace is None:
+        bound = max_len or (c.S_max if seq_lens is not None else c.len)
+        nbytes = lib.vsp_attn_decode_workspace_bytes(q.shape[0] * q.shape[2], q.shape[1], q.shape[3], max(int(bound), 1))
+        workspace = _workspace(q.device, nbytes)
+    dq, do = _desc(q), _desc(out)
+    sl = C.c_void_p(seq_lens.data_ptr()) if seq_lens is not None else None
+    check(lib.vsp_attn_decode_multi(C.byref(dq), C.byref(c), sl, int(max_len), C.byref(do), float(scale),
+                                    C.c_void_p(workspace.data_ptr()), workspace.numel(), _stream(q)))
+    return out
+
+
 def decode_attention_proj(q, cache, wo, bias=None, seq_lens=None, max_len=0, scale=None, out=None, workspace=None):
     """decode_attention followed by the module's output projection (src/nn/gqa_attention.cpp:151-152, Linear::forward
     src/nn/linear.cpp:41-49) in one call: q [B,Hq,1,D], wo [N, Hq*D], bias [N] or None -> y [B,1,N]."""

@@ -330,9 +330,22 @@ public:
     // Chunked prefill: attention of the LAST T tokens of the context (q [B,Hq,T,D], already appended to the cache)
     // with K/V read in place from the planes.  The reference's scaled_dot_product_attention throws for a causal
     // T != L (src/nn/functional.cpp:406-410); the rows returned are [len-T, len) of its full causal forward.
+    // A causal chunk of a few tokens (T * query heads per kv head <= 16: speculative verification, multi-token
+    // prediction) takes the split-K decode kernels instead (vsp_attn_decode_multi): K and V read once per kv head at the
+    // HBM rate, the context split over the chip, where the prefill kernel would walk it with one wavefront per query head.
     Tensor attend(const Tensor& q, bool is_causal = true) const {
         Tensor out = empty(q.shape(), q.dtype());
         vsp_tensor dq = q.desc(), dout = out.desc();
+        const int64_t T = q.ndim() == 4 ? q.shape()[2] : 0, D = q.ndim() == 4 ? q.shape()[3] : 0;
+        if (is_causal && T > 1 && st_->c.Hkv > 0 && q.shape()[1] % st_->c.Hkv == 0 && T * (q.shape()[1] / st_->c.Hkv) <= 16 &&
+            (D == 64 || D == 128) && (int64_t)st_->c.len >= T) {
+            const float sc = 1.0f / std::sqrt(static_cast<float>(D));
+            const size_t nb = vsp_attn_decode_workspace_bytes((int32_t)(q.shape()[0] * T), (int32_t)q.shape()[1], (int32_t)D,
+                                                              (int32_t)st_->c.len);
+            Storage ws(nb ? nb : 16);
+            throw_status(vsp_attn_decode_multi(&dq, &st_->c, nullptr, 0, &dout, sc, ws.data(), nb, current_stream()));
+            return out;
+        }
         const size_t ws_bytes = vsp_attn_prefill_cached_workspace_bytes(&st_->c, 0);
         std::shared_ptr<Storage> ws = ws_bytes ? std::make_shared<Storage>(ws_bytes) : nullptr;
         const float scale = 1.0f / std::sqrt(static_cast<float>(q.shape()[3]));

@@ -31,7 +31,8 @@ constexpr int kGroup = 64;  // keys per wave iteration
 
 struct DecodeArgs {
     const void* q;
-    int64_t sq_b, sq_h;  // q strides (elements) of dims 0, 1
+    int64_t sq_b, sq_h, sq_t;  // q strides (elements) of dims 0, 1, 2
+    int32_t T;                 // query tokens per sequence: token t sits at position L - T + t and sees the keys up to itself
     const void* k;
     const void* v;
     const void* k_scale;
@@ -46,8 +47,8 @@ struct DecodeArgs {
     int32_t chunk;
     int32_t max_splits;
     float scale_log2;  // scale * log2(e)
-    float* ws_o;       // [B][Hq][max_splits][D]
-    float* ws_ml;      // [B][Hq][max_splits][2]  (m in log2 domain, l)
+    float* ws_o;       // [B][Hq][T][max_splits][D]
+    float* ws_ml;      // [B][Hq][T][max_splits][2]  (m in log2 domain, l)
     // paged cache: sequence b's 64-key group starting at token t lives in page page_table[b * pages_per_seq +
     // t / page_tokens] (page_tokens is a multiple of 64, so a group never straddles two pages); S is then the
     // page size.  nullptr for a contiguous cache.
@@ -78,6 +79,25 @@ __device__ inline float wave_sum_over_groups(float x) {
     x += __shfl_xor(x, 16);
     x += __shfl_xor(x, 32);
     return x;
+}
+
+// The 16 MFMA columns of a work item are the (token, query head of the kv head) pairs of the call, token-major:
+// column c = t * n_rep + r.  With one token per sequence (the plain decode step) a column is a query head.
+struct Column {
+    int t, r;
+    bool live;
+};
+__device__ inline Column column_of(const DecodeArgs& a, int c) {
+    const int n = a.n_rep * a.T, cc = min(c, n - 1);
+    return Column{cc / a.n_rep, cc % a.n_rep, c < n};
+}
+// Keys [0, limit) are visible to column col: token t of T sits at position L - T + t and attends up to itself.
+__device__ inline int column_limit(const DecodeArgs& a, const Column& col, int L, int chunk_end) {
+    return min(chunk_end, L - (a.T - 1 - col.t));
+}
+// Row of the split-K partials that column col of (batch row b, kv head) writes for `split`.
+__device__ inline int64_t partial_row(const DecodeArgs& a, int b, int kvh, const Column& col, int split) {
+    return (((int64_t)b * a.Hq + kvh * a.n_rep + col.r) * a.T + col.t) * a.max_splits + split;
 }
 
 __device__ inline uint4 mask_tail_u16x8(uint4 v, int nvalid) {
@@ -150,14 +170,16 @@ __global__ void __launch_bounds__(256, 2) decode_bf16_kernel(DecodeArgs a) {
 
     const int c = lane & 15, g = lane >> 4;
 
-    // Q^T operands: column c = query head kvh*n_rep + c (zero beyond n_rep)
+    // Q^T operands: column c = (token, query head of this kv head), zero beyond the last one
+    const Column col = column_of(a, c);
+    const int lim = column_limit(a, col, L, chunk_end);
     bf16x8_t qf[KS];
     {
-        const uint16_t* qrow = (const uint16_t*)a.q + (int64_t)b * a.sq_b + (int64_t)(kvh * a.n_rep + min(c, a.n_rep - 1)) * a.sq_h;
+        const uint16_t* qrow = (const uint16_t*)a.q + (int64_t)b * a.sq_b + (int64_t)(kvh * a.n_rep + col.r) * a.sq_h + (int64_t)col.t * a.sq_t;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             uint4 w = *(const uint4*)(qrow + 32 * ks + 8 * g);
-            if (c >= a.n_rep) w = uint4{0, 0, 0, 0};
+            if (!col.live) w = uint4{0, 0, 0, 0};
             qf[ks] = __builtin_bit_cast(bf16x8_t, w);
         }
     }
@@ -210,26 +232,30 @@ __global__ void __launch_bounds__(256, 2) decode_bf16_kernel(DecodeArgs a) {
                 s[jj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kf[jj][ks]), qf[ks], s[jj], 0, 0, 0);
         }
         if (knext < chunk_end) load_k(knext);
-        const bool tail = kbase + kGroup > chunk_end;
+        const bool tail = kbase + kGroup > chunk_end;               // keys past the end of the split: stale rows of the planes
+        const bool tail_s = kbase + kGroup > chunk_end - (a.T - 1);  // keys past some column's limit
         float mloc = -INFINITY;
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj)
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 float t = s[jj][v] * a.scale_log2;
-                if (tail && kbase + 16 * g + 4 * jj + v >= chunk_end) t = -INFINITY;
+                if (tail_s && kbase + 16 * g + 4 * jj + v >= lim) t = -INFINITY;
                 s[jj][v] = t;
                 mloc = fmaxf(mloc, t);
             }
         mloc = wave_max_over_groups(mloc);
-        const float m_new = fmaxf(m, mloc);  // finite: the group holds at least one valid key
-        const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+        const float m_new = fmaxf(m, mloc);
+        // -inf while a column has seen no key yet (several tokens per sequence: the last keys of a context lie past the
+        // earlier tokens' limits); its sums then stay zero
+        const float m_ref = m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m - m_ref);
         float lsum = 0.f;
         uint32_t pw[2][4];
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj) {
-            float p0 = __builtin_amdgcn_exp2f(s[jj][0] - m_new), p1 = __builtin_amdgcn_exp2f(s[jj][1] - m_new);
-            float p2 = __builtin_amdgcn_exp2f(s[jj][2] - m_new), p3 = __builtin_amdgcn_exp2f(s[jj][3] - m_new);
+            float p0 = __builtin_amdgcn_exp2f(s[jj][0] - m_ref), p1 = __builtin_amdgcn_exp2f(s[jj][1] - m_ref);
+            float p2 = __builtin_amdgcn_exp2f(s[jj][2] - m_ref), p3 = __builtin_amdgcn_exp2f(s[jj][3] - m_ref);
             lsum += (p0 + p1) + (p2 + p3);
             pw[jj >> 1][2 * (jj & 1)] = pack_bf16x2(p0, p1);
             pw[jj >> 1][2 * (jj & 1) + 1] = pack_bf16x2(p2, p3);
@@ -259,7 +285,7 @@ __global__ void __launch_bounds__(256, 2) decode_bf16_kernel(DecodeArgs a) {
     // ---- combine the four wavefronts through LDS, write one partial per (b, head, split)
     __shared__ float sm_o[kWaves][16][D + 4];
     __shared__ float sm_m[kWaves][16], sm_l[kWaves][16];
-    if (c < a.n_rep) {
+    if (col.live) {
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -270,19 +296,20 @@ __global__ void __launch_bounds__(256, 2) decode_bf16_kernel(DecodeArgs a) {
         }
     }
     __syncthreads();
-    for (int i = tid; i < a.n_rep * D; i += 256) {
+    for (int i = tid; i < a.n_rep * a.T * D; i += 256) {
         const int hc = i / D, d = i % D;
         float mm = sm_m[0][hc];
 #pragma unroll
         for (int w = 1; w < kWaves; ++w) mm = fmaxf(mm, sm_m[w][hc]);
+        const float mm_ref = mm == -INFINITY ? 0.f : mm;   // a column without a key in this split: zero sums, m = -inf
         float o = 0.f, ll = 0.f;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) {
-            const float f = __builtin_amdgcn_exp2f(sm_m[w][hc] - mm);
+            const float f = __builtin_amdgcn_exp2f(sm_m[w][hc] - mm_ref);
             o += f * sm_o[w][hc][d];
             ll += f * sm_l[w][hc];
         }
-        const int64_t row = ((int64_t)b * a.Hq + kvh * a.n_rep + hc) * a.max_splits + split;
+        const int64_t row = partial_row(a, b, kvh, column_of(a, hc), split);
         a.ws_o[row * D + d] = o;
         if (d == 0) {
             a.ws_ml[row * 2] = mm;
@@ -325,9 +352,11 @@ __global__ void __launch_bounds__(256, 2) decode_q8_kernel(DecodeArgs a) {
 
     // Q^T operands in fp16.  Contraction slot (ks, g, e) is head-dim index
     // 64*(ks/2) + 16*g + 8*(ks%2) + e, so that one 16-byte K load (16 int8) feeds two k-steps.
+    const Column col = column_of(a, c);
+    const int lim = column_limit(a, col, L, chunk_end);
     f16x8_t qf[KS];
     {
-        const uint16_t* qrow = (const uint16_t*)a.q + (int64_t)b * a.sq_b + (int64_t)(kvh * a.n_rep + min(c, a.n_rep - 1)) * a.sq_h;
+        const uint16_t* qrow = (const uint16_t*)a.q + (int64_t)b * a.sq_b + (int64_t)(kvh * a.n_rep + col.r) * a.sq_h + (int64_t)col.t * a.sq_t;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             uint4 w = *(const uint4*)(qrow + 64 * (ks >> 1) + 16 * g + 8 * (ks & 1));
@@ -337,7 +366,7 @@ __global__ void __launch_bounds__(256, 2) decode_q8_kernel(DecodeArgs a) {
                 float lo = bf16_bits_to_f32((uint16_t)(ww[i] & 0xFFFFu)), hi = bf16_bits_to_f32((uint16_t)(ww[i] >> 16));
                 lo = fminf(fmaxf(lo, -65504.f), 65504.f);
                 hi = fminf(fmaxf(hi, -65504.f), 65504.f);
-                if (c >= a.n_rep) lo = hi = 0.f;
+                if (!col.live) lo = hi = 0.f;
                 qf[ks][2 * i] = (_Float16)lo;
                 qf[ks][2 * i + 1] = (_Float16)hi;
             }
@@ -392,6 +421,7 @@ __global__ void __launch_bounds__(256, 2) decode_q8_kernel(DecodeArgs a) {
     }
     for (int kbase = kfirst; kbase < chunk_end; kbase += kWaves * kGroup) {
         const bool tail = kbase + kGroup > chunk_end;
+        const bool tail_s = kbase + kGroup > chunk_end - (a.T - 1);
         const int knext = kbase + kWaves * kGroup;
         // ---- S^T
         f32x4_t s[4];
@@ -424,20 +454,21 @@ __global__ void __launch_bounds__(256, 2) decode_q8_kernel(DecodeArgs a) {
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 float t = s[jj][v] * a.scale_log2;
-                if (tail && kbase + 16 * g + 4 * jj + v >= chunk_end) t = -INFINITY;
+                if (tail_s && kbase + 16 * g + 4 * jj + v >= lim) t = -INFINITY;
                 s[jj][v] = t;
                 mloc = fmaxf(mloc, t);
             }
         mloc = wave_max_over_groups(mloc);
         const float m_new = fmaxf(m, mloc);
-        const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+        const float m_ref = m_new == -INFINITY ? 0.f : m_new;   // see decode_bf16_kernel
+        const float alpha = __builtin_amdgcn_exp2f(m - m_ref);
         float lsum = 0.f;
         f16x8_t pf[2];
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj)
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
-                const float p = __builtin_amdgcn_exp2f(s[jj][v] - m_new);
+                const float p = __builtin_amdgcn_exp2f(s[jj][v] - m_ref);
                 lsum += p;
                 pf[jj >> 1][4 * (jj & 1) + v] = (_Float16)p;
             }
@@ -473,7 +504,7 @@ __global__ void __launch_bounds__(256, 2) decode_q8_kernel(DecodeArgs a) {
 
     __shared__ float sm_o[kWaves][16][D + 4];
     __shared__ float sm_m[kWaves][16], sm_l[kWaves][16];
-    if (c < a.n_rep) {
+    if (col.live) {
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -484,19 +515,20 @@ __global__ void __launch_bounds__(256, 2) decode_q8_kernel(DecodeArgs a) {
         }
     }
     __syncthreads();
-    for (int i = tid; i < a.n_rep * D; i += 256) {
+    for (int i = tid; i < a.n_rep * a.T * D; i += 256) {
         const int hc = i / D, d = i % D;
         float mm = sm_m[0][hc];
 #pragma unroll
         for (int w = 1; w < kWaves; ++w) mm = fmaxf(mm, sm_m[w][hc]);
+        const float mm_ref = mm == -INFINITY ? 0.f : mm;   // a column without a key in this split: zero sums, m = -inf
         float o = 0.f, ll = 0.f;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) {
-            const float f = __builtin_amdgcn_exp2f(sm_m[w][hc] - mm);
+            const float f = __builtin_amdgcn_exp2f(sm_m[w][hc] - mm_ref);
             o += f * sm_o[w][hc][d];
             ll += f * sm_l[w][hc];
         }
-        const int64_t row = ((int64_t)b * a.Hq + kvh * a.n_rep + hc) * a.max_splits + split;
+        const int64_t row = partial_row(a, b, kvh, column_of(a, hc), split);
         a.ws_o[row * D + d] = o;
         if (d == 0) {
             a.ws_ml[row * 2] = mm;
@@ -649,13 +681,15 @@ __global__ void __launch_bounds__(256, 2) decode_f32_mfma_kernel(DecodeArgs a) {
     const int chunk_end = min(L, chunk_start + a.chunk);
     const int c = lane & 15, g = lane >> 4;
 
+    const Column col = column_of(a, c);
+    const int lim = column_limit(a, col, L, chunk_end);
     float qf[C4][4];
     {
-        const float* qrow = (const float*)a.q + (int64_t)b * a.sq_b + (int64_t)(kvh * a.n_rep + min(c, a.n_rep - 1)) * a.sq_h;
+        const float* qrow = (const float*)a.q + (int64_t)b * a.sq_b + (int64_t)(kvh * a.n_rep + col.r) * a.sq_h + (int64_t)col.t * a.sq_t;
 #pragma unroll
         for (int cc = 0; cc < C4; ++cc) {
             const float4 w = *(const float4*)(qrow + 16 * cc + 4 * g);
-            const float f = c < a.n_rep ? a.scale_log2 : 0.f;
+            const float f = col.live ? a.scale_log2 : 0.f;
             qf[cc][0] = w.x * f, qf[cc][1] = w.y * f, qf[cc][2] = w.z * f, qf[cc][3] = w.w * f;
         }
     }
@@ -709,26 +743,27 @@ __global__ void __launch_bounds__(256, 2) decode_f32_mfma_kernel(DecodeArgs a) {
             }
         }
         if (knext < chunk_end) load_k(knext);
-        const bool tail = kbase + GROUP > chunk_end;
+        const bool tail_s = kbase + GROUP > chunk_end - (a.T - 1);
         float mloc = -INFINITY;
 #pragma unroll
         for (int t = 0; t < KT; ++t)
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 float x = s[t][v];
-                if (tail && kbase + 16 * t + 4 * g + v >= chunk_end) x = -INFINITY;
+                if (tail_s && kbase + 16 * t + 4 * g + v >= lim) x = -INFINITY;
                 s[t][v] = x;
                 mloc = fmaxf(mloc, x);
             }
         mloc = wave_max_over_groups(mloc);
-        const float m_new = fmaxf(m, mloc);  // finite: the group holds at least one valid key
-        const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+        const float m_new = fmaxf(m, mloc);
+        const float m_ref = m_new == -INFINITY ? 0.f : m_new;   // see decode_bf16_kernel
+        const float alpha = __builtin_amdgcn_exp2f(m - m_ref);
         float lsum = 0.f;
 #pragma unroll
         for (int t = 0; t < KT; ++t)
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
-                s[t][v] = __builtin_amdgcn_exp2f(s[t][v] - m_new);
+                s[t][v] = __builtin_amdgcn_exp2f(s[t][v] - m_ref);
                 lsum += s[t][v];
             }
         l = l * alpha + lsum;
@@ -754,7 +789,7 @@ __global__ void __launch_bounds__(256, 2) decode_f32_mfma_kernel(DecodeArgs a) {
     // ---- combine the four wavefronts through LDS, write one partial per (b, head, split)
     __shared__ float sm_o[kWaves][16][D + 4];
     __shared__ float sm_m[kWaves][16], sm_l[kWaves][16];
-    if (c < a.n_rep) {
+    if (col.live) {
 #pragma unroll
         for (int vc = 0; vc < VC; ++vc)
 #pragma unroll
@@ -767,7 +802,7 @@ __global__ void __launch_bounds__(256, 2) decode_f32_mfma_kernel(DecodeArgs a) {
         }
     }
     __syncthreads();
-    for (int i = tid; i < a.n_rep * D; i += 256) {
+    for (int i = tid; i < a.n_rep * a.T * D; i += 256) {
         const int hc = i / D, d = i % D;
         float mm = sm_m[0][hc];
 #pragma unroll
@@ -775,12 +810,12 @@ __global__ void __launch_bounds__(256, 2) decode_f32_mfma_kernel(DecodeArgs a) {
         float o = 0.f, ll = 0.f;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) {
-            // a wavefront that saw no key of a short split carries m = -inf, l = 0 and zero sums
+            // a wavefront that saw no key of a short split, or a column with no key in it, carries m = -inf, l = 0 and zero sums
             const float f = sm_m[w][hc] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(sm_m[w][hc] - mm);
             o += f * sm_o[w][hc][d];
             ll += f * sm_l[w][hc];
         }
-        const int64_t row = ((int64_t)b * a.Hq + kvh * a.n_rep + hc) * a.max_splits + split;
+        const int64_t row = partial_row(a, b, kvh, column_of(a, hc), split);
         a.ws_o[row * D + d] = o;
         if (d == 0) {
             a.ws_ml[row * 2] = mm;
@@ -796,11 +831,11 @@ template <typename OutT, int BLK>
 __global__ void __launch_bounds__(256) decode_combine_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
                                                              const int32_t* __restrict__ seq_lens, int32_t len, int32_t chunk,
                                                              int32_t max_splits, int32_t Hq, int32_t D, OutT* __restrict__ out,
-                                                             int64_t so_b, int64_t so_h, int32_t L_cap) {
-    const int hq = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+                                                             int64_t so_b, int64_t so_h, int32_t L_cap, int32_t T, int64_t so_t) {
+    const int hq = blockIdx.x / T, t = blockIdx.x % T, b = blockIdx.y, d = threadIdx.x;
     const int L = min(max(seq_lens ? seq_lens[b] : len, 0), L_cap);  // the producers' clamp (locate_work)
     const int ns = min((L + chunk - 1) / chunk, max_splits);
-    const int64_t row0 = ((int64_t)b * Hq + hq) * max_splits;
+    const int64_t row0 = (((int64_t)b * Hq + hq) * T + t) * max_splits;
     // One pass over blocks of BLK splits (8, 16 or 32, the smallest that covers the launch's split count): everything a block needs (maxima, sums, partial rows) is requested before any of
     // it is used, so the workgroup pays one memory latency per block instead of one per dependent step; across blocks
     // the reference point moves as in the online softmax.  Within a block and across blocks the sums run over the
@@ -832,8 +867,8 @@ __global__ void __launch_bounds__(256) decode_combine_kernel(const float* __rest
             }
     }
     if (d < D) {
-        const float r = ns > 0 ? o / l : 0.f;
-        OutT* p = out + (int64_t)b * so_b + (int64_t)hq * so_h + d;
+        const float r = (ns > 0 && l > 0.f) ? o / l : 0.f;   // l = 0: a token placed before the start of its context
+        OutT* p = out + (int64_t)b * so_b + (int64_t)hq * so_h + (int64_t)t * so_t + d;
         if constexpr (sizeof(OutT) == 4) *p = r;
         else *p = f32_to_bf16_bits(r);
     }
@@ -1096,13 +1131,13 @@ int scratch_for_current_device(void** out) {
 // Both decode entry points: validation, split sizing and the two launches.  `own_scratch` selects the
 // library's fixed per-device array instead of a caller workspace.
 int decode_impl(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, int32_t max_len, vsp_tensor* out,
-                float scale, void* workspace, size_t workspace_bytes, bool own_scratch, void* stream) {
+                float scale, void* workspace, size_t workspace_bytes, bool own_scratch, void* stream, bool multi = false) {
     if (!q || !out) return VSP_ERR_NULL;
     int rc = check_kv_cache(cache);
     if (rc != VSP_OK) return rc;
     if (q->ndim != 4 || out->ndim != 4) return VSP_ERR_NDIM;
     const int64_t B = q->shape[0], Hq = q->shape[1], T = q->shape[2], D = q->shape[3];
-    if (T != 1 || B != cache->B || D != cache->D) return VSP_ERR_SHAPE;
+    if ((multi ? T < 1 : T != 1) || B != cache->B || D != cache->D) return VSP_ERR_SHAPE;
     for (int i = 0; i < 4; ++i)
         if (out->shape[i] != q->shape[i]) return VSP_ERR_SHAPE;
     if (cache->Hkv <= 0 || Hq <= 0 || Hq % cache->Hkv != 0) return VSP_ERR_GQA_HEADS;
@@ -1112,11 +1147,14 @@ int decode_impl(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* s
     if (q->dtype != want_dtype) return VSP_ERR_UNSUPPORTED;
     if (cache->format != VSP_KV_F32 && n_rep > 16) return VSP_ERR_UNSUPPORTED;
     if (cache->format == VSP_KV_F32 && D > 256) return VSP_ERR_UNSUPPORTED;
+    // several tokens per sequence: they and the query heads of a kv head share the 16 columns of the matrix instructions
+    if (T > 1 && (n_rep * T > 16 || (D != 64 && D != 128))) return VSP_ERR_UNSUPPORTED;
     if (B == 0) return VSP_OK;
     if (!q->data || !out->data) return VSP_ERR_NULL;
     if (q->stride[3] != 1 || out->stride[3] != 1) return VSP_ERR_STRIDE;
     const int esz = q->dtype == VSP_F32 ? 4 : 2;
-    if (!is_aligned16(q->data) || (q->stride[0] * esz) % 16 || (q->stride[1] * esz) % 16) return VSP_ERR_ALIGN;
+    if (!is_aligned16(q->data) || (q->stride[0] * esz) % 16 || (q->stride[1] * esz) % 16 || (T > 1 && (q->stride[2] * esz) % 16))
+        return VSP_ERR_ALIGN;
     if (max_len < 0 || max_len > cache->S_max) return VSP_ERR_ARG;
     // a host-side length above the bound the launch is sized from is a caller error; device-side lengths
     // cannot be read here and are clamped to the bound inside the kernels instead
@@ -1126,7 +1164,7 @@ int decode_impl(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* s
 
     const int chunk = max_len > 0 ? pick_chunk(cache->format, B, cache->Hkv, max_len) : 256;
     const int max_splits = max_len > 0 ? (int)ceil_div(max_len, chunk) : 1;
-    const size_t need = (size_t)(B * Hq * max_splits * (D + 2) * 4);
+    const size_t need = (size_t)(B * Hq * T * max_splits * (D + 2) * 4);
     if (own_scratch) {
         if (need > kScratchBytes) return VSP_ERR_WORKSPACE;
         rc = scratch_for_current_device(&workspace);
@@ -1139,6 +1177,8 @@ int decode_impl(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* s
     a.q = q->data;
     a.sq_b = q->stride[0];
     a.sq_h = q->stride[1];
+    a.sq_t = q->stride[2];
+    a.T = (int)T;
     a.k = cache->k;
     a.v = cache->v;
     a.k_scale = cache->k_scale;
@@ -1159,7 +1199,7 @@ int decode_impl(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* s
     a.max_splits = max_splits;
     a.scale_log2 = scale * kLog2e;
     a.ws_o = (float*)workspace;
-    a.ws_ml = a.ws_o ? a.ws_o + (size_t)B * Hq * max_splits * D : nullptr;
+    a.ws_ml = a.ws_o ? a.ws_o + (size_t)B * Hq * T * max_splits * D : nullptr;
 
     if (max_len > 0) {
         if (cache->format == VSP_KV_BF16) {
@@ -1197,13 +1237,13 @@ int decode_impl(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* s
         if (rc != VSP_OK) return rc;
     }
     // with max_len == 0 every row is empty: the combine kernel reads nothing and writes zeros
-    dim3 cgrid((unsigned)Hq, (unsigned)B);
+    dim3 cgrid((unsigned)(Hq * T), (unsigned)B);
     const int cthreads = D <= 64 ? 64 : (D <= 128 ? 128 : 256);
     auto combine = [&](auto out_tag, auto blk) {
         using OutT = decltype(out_tag);
         hipLaunchKernelGGL((decode_combine_kernel<OutT, decltype(blk)::value>), cgrid, dim3(cthreads), 0, st, a.ws_o, a.ws_ml, seq_lens,
                            max_len > 0 ? cache->len : 0, chunk, max_splits, (int)Hq, (int)D, (OutT*)out->data, out->stride[0],
-                           out->stride[1], a.L_cap);
+                           out->stride[1], a.L_cap, (int)T, out->stride[2]);
     };
     auto combine_blk = [&](auto out_tag) {
         if (max_splits <= 8) combine(out_tag, std::integral_constant<int, 8>{});
@@ -1241,6 +1281,11 @@ size_t vsp_attn_decode_workspace_bytes(int32_t B, int32_t Hq, int32_t D, int32_t
 int vsp_attn_decode(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, int32_t max_len,
                     vsp_tensor* out, float scale, void* workspace, size_t workspace_bytes, void* stream) {
     return decode_impl(q, cache, seq_lens, max_len, out, scale, workspace, workspace_bytes, false, stream);
+}
+
+int vsp_attn_decode_multi(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, int32_t max_len,
+                          vsp_tensor* out, float scale, void* workspace, size_t workspace_bytes, void* stream) {
+    return decode_impl(q, cache, seq_lens, max_len, out, scale, workspace, workspace_bytes, false, stream, true);
 }
 
 int vsp_attn_decode_noalloc(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, int32_t max_len,
