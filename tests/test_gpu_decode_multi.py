@@ -94,6 +94,35 @@ def test_ragged_lengths_and_strided_queries(va):
     assert torch.equal(out, va.decode_attention_multi(tq, poisoned, seq_lens=sl))
 
 
+@pytest.mark.parametrize("fmt", ["bf16", "q8_0"])
+def test_small_chunks_of_a_continuous_batch_over_pages(va, fmt):
+    # RaggedKVCache.prefill_chunk sends a full chunk of a few tokens through the decode kernels; over a paged cache
+    # (shuffled page table, chunks that cross pages) the results are those of the contiguous cache, bit for bit
+    B, Hq, Hkv, D, S_max, P, T = 3, 8, 2, 128, 640, 128, 4
+    n_pages = B * (S_max // P) + 2
+    flat = va.RaggedKVCache(B, Hkv, S_max, D, fmt=fmt)
+    paged = va.RaggedKVCache(B, Hkv, S_max, D, fmt=fmt, paging=(P, n_pages))
+    perm = np.random.default_rng(5).permutation(n_pages)[:B * (S_max // P)].astype(np.int32).reshape(B, S_max // P)
+    paged.page_table.copy_(torch.from_numpy(perm))
+    lens = [386, 130, 259]          # each chunk of 4 straddles a page boundary or a 256-token split
+    q, k, v = [O.bf16_round(x * np.float32(0.5)) for x in I.qkv(5300, B, Hq, Hkv, 400, 400, D)]
+    n0 = torch.tensor([l - T for l in lens], dtype=torch.int32, device=G.dev())
+    outs = []
+    for c in (flat, paged):
+        c.append(G.to_bf16_dev(k[:, :, :390]), G.to_bf16_dev(v[:, :, :390]), n_new=n0)
+        ck = np.stack([k[b, :, lens[b] - T:lens[b]] for b in range(B)])
+        cvv = np.stack([v[b, :, lens[b] - T:lens[b]] for b in range(B)])
+        c.append(G.to_bf16_dev(ck), G.to_bf16_dev(cvv))
+        cq = np.stack([q[b, :, lens[b] - T:lens[b]] for b in range(B)])
+        outs.append(c.prefill_chunk(G.to_bf16_dev(cq)))
+    assert paged.seq_lens.cpu().tolist() == lens
+    assert torch.equal(outs[0], outs[1])
+    kk, vv = (k, v) if fmt == "bf16" else (O.q8_0_dequantize(*O.q8_0_quantize(k)), O.q8_0_dequantize(*O.q8_0_quantize(v)))
+    for b in range(B):
+        want = _expected_rows(q[b:b + 1], kk[b:b + 1], vv[b:b + 1], lens[b], T)
+        G.assert_bf16_close(G.bf16_to_np(outs[1][b:b + 1]), want, f"row {b}")
+
+
 def test_config4_shape_four_tokens(va):
     # benchmark config 4's shape (B32, 32/8 heads, D128, lengths U[1024, 32768]) with four tokens per sequence: sampled
     # sequences against the chunked prefill over the same planes

@@ -271,7 +271,11 @@ class RaggedKVCache(KVCache):
         return decode_attention(q, self, seq_lens=self.seq_lens, max_len=max(self.upper, 1), scale=scale, out=out)
 
     def prefill_chunk(self, q, n_new=None, scale=None):
-        """Attention of the chunk just appended (q [B,Hq,T,D], row b valid for n_new[b] rows) over each row's context."""
+        """Attention of the chunk just appended (q [B,Hq,T,D], row b valid for n_new[b] rows) over each row's context.
+        A full chunk of a few tokens (T * query heads per kv head <= 16) goes through the decode kernels."""
+        T, D = q.shape[2], q.shape[3]
+        if n_new is None and T > 1 and T * (q.shape[1] // self._c.Hkv) <= 16 and D in (64, 128):
+            return decode_attention_multi(q, self, seq_lens=self.seq_lens, max_len=max(self.upper, 1), scale=scale)
         return self.prefill(q, seq_lens=self.seq_lens, chunk_lens=n_new, scale=scale)
 
 
