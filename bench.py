@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on ONE MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|p4k|c3|c2f|c4|c5|c4f|c4p|c4w|c2c|c3c|r2|b2|b3|b2f] [--no-cpu] [--no-extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|p4k|c3|c2f|c4|c5|c4f|c4p|c4w|c4m|c2c|c3c|r2|b2|b3|b2f] [--no-cpu] [--no-extra]
 
 A "step" is one pass of the hot path over one batch of synthetic input that is already resident in
 HBM: one prefill launch (c2, p4k, c3) or one decode call = split-K kernel + combine kernel (c4, c5).
@@ -48,6 +48,10 @@ WORKLOADS = {
     "c4w": dict(kind="decode", fmt="bf16", B=32, Hq=32, Hkv=8, D=128, S=32768, lens=(1024, 32768, 4004), proj=True,
                 name="config 4 through the module's output projection: decode as config 4, heads merged, y = x Wo^T with "
                      "Wo [4096, 4096] bf16 in the same call (algorithmic bytes: KV + Wo)"),
+    "c4m": dict(kind="decode", fmt="bf16", B=32, Hq=32, Hkv=8, D=128, S=32768, lens=(1024, 32768, 4004), tokens=4,
+                name="config 4 with four tokens per sequence in one decode step (speculative verification: the tokens and the query "
+                     "heads of a kv head share the MFMA columns, K/V read once per kv head): otherwise as config 4; algorithmic "
+                     "bytes = config 4's KV rows + the four tokens' q / out"),
     "c2c": dict(kind="prefill_cached", fmt="bf16", B=4, Hq=32, Hkv=8, D=128, N=2048,
                 name="config 2 through the cache: causal GQA prefill bf16 reading K/V from the bf16 cache planes, "
                      "B4, 32 q / 8 kv heads, D128, N2048"),
@@ -82,7 +86,7 @@ def prefill_flops(w):
 def decode_bytes(w, lens):
     esz = {"bf16": 2, "f32": 4}.get(w["fmt"])
     row = esz * w["D"] if esz else (w["D"] + 2 * (w["D"] // 32))  # bytes per (token, kv head) per plane
-    return float(sum(2 * w["Hkv"] * int(L) * row for L in lens) + w["B"] * w["Hq"] * w["D"] * 2 * (esz or 2))
+    return float(sum(2 * w["Hkv"] * int(L) * row for L in lens) + w["B"] * w["Hq"] * w.get("tokens", 1) * w["D"] * 2 * (esz or 2))
 
 
 class Runner:
@@ -180,7 +184,7 @@ class Runner:
                     del kb, vb
             self.cache.set_len(S)
             self.seq_lens = torch.from_numpy(lens).to(dev)
-            self.q = torch.randn(B, Hq, 1, D, device=dev, generator=g).to(torch.float32 if w["fmt"] == "f32" else torch.bfloat16)
+            self.q = torch.randn(B, Hq, w.get("tokens", 1), D, device=dev, generator=g).to(torch.float32 if w["fmt"] == "f32" else torch.bfloat16)
             self.out = torch.empty_like(self.q)
             self.scale = 1.0 / math.sqrt(D)
             self.work = decode_bytes(w, lens)
@@ -230,6 +234,9 @@ class Runner:
         if self.w.get("proj"):
             return self.va.decode_attention_proj(self.q, self.cache, self.wo, None, seq_lens=self.seq_lens, max_len=self.max_len,
                                                  scale=self.scale, out=self.y)
+        if self.w.get("tokens", 1) > 1:
+            return self.va.decode_attention_multi(self.q, self.cache, seq_lens=self.seq_lens, max_len=self.max_len,
+                                                  scale=self.scale, out=self.out)
         return self.va.decode_attention(self.q, self.cache, seq_lens=self.seq_lens, max_len=self.max_len,
                                         scale=self.scale, out=self.out)
 
@@ -445,7 +452,7 @@ def main():
 
     if not args.no_extra:
         others = {}
-        for key in ("c2", "p4k", "c3", "c2f", "c4", "c5", "c4f", "c4p", "c4w", "c2c", "c3c", "r2", "b2", "b3", "b2f"):
+        for key in ("c2", "p4k", "c3", "c2f", "c4", "c5", "c4f", "c4p", "c4w", "c4m", "c2c", "c3c", "r2", "b2", "b3", "b2f"):
             if key == args.workload:
                 continue
             r = Runner(key, torch, va)
