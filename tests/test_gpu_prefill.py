@@ -171,6 +171,41 @@ def test_bf16_negative_scale_and_large_logits(va):
     G.assert_bf16_close(out, closed_form64(q, k2, v, 1.0, False).astype(np.float32), "growing logits")
 
 
+@pytest.mark.parametrize("N", [160, 300, 1111])
+@pytest.mark.parametrize("kind", ["growing", "spike_first", "spike_mid", "spike_last", "alternating_tiles", "negative_scale"])
+def test_bf16_d128_logits_in_the_tens_and_hundreds(va, N, kind):
+    # head_dim 128 (the pipelined kernel, and the same kernel over a cache's planes) with scale 1 on unit-variance
+    # operands: logits of standard deviation 11, up to several hundred in the scaled cases.  The reference maximum of a
+    # row is raised many times, by single keys hundreds above the rest in the spike cases (the exp2 of a tile overflows
+    # before the raise), and a score that carried a rounding of 2^-9 (Q multiplied by the scale in bf16) would miss the
+    # bar by an order of magnitude here.
+    q, k, v = [O.bf16_round(x) for x in I.qkv(70 + N, 1, 4, 2, N, N, 128)]
+    scale = 1.0
+    if kind in ("growing", "negative_scale"):
+        k = O.bf16_round(k * np.linspace(0.1, 6.0, N, dtype=np.float32)[None, None, :, None])
+        scale = -1.0 if kind == "negative_scale" else 1.0
+    elif kind == "alternating_tiles":
+        k = O.bf16_round(k * np.where(np.arange(N) % 64 < 32, 0.05, 5.0).astype(np.float32)[None, None, :, None])
+    else:  # one key aligned with the last query of each head pair: its score is about 4 |q|^2 = 512
+        pos = {"spike_first": 0, "spike_mid": N // 2, "spike_last": N - 1}[kind]
+        k = k.copy()
+        k[:, :, pos] = O.bf16_round(q[:, ::2, N - 1] * 4.0)
+    tq, tk, tv = G.to_bf16_dev(q), G.to_bf16_dev(k), G.to_bf16_dev(v)
+    for causal in (True, False):
+        want = closed_form64(q, k, v, scale, causal).astype(np.float32)
+        # outputs reach |v| ~ 4, where one bf16 step is 0.0156 - 0.031: the bar is the usual one plus that rounding
+        got = G.bf16_to_np(va.flash_attention(tq, tk, tv, scale, causal))
+        assert np.isfinite(got).all()
+        err = np.abs(got.astype(np.float64) - want)
+        assert err.max() <= 3.5e-2 and err.mean() <= G.BF16_MEAN_ABS, f"{kind} N={N} causal={causal}: {err.max():.3g} / {err.mean():.3g}"
+    c = va.KVCache(1, 2, (N + 63) // 64 * 64, 128, fmt="bf16")
+    c.update(tk, tv, 0, return_views=False)
+    want = closed_form64(q, k, v, scale, True).astype(np.float32)
+    got = G.bf16_to_np(c.prefill(tq, scale=scale))
+    err = np.abs(got.astype(np.float64) - want)
+    assert np.isfinite(got).all() and err.max() <= 3.5e-2 and err.mean() <= G.BF16_MEAN_ABS, f"planes {kind} N={N}: {err.max():.3g}"
+
+
 def test_bf16_full_size_properties(va):
     # benchmark config 2 shape (B4, 32/8 heads, D128, N2048): properties that need no oracle at this size
     B, Hq, Hkv, N, D = 4, 32, 8, 2048, 128

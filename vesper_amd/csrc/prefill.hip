@@ -732,8 +732,9 @@ __global__ void __launch_bounds__(256, 2) prefill_split_kernel(PrefillArgs a) {
 // Vector-ALU instructions of one wavefront hardly overlap with MFMAs of ANOTHER wavefront on the same SIMD (a wavefront
 // of nothing but vector-ALU work gets about one instruction in per MFMA of its neighbour), while those that follow an
 // MFMA in the same instruction stream are nearly free; hence this structure, and the diet of the softmax stage:
-//   - scale * log2(e) is folded into Q once per workgroup, and -m (the row's reference maximum) enters as the C
-//     operand of the first QK^T MFMA, so the scores arrive as s' = s - m and P is a bare exp2;
+//   - -m / c (m: the row's reference maximum, c = |scale| * log2(e)) enters as the C operand of the first QK^T MFMA,
+//     so P is one multiply and one exp2 per score (Q is not pre-multiplied by c: rounding Q * c to bf16 again costs
+//     2^-9 of every score, which shows in the output once logits reach the tens);
 //   - the row sum uses plain adds (v_dot2c_f32_bf16 occupies the matrix pipe);
 //   - no row maximum per tile: m is raised only when the row sum shows that it has fallen behind (rare), and is
 //     kept integer-valued (log2 domain) so that the rescale factor is a power of two and the P tile that has been
@@ -828,19 +829,17 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_pipe_kernel(PrefillArgs a
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) qraw[ks] = *(const uint4*)(Qp + (int64_t)qrow * a.sq[2] + 16 * ks + 8 * h);
     bf16x8_t qf[KS];
+    // Q goes into the MFMAs as stored (a negative scale flips its sign bits: exact); |scale| * log2(e) multiplies the
+    // fp32 scores in front of the exp2, so the scores carry no rounding beyond the fp32 accumulation
+    const float cexp = a.scale_log2;
+    const float inv_cexp = 1.0f / cexp;
     auto prescale_q = [&]() {
+        const uint32_t flip = a.negate_q ? 0x80008000u : 0u;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-        const uint4 w = qraw[ks];
-        // fold scale * log2(e) (and the sign of a negative scale) into Q: one more bf16 rounding of Q
-        const float c = a.negate_q ? -a.scale_log2 : a.scale_log2;
-        const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
-        uint32_t o[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            o[i] = cvt_pk_bf16(__builtin_bit_cast(float, ww[i] << 16) * c, __builtin_bit_cast(float, ww[i] & 0xffff0000u) * c);
-        qf[ks] = __builtin_bit_cast(bf16x8_t, uint4{o[0], o[1], o[2], o[3]});
-    }
+        for (int ks = 0; ks < KS; ++ks) {
+            const uint4 w = qraw[ks];
+            qf[ks] = __builtin_bit_cast(bf16x8_t, uint4{w.x ^ flip, w.y ^ flip, w.z ^ flip, w.w ^ flip});
+        }
     };
 
     const int wg_qmax = min(qt * kBM + kBM - 1, a.T - 1);
@@ -933,11 +932,12 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_pipe_kernel(PrefillArgs a
         va[db] = VBLK ? lds0 + 16u * (uint32_t)(h * D + ql) : lds0 + 2u * (uint32_t)v_lane_off + 64u * (uint32_t)(db ^ vswz);
 
     Frag fr[16];         // operand of MFMA slot s of the current step (slots < kLead: already requested)
-    // Scores are kept as S' = s * scale * log2(e) - m: the factor is folded into Q (below), and -m, the row's reference
-    // maximum, enters as the C operand of the first QK^T MFMA from a tile of 16 registers that all hold -m.
+    // With c = |scale| * log2(e), scores are kept as u = q.k - m / c: -m / c (m = the row's reference maximum in the
+    // log2 domain) enters as the C operand of the first QK^T MFMA from a tile of 16 registers that all hold it, and
+    // P = exp2(c * u).
     f32x16_t sb[2];      // step tau finishes S'(tau+2) in sb[tau & 1] and consumes S'(tau+1) from sb[(tau+1) & 1]
     uint32_t pb[2][8];   // packed bf16 P: step tau consumes P(tau) from pb[tau & 1] and writes P(tau+1) to pb[(tau+1) & 1]
-    f32x16_t negm;       // every element = -m_ref of this lane's query
+    f32x16_t negm;       // every element = -m_ref / c of this lane's query
 #pragma unroll
     for (int j = 0; j < 16; ++j) negm[j] = 0.f;
     m_ref = 0.f;  // "no reference yet": the first tile sets it
@@ -999,7 +999,11 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_pipe_kernel(PrefillArgs a
         // contexts are normalised by exactly what was accumulated (a single key reproduces V bit for bit).
         auto softmax_op = [&](auto i_c) {
             constexpr int i = decltype(i_c)::value, p = i / 4, k = i % 4;
-            if constexpr (k < 2) es[2 * p + k] = __builtin_amdgcn_exp2f(s_cur[2 * p + k]);
+            if constexpr (k == 0) {  // both multiplies first: neither exp2 waits on the instruction right before it
+                es[2 * p] = s_cur[2 * p] * cexp;
+                es[2 * p + 1] = s_cur[2 * p + 1] * cexp;
+                es[2 * p] = __builtin_amdgcn_exp2f(es[2 * p]);
+            } else if constexpr (k == 1) es[2 * p + 1] = __builtin_amdgcn_exp2f(es[2 * p + 1]);
             else if constexpr (k == 2) p_nxt[p] = cvt_pk_bf16(es[2 * p], es[2 * p + 1]);
             else if constexpr (FAST && !MASK) { lsum += es[2 * p]; lsum2 += es[2 * p + 1]; }
             else lsum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, p_nxt[p]), __builtin_bit_cast(bf16x2_t, 0x3f803f80u), lsum, false);
@@ -1071,8 +1075,10 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_pipe_kernel(PrefillArgs a
 #pragma unroll
                 for (int v = 1; v < 16; ++v) mx = fmaxf(mx, s_cur[v]);
                 mx = half_swap_max(mx);
-                float delta = (mx == -INFINITY) ? 0.f : ceilf(mx);  // raise (first tile: set) the reference by delta
+                // raise (first tile: set) the reference by delta, an integer in the log2 domain; the scores move by du
+                float delta = (mx == -INFINITY) ? 0.f : ceilf(mx * cexp);
                 if (!first) delta = fmaxf(delta, 0.f);
+                const float du = delta == 0.f ? 0.f : delta * inv_cexp;  // (a scale in the denormal range has 1 / c = inf)
                 if constexpr (!first) {  // nothing has been accumulated before the first tile
                     const float alpha = __builtin_amdgcn_exp2f(-delta);
                     l *= alpha;
@@ -1083,15 +1089,15 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_pipe_kernel(PrefillArgs a
                 }
                 lsum = lsum2 = 0.f;
 #pragma unroll
-                for (int v = 0; v < 16; ++v) s_cur[v] -= delta;
+                for (int v = 0; v < 16; ++v) s_cur[v] -= du;
                 static_for<32>([&](auto i_c) { softmax_op(i_c); });
                 if (qk_on) {
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) s_nxt[v] -= delta;  // finished this step against the old reference
+                    for (int v = 0; v < 16; ++v) s_nxt[v] -= du;  // finished this step against the old reference
                 }
                 m_ref += delta;
 #pragma unroll
-                for (int j = 0; j < 16; ++j) negm[j] = -m_ref;
+                for (int j = 0; j < 16; ++j) negm[j] = m_ref == 0.f ? 0.f : -m_ref * inv_cexp;
             }
             l += lsum + lsum2;
         }
