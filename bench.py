@@ -10,7 +10,9 @@ causal GQA prefill bf16, B4, 32/8 heads, D128, N2048, in TFLOP/s of algorithmic 
 2*D*B*Hq*N*(N+1)); `other_workloads` carries the remaining benchmark configs (decode in GB/s of
 algorithmic KV bytes).  `roofline` is for the primary workload's dominant kernel, timed with events
 on the launch stream; `cpu_baseline` is the reference's own CPU path (oracle/_ref, else the oracle
-port) timed on this host on a bounded sample of the same workload.
+port) timed on this host on a bounded sample of the same workload.  `yardsticks` (with the other workloads) says what
+the same box sustains on the bf16 matrix cores outside this library: the vendor GEMM behind torch.matmul and torch's own
+attention on config 2's tensors; context for the fractions, nothing else.
 """
 import argparse
 import json
@@ -381,6 +383,46 @@ def traffic_from_profile(key):
     return out
 
 
+def yardsticks(torch):
+    """What the same box sustains on the bf16 matrix cores outside this library, for scale next to the roofline fractions
+    (not a baseline and not part of any figure above): the vendor GEMM behind torch.matmul on 8192^3 bf16 operands, and
+    torch's own scaled_dot_product_attention on config 2's tensors."""
+    import time as _t
+
+    def rate(fn, flops, n):
+        t0 = _t.time()
+        while _t.time() - t0 < CONDITION_SECONDS:
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return round(flops / (e0.elapsed_time(e1) / n * 1e-3) / 1e12, 1)
+
+    out = {"note": "same box, same process; outside this library (torch.matmul -> vendor GEMM, torch SDPA); TFLOP/s"}
+    g = torch.Generator(device="cuda").manual_seed(5)
+    mk = lambda *shape: (torch.randn(*shape, device="cuda:0", generator=g) * 0.5).to(torch.bfloat16)
+    try:
+        a, b = mk(8192, 8192), mk(8192, 8192)
+        out["bf16_gemm_8192_nt"] = rate(lambda: torch.matmul(a, b.t()), 2 * 8192 ** 3, 20)
+        out["bf16_gemm_8192_nn"] = rate(lambda: torch.matmul(a, b), 2 * 8192 ** 3, 20)
+        del a, b
+    except Exception as e:  # a yardstick, never a reason to fail the run
+        out["bf16_gemm_error"] = repr(e)[:200]
+    try:
+        import torch.nn.functional as F
+        q, k, v = mk(4, 32, 2048, 128), mk(4, 8, 2048, 128), mk(4, 8, 2048, 128)
+        out["torch_sdpa_config2"] = rate(lambda: F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True),
+                                         2 * 128 * 4 * 32 * 2048 * 2049, 10)
+    except Exception as e:
+        out["torch_sdpa_error"] = repr(e)[:200]
+    torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -467,6 +509,7 @@ def main():
             del r
             torch.cuda.empty_cache()
         result["other_workloads"] = others
+        result["yardsticks"] = yardsticks(torch)
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(args.workload)
