@@ -91,6 +91,15 @@ def decode_bytes(w, lens):
     return float(sum(2 * w["Hkv"] * int(L) * row for L in lens) + w["B"] * w["Hq"] * w.get("tokens", 1) * w["D"] * 2 * (esz or 2))
 
 
+def prefill_kernel_name(torch, B, Hq, N, planes):
+    """The library's own choice between its two head_dim-128 bf16 kernels (launch_prefill in csrc/prefill.hip): the general
+    kernel for contexts up to 2560 tokens on a grid of at least 3 x CUs workgroups, the software-pipelined one otherwise."""
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    short = N <= 2560 and -(-N // 128) * B * Hq >= 3 * cus
+    p = "true" if planes else "false"
+    return f"prefill_bf16_kernel<128, {p}>" if short else f"prefill_bf16_pipe_kernel<{p}>"
+
+
 class Runner:
     """Builds the device-resident inputs of one workload and exposes step()."""
 
@@ -106,7 +115,7 @@ class Runner:
             self.scale = 1.0 / math.sqrt(D)
             self.work = prefill_flops(w)
             self.unit, self.peak, self.bound = "TFLOP/s", MFMA_BF16_PEAK_TFLOPS, "mfma"
-            self.kernel = "prefill_bf16_pipe_kernel"
+            self.kernel = prefill_kernel_name(torch, B, Hq, N, False)
         elif w["kind"] == "prefill_split":
             B, Hq, Hkv, D, N = w["B"], w["Hq"], w["Hkv"], w["D"], w["N"]
             mk = lambda h: torch.randn(B, h, N, D, device=dev, generator=g) * 0.5
@@ -124,7 +133,7 @@ class Runner:
             self.cache.update(mk(Hkv), mk(Hkv), 0, return_views=False)
             self.work = prefill_flops(w)
             self.unit, self.peak, self.bound = "TFLOP/s", MFMA_BF16_PEAK_TFLOPS, "mfma"
-            self.kernel = "prefill_bf16_pipe_kernel<true>"
+            self.kernel = prefill_kernel_name(torch, B, Hq, N, True)
         elif w["kind"] == "backward":
             B, Hq, Hkv, D, N = w["B"], w["Hq"], w["Hkv"], w["D"], w["N"]
             mk = lambda h: (torch.randn(B, h, N, D, device=dev, generator=g) * 0.5).to(torch.bfloat16)
@@ -342,7 +351,7 @@ PROFILE_OF = {
     "c2": ("prefill_bf16_config2.txt", "prefill_bf16", 96 * 2**20 + 65 * 2**20),
     "p4k": ("prefill_bf16_4k.txt", "prefill_bf16", 96 * 2**20 + 65 * 2**20),
     "c3": ("prefill_bf16_config3.txt", "prefill_bf16", 96 * 2**20 + 65 * 2**20),
-    "c2c": ("prefill_bf16_cache_planes_config2.txt", "prefill_bf16_pipe_kernel<true>", 96 * 2**20 + 65 * 2**20),
+    "c2c": ("prefill_bf16_cache_planes_config2.txt", "prefill_bf16", 96 * 2**20 + 65 * 2**20),
     "r2": ("rope_append_bf16_config2.txt", "append_bf16_tile_kernel<unsigned short, true", 202375168),
     "c4": ("decode_bf16_config4.txt", "decode_bf16_kernel", 2614935552),
     "c5": ("decode_q8_0_config5.txt", "decode_q8_kernel", 2282225664),

@@ -171,15 +171,17 @@ def test_bf16_negative_scale_and_large_logits(va):
     G.assert_bf16_close(out, closed_form64(q, k2, v, 1.0, False).astype(np.float32), "growing logits")
 
 
+@pytest.mark.parametrize("D", [128, 64])
 @pytest.mark.parametrize("N", [160, 300, 1111])
 @pytest.mark.parametrize("kind", ["growing", "spike_first", "spike_mid", "spike_last", "alternating_tiles", "negative_scale"])
-def test_bf16_d128_logits_in_the_tens_and_hundreds(va, N, kind):
-    # head_dim 128 (the pipelined kernel, and the same kernel over a cache's planes) with scale 1 on unit-variance
-    # operands: logits of standard deviation 11, up to several hundred in the scaled cases.  The reference maximum of a
-    # row is raised many times, by single keys hundreds above the rest in the spike cases (the exp2 of a tile overflows
+def test_bf16_logits_in_the_tens_and_hundreds(va, N, kind, D):
+    # head_dim 128 (the pipelined kernel, and the same kernel over a cache's planes) and 64 (the general kernel) with
+    # scale 1 on unit-variance operands: logits of standard deviation 11 (8 at head_dim 64), up to several hundred in the
+    # scaled cases.  Both kernels raise a row's reference maximum only when the row sum shows it has fallen behind: here
+    # that happens many times, by single keys hundreds above the rest in the spike cases (the exp2 of a tile overflows
     # before the raise), and a score that carried a rounding of 2^-9 (Q multiplied by the scale in bf16) would miss the
-    # bar by an order of magnitude here.
-    q, k, v = [O.bf16_round(x) for x in I.qkv(70 + N, 1, 4, 2, N, N, 128)]
+    # bar by an order of magnitude.
+    q, k, v = [O.bf16_round(x) for x in I.qkv(70 + N, 1, 4, 2, N, N, D)]
     scale = 1.0
     if kind in ("growing", "negative_scale"):
         k = O.bf16_round(k * np.linspace(0.1, 6.0, N, dtype=np.float32)[None, None, :, None])
@@ -198,12 +200,51 @@ def test_bf16_d128_logits_in_the_tens_and_hundreds(va, N, kind):
         assert np.isfinite(got).all()
         err = np.abs(got.astype(np.float64) - want)
         assert err.max() <= 3.5e-2 and err.mean() <= G.BF16_MEAN_ABS, f"{kind} N={N} causal={causal}: {err.max():.3g} / {err.mean():.3g}"
-    c = va.KVCache(1, 2, (N + 63) // 64 * 64, 128, fmt="bf16")
+    c = va.KVCache(1, 2, (N + 63) // 64 * 64, D, fmt="bf16")
     c.update(tk, tv, 0, return_views=False)
     want = closed_form64(q, k, v, scale, True).astype(np.float32)
     got = G.bf16_to_np(c.prefill(tq, scale=scale))
     err = np.abs(got.astype(np.float64) - want)
     assert np.isfinite(got).all() and err.max() <= 3.5e-2 and err.mean() <= G.BF16_MEAN_ABS, f"planes {kind} N={N}: {err.max():.3g}"
+
+
+@pytest.mark.parametrize("kind", ["growing", "spike_mid"])
+def test_bf16_d128_general_kernel_logits_in_the_tens_and_hundreds(va, kind):
+    # the same inputs on a grid large enough (3 x 32 heads x 9 query tiles = 864 workgroups, context <= 2560) that
+    # head_dim 128 goes to the general kernel
+    B, Hq, Hkv, N, D = 3, 32, 8, 1111, 128
+    q, k, v = [O.bf16_round(x) for x in I.qkv(77, B, Hq, Hkv, N, N, D)]
+    if kind == "growing":
+        k = O.bf16_round(k * np.linspace(0.1, 6.0, N, dtype=np.float32)[None, None, :, None])
+    else:
+        k = k.copy()
+        k[:, :, N // 2] = O.bf16_round(q[:, ::4, N - 1] * 4.0)
+    got = G.bf16_to_np(va.flash_attention(G.to_bf16_dev(q), G.to_bf16_dev(k), G.to_bf16_dev(v), 1.0, True))
+    want = closed_form64(q, k, v, 1.0, True).astype(np.float32)
+    err = np.abs(got.astype(np.float64) - want)
+    assert np.isfinite(got).all() and err.max() <= 3.5e-2 and err.mean() <= G.BF16_MEAN_ABS, (err.max(), err.mean())
+
+
+def test_bf16_d128_the_two_kernels_agree(va):
+    # head_dim 128 is served by two kernels: short contexts on a grid that fills the chip (here B2 x 32 heads x 2048:
+    # 1024 workgroups) go to the general kernel, the same rows one batch row at a time (512 workgroups) and longer
+    # contexts to the software-pipelined one.  Same inputs, same rows: the results differ by bf16 roundings only, and
+    # the sampled rows match the oracle.
+    B, Hq, Hkv, N, D = 2, 32, 8, 2048, 128
+    g = torch.Generator(device="cuda").manual_seed(11)
+    mk = lambda h: (torch.randn(B, h, N, D, device=G.dev(), generator=g) * 0.5).to(torch.bfloat16)
+    q, k, v = mk(Hq), mk(Hkv), mk(Hkv)
+    scale = 1.0 / math.sqrt(D)
+    both = va.flash_attention(q, k, v, scale, True)
+    for b in range(B):
+        one = va.flash_attention(q[b:b + 1], k[b:b + 1], v[b:b + 1], scale, True)
+        d = (both[b:b + 1].float() - one.float()).abs()
+        assert d.max().item() <= 1.6e-2 and d.mean().item() <= 1e-3, (b, d.max().item(), d.mean().item())
+    # oracle on one (batch row, kv head): 4 query heads, all 2048 rows
+    qn = q[1:2, 4:8].float().cpu().numpy()
+    kn, vn = k[1:2, 1:2].float().cpu().numpy(), v[1:2, 1:2].float().cpu().numpy()
+    want, _ = oracle_gqa_flash(qn, kn, vn, float(np.float32(scale)), True)
+    G.assert_bf16_close(G.bf16_to_np(both[1:2, 4:8]), want, "general kernel, head_dim 128, N 2048")
 
 
 def test_bf16_full_size_properties(va):

@@ -1061,19 +1061,6 @@ __global__ void __launch_bounds__(256) proj_f32_kernel(const float* __restrict__
     }
 }
 
-int device_cu_count() {
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) == hipSuccess &&
-            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-            cus = n;
-        else
-            cus = 256;
-    }
-    return cus;
-}
-
 // Tokens per split.  Every work item pays a fixed cost (locating itself, loading Q, merging four wavefronts, writing a
 // partial) and every split is one more row for the combine kernel, so splits should be as long as they can be while
 // the launch still spreads over the chip: the largest candidate that yields at least one work item per two CUs

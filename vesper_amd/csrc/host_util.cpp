@@ -20,6 +20,16 @@ int check_launch() {
     }
     return VSP_OK;
 }
+int device_cu_count() {
+    static const int cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            return n;
+        return 256;
+    }();
+    return cus;
+}
 }  // namespace vsp
 
 extern "C" {

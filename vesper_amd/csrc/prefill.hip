@@ -330,30 +330,42 @@ __global__ void __launch_bounds__(256, 3) prefill_bf16_kernel(PrefillArgs a) {
                 if (key > lim) s[0][v] = -INFINITY;
             }
         }
-        float mx = s[0][0];
+        // P is taken against the row's reference maximum as it stands, and the row sum says whether that reference
+        // has fallen behind: below 2^10 no P of the tile exceeds 2^10, far from overflow in the fp32 accumulators.
+        // Otherwise (rare on real data; always for the first tile, which has no reference yet) the true maximum of
+        // these scores becomes the reference, what has been accumulated is rescaled and this tile's P is redone.  The
+        // mathematics is the reference's online softmax (src/ops/flash_attention.cpp:309-343) with a reference point
+        // that moves only when it has to, which takes the per-tile row maximum (16 max + a cross-half exchange) out of
+        // the steady state.  The row sum is taken from the rounded bf16 P (packed dot product against (1, 1)): exactly
+        // what the PV MFMAs accumulate.
+        uint32_t pw[NJ][4];
+        float lsum = 0.f;
+        auto softmax = [&](float neg_m) {
+            lsum = 0.f;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[0][v]);
-        mx = half_swap_max(mx) * a.scale_log2;
-        if (__any(mx > m_ref + kRescaleThreshold)) {
+            for (int v = 0; v < 16; v += 2) {
+                const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[0][v], a.scale_log2, neg_m));
+                const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[0][v + 1], a.scale_log2, neg_m));
+                const uint32_t pk = cvt_pk_bf16(p0, p1);
+                pw[v >> 3][(v & 7) >> 1] = pk;
+                lsum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pk), __builtin_bit_cast(bf16x2_t, 0x3f803f80u), lsum, false);
+            }
+        };
+        if (t > 0) softmax(m_ref == -INFINITY ? 0.f : -m_ref);
+        if (t == 0 || __any(!(lsum < 1024.f))) {
+            float mx = s[0][0];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[0][v]);
+            mx = half_swap_max(mx) * a.scale_log2;
             const float m_new = fmaxf(m_ref, mx);
-            const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_ref - m_new);
+            const float alpha = (m_new == -INFINITY || m_ref == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_ref - m_new);
             l *= alpha;
 #pragma unroll
             for (int i = 0; i < DB; ++i)
 #pragma unroll
                 for (int j = 0; j < 16; ++j) acc[i][j] *= alpha;
             m_ref = m_new;
-        }
-        const float neg_m = (m_ref == -INFINITY) ? 0.f : -m_ref;
-        uint32_t pw[NJ][4];
-        float lsum = 0.f;
-#pragma unroll
-        for (int v = 0; v < 16; v += 2) {
-            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[0][v], a.scale_log2, neg_m));
-            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[0][v + 1], a.scale_log2, neg_m));
-            const uint32_t pk = cvt_pk_bf16(p0, p1);
-            pw[v >> 3][(v & 7) >> 1] = pk;
-            lsum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pk), __builtin_bit_cast(bf16x2_t, 0x3f803f80u), lsum, false);
+            softmax(m_ref == -INFINITY ? 0.f : -m_ref);
         }
         l += lsum;
         // PV
@@ -1309,13 +1321,19 @@ int launch_prefill(const PrefillArgs& a, int dtype, int64_t D, bool cache_planes
     hipStream_t st = (hipStream_t)stream;
     dim3 grid((unsigned)blocks), block(256);
     if (dtype == VSP_BF16) {
+        // head_dim 128 has two kernels.  The software-pipelined one (two workgroups per CU) has the faster steady state;
+        // the general one (three per CU, no pipeline to fill and drain) has the cheaper workgroup and wins while contexts
+        // are short, provided the grid fills its 3 x CUs slots: measured crossover between 2560 and 3072 tokens
+        // (+3 % at 2048, +10 % at 1024, +14 % at 512; -2 % at 3072, -3 % at 8192).
+        const bool short_ctx = a.L <= 2560 && blocks >= 3 * (int64_t)device_cu_count();
         if (cache_planes) {
-            if (D == 128) hipLaunchKernelGGL(prefill_bf16_pipe_kernel<true>, grid, block, 0, st, a);
+            if (D == 128 && !short_ctx) hipLaunchKernelGGL(prefill_bf16_pipe_kernel<true>, grid, block, 0, st, a);
+            else if (D == 128) hipLaunchKernelGGL((prefill_bf16_kernel<128, true>), grid, block, 0, st, a);
             else hipLaunchKernelGGL((prefill_bf16_kernel<64, true>), grid, block, 0, st, a);
         } else {
             // the software-pipelined kernel takes one context length for the batch; dense K/V with per-row lengths
             // (a Q8_0 cache read out into the workspace) stay with the general kernel
-            if (D == 128 && !a.seq_lens && !a.chunk_lens) hipLaunchKernelGGL(prefill_bf16_pipe_kernel<false>, grid, block, 0, st, a);
+            if (D == 128 && !a.seq_lens && !a.chunk_lens && !short_ctx) hipLaunchKernelGGL(prefill_bf16_pipe_kernel<false>, grid, block, 0, st, a);
             else if (D == 128) hipLaunchKernelGGL((prefill_bf16_kernel<128, false>), grid, block, 0, st, a);
             else hipLaunchKernelGGL((prefill_bf16_kernel<64, false>), grid, block, 0, st, a);
         }

@@ -50,6 +50,7 @@ __device__ inline uint32_t pack_bf16x2(float a, float b) {
 // per-thread last HIP error text (vsp_last_hip_error)
 void set_hip_error(hipError_t e);
 int check_launch();  // VSP_OK or VSP_ERR_LAUNCH after a kernel launch
+int device_cu_count();  // compute units of the device that was current at the first call (256 if the query fails)
 
 inline bool is_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
