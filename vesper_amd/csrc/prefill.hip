@@ -1184,6 +1184,8 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_pipe_kernel(PrefillArgs a
         if (a.lse && h == 0)
             a.lse[(int64_t)b * a.sl[0] + (int64_t)hq * a.sl[1] + (int64_t)qi * a.sl[2]] = (m_ref + __builtin_amdgcn_logf(l)) * 0.6931471805599453f;
     }
+    // the clamped tile requests of the last steps write LDS: they have landed before the workgroup gives its LDS back
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #endif
 }
 
