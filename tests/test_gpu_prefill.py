@@ -225,6 +225,28 @@ def test_bf16_d128_general_kernel_logits_in_the_tens_and_hundreds(va, kind):
     assert np.isfinite(got).all() and err.max() <= 3.5e-2 and err.mean() <= G.BF16_MEAN_ABS, (err.max(), err.mean())
 
 
+@pytest.mark.parametrize("causal", [True, False])
+def test_bf16_d128_general_kernel_chunk_over_longer_context(va, causal):
+    # T < L on a grid of 8 x 32 heads x 3 query tiles = 768 workgroups: head_dim 128 through the general kernel, causal
+    # mask aligned to the end of the context, a context that ends inside a key tile, strided K/V views of a larger buffer
+    B, Hq, Hkv, T, L, D, S_max = 8, 32, 8, 384, 700, 128, 768
+    q, k, v = [O.bf16_round(x) for x in I.qkv(78, B, Hq, Hkv, T, L, D, scale=0.5)]
+    kb = torch.zeros(B, Hkv, S_max, D, dtype=torch.bfloat16, device=G.dev())
+    vb = torch.full((B, Hkv, S_max, D), float("nan"), dtype=torch.bfloat16, device=G.dev())
+    kb[:, :, :L], vb[:, :, :L] = G.to_bf16_dev(k), G.to_bf16_dev(v)
+    scale = 1.0 / math.sqrt(D)
+    out, lse = va.flash_attention(G.to_bf16_dev(q), kb[:, :, :L], vb[:, :, :L], scale, causal, return_lse=True)
+    G.assert_bf16_close(G.bf16_to_np(out), closed_form64(q, k, v, scale, causal).astype(np.float32), f"T<L causal={causal}")
+    # lse of a few rows against the definition
+    n = Hq // Hkv
+    for (b, h, t) in ((0, 0, 0), (3, 17, 200), (7, 31, 383)):
+        s = (k[b, h // n, :L].astype(np.float64) @ q[b, h, t].astype(np.float64)) * scale
+        if causal:
+            s = s[:L - T + t + 1]
+        want = np.log(np.exp(s - s.max()).sum()) + s.max()
+        assert abs(lse[b, h, t].item() - want) < 2e-2
+
+
 def test_bf16_d128_the_two_kernels_agree(va):
     # head_dim 128 is served by two kernels: short contexts on a grid that fills the chip (here B2 x 32 heads x 2048:
     # 1024 workgroups) go to the general kernel, the same rows one batch row at a time (512 workgroups) and longer
