@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on ONE MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|p4k|c3|c2f|c4|c5|c4f|c4p|c4w|c4m|c2c|c3c|r2|b2|b3|b2f] [--no-cpu] [--no-extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|p4k|c3|c2f|c4|c5|c4f|c4p|c4w|c4m|c2c|c3c|k512|r2|b2|b3|b2f] [--no-cpu] [--no-extra]
 
 A "step" is one pass of the hot path over one batch of synthetic input that is already resident in
 HBM: one prefill launch (c2, p4k, c3) or one decode call = split-K kernel + combine kernel (c4, c5).
@@ -60,6 +60,10 @@ WORKLOADS = {
     "c3c": dict(kind="prefill_cached", fmt="bf16", B=1, Hq=32, Hkv=8, D=128, N=8192,
                 name="config 3 through the cache: causal GQA prefill bf16 reading K/V from the bf16 cache planes, "
                      "B1, 32 q / 8 kv heads, D128, N8192"),
+    "k512": dict(kind="prefill_cached", fmt="bf16", B=1, Hq=32, Hkv=8, D=128, N=32768, T=512,
+                 name="one chunk of a long prompt: the last 512 tokens of a 32768-token context read from the bf16 cache planes, "
+                      "B1, 32 q / 8 kv heads, D128 (128 workgroups of queries: the context is split over workgroups and merged by "
+                      "the decode step's combine kernel)"),
     "b2": dict(kind="backward", B=4, Hq=32, Hkv=8, D=128, N=2048,
                name="attention backward at config 2's shape: causal GQA bf16 in/out, bf16 MFMA with fp32 accumulation, "
                     "B4, 32 q / 8 kv heads, D128, N2048 (dq, dk, dv; 2.5 x the forward's FLOPs)"),
@@ -82,7 +86,8 @@ def rope_bytes(w):
 
 
 def prefill_flops(w):
-    return 2.0 * w["D"] * w["B"] * w["Hq"] * w["N"] * (w["N"] + 1)
+    T = w.get("T", w["N"])  # the last T rows of the causal triangle over N keys
+    return 4.0 * w["D"] * w["B"] * w["Hq"] * (T * (w["N"] - T) + T * (T + 1) / 2.0)
 
 
 def decode_bytes(w, lens):
@@ -127,13 +132,15 @@ class Runner:
             self.kernel = "split_f32_kernel + prefill_split_kernel<128>"
         elif w["kind"] == "prefill_cached":
             B, Hq, Hkv, D, N = w["B"], w["Hq"], w["Hkv"], w["D"], w["N"]
-            mk = lambda h: (torch.randn(B, h, N, D, device=dev, generator=g) * 0.5).to(torch.bfloat16)
-            self.q = mk(Hq)
+            T = w.get("T", N)
+            mk = lambda h, n=N: (torch.randn(B, h, n, D, device=dev, generator=g) * 0.5).to(torch.bfloat16)
+            self.q = mk(Hq, T)
             self.cache = va.KVCache(B, Hkv, N, D, fmt=w["fmt"])
             self.cache.update(mk(Hkv), mk(Hkv), 0, return_views=False)
             self.work = prefill_flops(w)
             self.unit, self.peak, self.bound = "TFLOP/s", MFMA_BF16_PEAK_TFLOPS, "mfma"
-            self.kernel = prefill_kernel_name(torch, B, Hq, N, True)
+            self.kernel = (prefill_kernel_name(torch, B, Hq, N, True) if T == N else
+                           "prefill_bf16_pipe_kernel<true> (context split) + decode_combine_kernel")
         elif w["kind"] == "backward":
             B, Hq, Hkv, D, N = w["B"], w["Hq"], w["Hkv"], w["D"], w["N"]
             mk = lambda h: (torch.randn(B, h, N, D, device=dev, generator=g) * 0.5).to(torch.bfloat16)
@@ -503,7 +510,7 @@ def main():
 
     if not args.no_extra:
         others = {}
-        for key in ("c2", "p4k", "c3", "c2f", "c4", "c5", "c4f", "c4p", "c4w", "c4m", "c2c", "c3c", "r2", "b2", "b3", "b2f"):
+        for key in ("c2", "p4k", "c3", "c2f", "c4", "c5", "c4f", "c4p", "c4w", "c4m", "c2c", "c3c", "k512", "r2", "b2", "b3", "b2f"):
             if key == args.workload:
                 continue
             r = Runner(key, torch, va)

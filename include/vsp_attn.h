@@ -259,8 +259,15 @@ int vsp_attn_prefill_backward_split(const vsp_tensor* dout, const vsp_tensor* q,
  *                The other formats need no workspace (NULL, 0).
  * Tokens past L_b in the planes are never used, whatever they hold.  lse as in vsp_attn_prefill.
  * chunk_lens (nullable): device int32[B], n_b <= T valid query rows per sequence (ragged chunks in one call):
- * query t < n_b sits at position L_b - n_b + t; rows t >= n_b of `out` are unspecified. */
+ * query t < n_b sits at position L_b - n_b + t; rows t >= n_b of `out` are unspecified.
+ * Context split (VSP_KV_BF16, D = 128, lse == NULL): a chunk of a few query tiles over a long context leaves most of
+ * the chip idle, each workgroup walking the whole context.  A caller that passes a 16-byte aligned workspace of at
+ * least vsp_attn_prefill_cached_split_workspace_bytes(cache, with_seq_lens, Hq, T) bytes (0 when the grid fills the chip
+ * anyway, or the context is short) gets the context cut into shares of at least 512 keys, one workgroup per (query
+ * tile, head, share), and the partials merged by the decode step's combine kernel in a fixed order.  Without that
+ * workspace the call runs unsplit; the results agree within bf16 rounding either way. */
 size_t vsp_attn_prefill_cached_workspace_bytes(const vsp_kv_cache* cache, int with_seq_lens);
+size_t vsp_attn_prefill_cached_split_workspace_bytes(const vsp_kv_cache* cache, int with_seq_lens, int32_t Hq, int32_t T);
 int vsp_attn_prefill_cached(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens,
                             const int32_t* chunk_lens, vsp_tensor* out, vsp_tensor* lse, float scale, int is_causal,
                             void* workspace, size_t workspace_bytes, void* stream);

@@ -299,6 +299,28 @@ static void test_validation() {
     vsp_tensor qf32 = tensor4(mem, VSP_F32, 1, 4, 8, 64);
     c.len = 40;
     CHECK(vsp_attn_prefill_cached(&qf32, &c, nullptr, nullptr, &qf32, nullptr, 0.1f, 1, nullptr, 0, nullptr) == VSP_ERR_DTYPE);
+    // the context split is offered for bf16 planes at head_dim 128 when a short grid meets a long context, and only then
+    {
+        vsp_kv_cache big = c;
+        big.format = VSP_KV_BF16;
+        big.B = 1;
+        big.D = 128;
+        big.S_max = 4096;
+        big.len = 4096;
+        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&big, 0, 8, 100) == (size_t)1 * 8 * 100 * 8 * 130 * 4);  // 128 tiles / 16
+        big.len = 900;
+        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&big, 0, 8, 100) == 0);   // under 32 key tiles
+        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&big, 1, 8, 100) > 0);    // device lengths: the bound is S_max
+        big.len = 4096;
+        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&big, 0, 64, 1024) == 0); // 512 workgroups already
+        big.D = 64;
+        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&big, 0, 8, 100) == 0);
+        big.D = 128;
+        big.format = VSP_KV_Q8_0;
+        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&big, 0, 8, 100) == 0);
+        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(nullptr, 0, 8, 100) == 0);
+        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&big, 0, 0, 100) == 0);
+    }
 }
 
 int main() {

@@ -168,6 +168,104 @@ def test_module_level_prefill_reads_the_planes_in_place(va, fmt, monkeypatch):
         va.attention_core(G.to_bf16_dev(q), G.to_bf16_dev(k), G.to_bf16_dev(v), va.KVCache(B, Hkv, 200, D, fmt=fmt), 5)
 
 
+def _chunk_rows64(q, k, v, L, causal):
+    """float64 attention of the chunk rows q [B,Hq,T,D] (the last T of L tokens) over k, v [B,Hkv,>=L,D]."""
+    B, Hq, T, D = q.shape
+    n = Hq // k.shape[1]
+    out = np.empty((B, Hq, T, D))
+    for b in range(B):
+        for h in range(Hq):
+            kk, vv = k[b, h // n, :L].astype(np.float64), v[b, h // n, :L].astype(np.float64)
+            s = q[b, h].astype(np.float64) @ kk.T / math.sqrt(D)
+            if causal:
+                s = np.where(np.arange(L)[None, :] <= (L - T + np.arange(T))[:, None], s, -np.inf)
+            p = np.exp(s - s.max(-1, keepdims=True))
+            out[b, h] = (p / p.sum(-1, keepdims=True)) @ vv
+    return out
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,T,L,causal", [(1, 8, 2, 100, 3000, True), (1, 8, 2, 100, 3000, False), (2, 8, 2, 300, 5000, True),
+                                                (1, 4, 1, 8, 8000, True), (1, 8, 2, 128, 1030, True)])
+def test_bf16_context_split_over_workgroups(va, B, Hq, Hkv, T, L, causal):
+    # a few query tiles over a long context: with the split workspace the context is cut into shares of >= 512 keys
+    # (5, 5, 9, 15 and 2 shares here), each written as a partial and merged by the decode step's combine kernel
+    D, S_max = 128, (L + 63) // 64 * 64
+    q, k, v = [O.bf16_round(x * np.float32(0.5)) for x in I.qkv(3300 + L + T, B, Hq, Hkv, T, L, D)]
+    c = va.KVCache(B, Hkv, S_max, D, fmt="bf16")
+    c.update(G.to_bf16_dev(k), G.to_bf16_dev(v), 0, return_views=False)
+    from vesper_amd import _ffi
+    import ctypes as C
+    assert _ffi.lib.vsp_attn_prefill_cached_split_workspace_bytes(C.byref(c._c), 0, Hq, T) > 0
+    tq = G.to_bf16_dev(q)
+    got = c.prefill(tq, is_causal=causal)
+    G.assert_bf16_close(G.bf16_to_np(got), _chunk_rows64(q, k, v, L, causal).astype(np.float32), "split")
+    assert torch.equal(got, c.prefill(tq, is_causal=causal))          # fixed merge order
+    whole = c.prefill(tq, is_causal=causal, split=False)
+    d = (got.float() - whole.float()).abs()
+    assert d.max().item() <= 1.6e-2 and d.mean().item() <= 1e-3
+    # with lse requested the call runs unsplit (the partials do not carry it)
+    o2, lse = c.prefill(tq, is_causal=causal, return_lse=True)
+    assert torch.equal(o2, whole) and torch.isfinite(lse).all()
+
+
+def test_bf16_context_split_ragged_rows_and_stale_tokens(va):
+    # per-row context and chunk lengths on the device, one row shorter than a share, stale NaN / Inf tokens past every length
+    B, Hq, Hkv, T, D, S_max = 3, 8, 2, 96, 128, 4096
+    lens = np.array([4000, 300, 1777], dtype=np.int32)
+    nq = np.array([96, 50, 7], dtype=np.int32)
+    q, k, v = [O.bf16_round(x * np.float32(0.5)) for x in I.qkv(3400, B, Hq, Hkv, T, S_max, D)]
+    kk, vv = G.to_bf16_dev(k).clone(), G.to_bf16_dev(v).clone()
+    for b in range(B):
+        kk[b, :, lens[b]:] = float("nan")
+        vv[b, :, lens[b]:] = float("inf")
+    c = va.KVCache(B, Hkv, S_max, D, fmt="bf16")
+    c.update(kk, vv, 0, return_views=False)
+    sl, cl = torch.from_numpy(lens).to(G.dev()), torch.from_numpy(nq).to(G.dev())
+    got = c.prefill(G.to_bf16_dev(q), seq_lens=sl, chunk_lens=cl)
+    whole = c.prefill(G.to_bf16_dev(q), seq_lens=sl, chunk_lens=cl, split=False)
+    for b in range(B):
+        n, L = int(nq[b]), int(lens[b])
+        want = _chunk_rows64(q[b:b + 1, :, :n], k[b:b + 1], v[b:b + 1], L, True).astype(np.float32)
+        G.assert_bf16_close(G.bf16_to_np(got[b:b + 1, :, :n]), want, f"row {b}")
+        assert (got[b, :, :n].float() - whole[b, :, :n].float()).abs().max().item() <= 1.6e-2
+
+
+def test_bf16_context_split_over_pages(va):
+    # the same over a paged cache with a shuffled page table: shares cross page boundaries
+    B, Hq, Hkv, T, D, S_max, P = 2, 8, 2, 64, 128, 2048, 128
+    n_pages = B * (S_max // P) + 3
+    flat = va.RaggedKVCache(B, Hkv, S_max, D, fmt="bf16")
+    paged = va.RaggedKVCache(B, Hkv, S_max, D, fmt="bf16", paging=(P, n_pages))
+    perm = np.random.default_rng(9).permutation(n_pages)[:B * (S_max // P)].astype(np.int32).reshape(B, S_max // P)
+    paged.page_table.copy_(torch.from_numpy(perm))
+    q, k, v = [O.bf16_round(x * np.float32(0.5)) for x in I.qkv(3500, B, Hq, Hkv, T, 2000, D)]
+    outs = []
+    for c in (flat, paged):
+        c.append(G.to_bf16_dev(k), G.to_bf16_dev(v))
+        outs.append(c.prefill_chunk(G.to_bf16_dev(q)))
+    assert torch.equal(outs[0], outs[1])
+    G.assert_bf16_close(G.bf16_to_np(outs[1]), _chunk_rows64(q, k, v, 2000, True).astype(np.float32), "paged")
+
+
+def test_context_split_is_not_offered_where_it_cannot_help(va):
+    from vesper_amd import _ffi
+    import ctypes as C
+    f = _ffi.lib.vsp_attn_prefill_cached_split_workspace_bytes
+    c = va.KVCache(1, 2, 4096, 128, fmt="bf16")
+    c.set_len(4096)
+    assert f(C.byref(c._c), 0, 8, 100) == 1 * 8 * 100 * 8 * 130 * 4      # 128 tiles, 8 workgroups: 8 shares of 16 tiles
+    c.set_len(900)
+    assert f(C.byref(c._c), 0, 8, 100) == 0                              # under 32 tiles
+    assert f(C.byref(c._c), 1, 8, 100) > 0                               # with device lengths the bound is S_max
+    big = va.KVCache(4, 8, 4096, 128, fmt="bf16")
+    big.set_len(4096)
+    assert f(C.byref(big._c), 0, 32, 512) == 0                           # 512 workgroups already
+    for fmt, D in (("q8_0", 128), ("bf16", 64)):
+        o = va.KVCache(1, 2, 4096, D, fmt=fmt)
+        o.set_len(4096)
+        assert f(C.byref(o._c), 0, 8, 100) == 0
+
+
 def test_argument_errors(va):
     q = torch.zeros(1, 4, 8, 64, device=G.dev(), dtype=torch.bfloat16)
     c = va.KVCache(1, 2, 64, 64, fmt="bf16")

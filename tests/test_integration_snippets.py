@@ -25,7 +25,7 @@ BLOCKS = [
      f"int32_t max_seq_len, int32_t head_dim_, float rope_base_, const float*& rope_table_, const float* (*upload)(const std::vector<float>&), "
      f"{_T} q_view, {_T} k_view, {_T} v_view, {_T} q_rot, vsp_kv_cache cache_desc, int64_t start_pos, void* stream"),
     ("chunked prefill over the cache", "function",
-     "vsp_tensor dq_rot, vsp_tensor dout, vsp_kv_cache cache_desc, int D, void* workspace, void* stream"),
+     "vsp_tensor dq_rot, vsp_tensor dout, vsp_kv_cache cache_desc, int32_t Hq, int32_t T, int D, void* workspace, void* stream"),
     ("a few tokens per sequence through the decode kernels", "function",
      "vsp_tensor dq_rot, vsp_tensor dout, vsp_kv_cache cache_desc, int32_t B, int32_t T, int32_t Hq, int D, void* workspace, void* stream"),
     ("flash_attention_backward_hip_dispatch", "global", ""),

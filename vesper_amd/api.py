@@ -179,9 +179,10 @@ class KVCache:
                                      C.c_void_p(rope.table.data_ptr()), rope.length, int(start_pos), sp, _stream(q)))
         return (q_out, self.views()) if return_views else q_out
 
-    def prefill(self, q, seq_lens=None, is_causal=True, scale=None, return_lse=False, chunk_lens=None):
+    def prefill(self, q, seq_lens=None, is_causal=True, scale=None, return_lse=False, chunk_lens=None, split=True):
         """Attention of the last T tokens (q [B,Hq,T,D]) over the cached context, read in place from the planes:
-        chunked prefill.  seq_lens: device int32[B] per-row context lengths (default: the cache's one length)."""
+        chunked prefill.  seq_lens: device int32[B] per-row context lengths (default: the cache's one length).
+        split=False withholds the workspace that lets the library split a long context over workgroups."""
         out = torch.empty_like(q)
         lse = torch.empty(q.shape[:3], dtype=torch.float32, device=q.device) if return_lse else None
         dq, do = _desc(q), _desc(out)
@@ -190,6 +191,9 @@ class KVCache:
         cl = C.c_void_p(chunk_lens.data_ptr()) if chunk_lens is not None else None
         sc = float(scale) if scale is not None else 1.0 / math.sqrt(q.shape[-1])
         nws = lib.vsp_attn_prefill_cached_workspace_bytes(C.byref(self._c), int(seq_lens is not None))
+        if not return_lse and split:  # a few query tiles over a long context: the context is split over workgroups
+            nws = max(nws, lib.vsp_attn_prefill_cached_split_workspace_bytes(C.byref(self._c), int(seq_lens is not None),
+                                                                            q.shape[1], q.shape[2]))
         ws = torch.empty(nws, dtype=torch.uint8, device=q.device) if nws else None
         check(lib.vsp_attn_prefill_cached(C.byref(dq), C.byref(self._c), sl, cl, C.byref(do),
                                           C.byref(dl) if dl is not None else None, sc, int(bool(is_causal)),

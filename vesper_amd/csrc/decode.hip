@@ -1078,6 +1078,29 @@ int pick_chunk(int format, int64_t B, int64_t Hkv, int64_t max_len) {
 }
 
 }  // namespace
+
+// out[b][h][t][:] from the split-K partials ws_o [B][Hq][T][max_splits][D], ws_ml [..][2] = (m in the log2 domain, l): the
+// combine of the decode step, also used by the context-split prefill over a cache.  A row's split count is
+// ceil(its length / chunk), its length seq_lens[b] (or len) clamped to [0, L_cap].
+int launch_split_combine(const float* ws_o, const float* ws_ml, const int32_t* seq_lens, int32_t len, int32_t chunk, int32_t max_splits,
+                         int64_t B, int64_t Hq, int64_t T, int64_t D, int32_t L_cap, vsp_tensor* out, hipStream_t st) {
+    dim3 cgrid((unsigned)(Hq * T), (unsigned)B);
+    const int cthreads = D <= 64 ? 64 : (D <= 128 ? 128 : 256);
+    auto combine = [&](auto out_tag, auto blk) {
+        using OutT = decltype(out_tag);
+        hipLaunchKernelGGL((decode_combine_kernel<OutT, decltype(blk)::value>), cgrid, dim3(cthreads), 0, st, ws_o, ws_ml, seq_lens, len,
+                           chunk, max_splits, (int)Hq, (int)D, (OutT*)out->data, out->stride[0], out->stride[1], L_cap, (int)T,
+                           out->stride[2]);
+    };
+    auto combine_blk = [&](auto out_tag) {
+        if (max_splits <= 8) combine(out_tag, std::integral_constant<int, 8>{});
+        else if (max_splits <= 16) combine(out_tag, std::integral_constant<int, 16>{});
+        else combine(out_tag, std::integral_constant<int, 32>{});
+    };
+    if (out->dtype == VSP_F32) combine_blk(float{});
+    else combine_blk(uint16_t{});
+    return check_launch();
+}
 }  // namespace vsp
 
 using namespace vsp;
@@ -1226,22 +1249,8 @@ int decode_impl(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* s
         if (rc != VSP_OK) return rc;
     }
     // with max_len == 0 every row is empty: the combine kernel reads nothing and writes zeros
-    dim3 cgrid((unsigned)(Hq * T), (unsigned)B);
-    const int cthreads = D <= 64 ? 64 : (D <= 128 ? 128 : 256);
-    auto combine = [&](auto out_tag, auto blk) {
-        using OutT = decltype(out_tag);
-        hipLaunchKernelGGL((decode_combine_kernel<OutT, decltype(blk)::value>), cgrid, dim3(cthreads), 0, st, a.ws_o, a.ws_ml, seq_lens,
-                           max_len > 0 ? cache->len : 0, chunk, max_splits, (int)Hq, (int)D, (OutT*)out->data, out->stride[0],
-                           out->stride[1], a.L_cap, (int)T, out->stride[2]);
-    };
-    auto combine_blk = [&](auto out_tag) {
-        if (max_splits <= 8) combine(out_tag, std::integral_constant<int, 8>{});
-        else if (max_splits <= 16) combine(out_tag, std::integral_constant<int, 16>{});
-        else combine(out_tag, std::integral_constant<int, 32>{});
-    };
-    if (out->dtype == VSP_F32) combine_blk(float{});
-    else combine_blk(uint16_t{});
-    return check_launch();
+    return launch_split_combine(a.ws_o, a.ws_ml, seq_lens, max_len > 0 ? cache->len : 0, chunk, max_splits, B, Hq, T, D, a.L_cap,
+                                out, st);
 }
 
 // vsp_attn_decode_proj's workspace: the merged heads x [B][Hq*D] (4 bytes an element whatever the dtype), the

@@ -29,6 +29,7 @@
 // the mask is evaluated only on tiles that straddle it.
 #include <math.h>
 
+#include <algorithm>
 #include <utility>
 
 #include "kv_layout.hpp"
@@ -59,6 +60,12 @@ struct PrefillArgs {
     // the caller's fp32 tensor
     const void* k_lo;
     const void* v_lo;
+    // cache-plane mode, context split over workgroups (n_splits > 1): split s of a query tile covers key tiles
+    // [s * split_tiles, (s + 1) * split_tiles) and writes an unnormalised partial instead of the output, row
+    // ((b * Hq + hq) * T + t) * n_splits + s of ws_o [..][D] and ws_ml [..][2] = (m in the log2 domain, l)
+    int32_t n_splits, split_tiles;
+    float* ws_o;
+    float* ws_ml;
 };
 
 constexpr int kBM = 128;       // queries per workgroup
@@ -807,7 +814,17 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_pipe_kernel(PrefillArgs a
     const uint32_t lds0 = lds_addr(smem);
 
     const int nbh = a.B * a.Hq;
-    const int bid = blockIdx.x;
+    int bid = blockIdx.x;
+    int tile0 = 0;  // first key tile of this workgroup's share of the context (a split context: cache-plane mode only)
+    int split = 0;
+    if constexpr (VBLK) {
+        if (a.n_splits > 1) {
+            const int inner = a.n_qtiles * nbh;
+            split = bid / inner;
+            bid -= split * inner;
+            tile0 = split * a.split_tiles;
+        }
+    }
     const int qt = a.n_qtiles - 1 - bid / nbh;
     const int pos = bid % nbh;
     int bh = pos;
@@ -856,13 +873,20 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_pipe_kernel(PrefillArgs a
 
     const int wg_qmax = min(qt * kBM + kBM - 1, a.T - 1);
     const int kv_end_wg = a.causal ? min(L, wg_qmax + off + 1) : L;
-    const int n_tiles = (kv_end_wg + kUnit - 1) / kUnit;  // tiles the workgroup loads
+    int n_tiles = (kv_end_wg + kUnit - 1) / kUnit;  // tiles the workgroup loads
     const int wave_qmax = min(q0 + 31, a.T - 1);
     const int kv_end_wave = (q0 < a.T) ? (a.causal ? min(L, wave_qmax + off + 1) : L) : 0;
-    const int nt_w = (kv_end_wave + kUnit - 1) / kUnit;  // tiles this wavefront uses
+    int nt_w = (kv_end_wave + kUnit - 1) / kUnit;  // tiles this wavefront uses
     // first tile of this wavefront that needs the mask (straddles the diagonal or the end of the context)
     int first_masked = min(nt_w, L / kUnit);
     if (a.causal) first_masked = min(first_masked, q0 + off - 31 < 0 ? 0 : (q0 + off - 31) / kUnit + 1);
+    if constexpr (VBLK) {
+        if (a.n_splits > 1) {  // this workgroup's share: tiles [tile0, tile0 + split_tiles), counted from tile0 below
+            n_tiles = max(0, min(n_tiles, tile0 + a.split_tiles) - tile0);
+            nt_w = min(max(0, nt_w - tile0), n_tiles);
+            first_masked = min(max(0, first_masked - tile0), nt_w);
+        }
+    }
     const int n_fast = max(0, first_masked - 2);  // steps [0, n_fast): all three stages active, no mask
     const int n_mid = max(0, nt_w - 2);           // steps [0, n_mid): all three stages active
 
@@ -908,7 +932,7 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_pipe_kernel(PrefillArgs a
     auto load_k_tile = [&](int t, int slot) {
         const char *kb, *vb;
         int local, cap, rows;
-        locate_tile(t * kUnit, kb, vb, local, cap, rows);
+        locate_tile((tile0 + t) * kUnit, kb, vb, local, cap, rows);
         __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc((void*)(kb + (int64_t)local * rowK), 0, (int)((int64_t)rows * rowK), 0x00020000);
         uint16_t* dst = smem + slot * SLOT;
 #pragma unroll
@@ -918,7 +942,7 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_pipe_kernel(PrefillArgs a
     auto load_v_tile = [&](int t, int slot) {
         const char *kb, *vb;
         int local, cap, rows;
-        locate_tile(t * kUnit, kb, vb, local, cap, rows);
+        locate_tile((tile0 + t) * kUnit, kb, vb, local, cap, rows);
         // VBLK: 32 tokens = 4 token blocks = kUnit * D contiguous elements; bound = the rest of this head's slab
         const int64_t v_base = VBLK ? (int64_t)local * D * 2 : (int64_t)local * rowV;
         const int64_t v_bytes = VBLK ? ((int64_t)cap - local) * D * 2 : (int64_t)rows * rowV;
@@ -1038,7 +1062,7 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_pipe_kernel(PrefillArgs a
                 if (pv_on) {
                     if constexpr (VBLK && MODE >= 2) {
                         // the planes hold stale tokens past L: P is 0 there, V must not be NaN
-                        const int nvalid = L - (tau * kUnit + 16 * j + 8 * h);  // slots e >= nvalid are past the context
+                        const int nvalid = L - ((tile0 + tau) * kUnit + 16 * j + 8 * h);  // slots e >= nvalid are past the context
                         if (nvalid < 8) {
 #pragma unroll
                             for (int w = 0; w < 4; ++w) {
@@ -1064,7 +1088,7 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_pipe_kernel(PrefillArgs a
             }
             if constexpr (MASK && S == 12) {
                 if (qk_on) {
-                    const int k0 = (tau + 2) * kUnit;
+                    const int k0 = (tile0 + tau + 2) * kUnit;
                     if ((a.causal && k0 + kUnit - 1 > q0 + off) || (k0 + kUnit > L)) {
                         const int q_abs = q0 + ql + off;
                         const int lim = a.causal ? min(q_abs, L - 1) : L - 1;
@@ -1168,6 +1192,25 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_pipe_kernel(PrefillArgs a
 
     l = half_swap_sum(l);
     const int qi = q0 + ql;
+    if constexpr (VBLK) {
+        if (a.n_splits > 1) {  // the unnormalised partial of this share of the context; the combine kernel finishes the row
+            if (qi < a.T) {
+                const int64_t row = (((int64_t)b * a.Hq + hq) * a.T + qi) * a.n_splits + split;
+                float* po = a.ws_o + row * D;
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+#pragma unroll
+                    for (int vq = 0; vq < 4; ++vq)
+                        *(float4*)(po + 32 * db + 8 * vq + 4 * h) = float4{acc[db][4 * vq], acc[db][4 * vq + 1], acc[db][4 * vq + 2], acc[db][4 * vq + 3]};
+                if (h == 0) {  // a row that met no key in this share (masked, or the share lies past its diagonal) says so
+                    a.ws_ml[row * 2] = l > 0.f ? m_ref : -INFINITY;
+                    a.ws_ml[row * 2 + 1] = l;
+                }
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            return;
+        }
+    }
     if (qi < a.T) {
         const float inv_l = l > 0.f ? 1.0f / l : 0.f;
         uint16_t* op = (uint16_t*)a.out + (int64_t)b * a.so[0] + (int64_t)hq * a.so[1] + (int64_t)qi * a.so[2];
@@ -1355,6 +1398,38 @@ int check_kv_cache(const vsp_kv_cache* c);  // kv_cache.hip
 
 using namespace vsp;
 
+namespace {
+// Context split for a chunk over a long cached context (bf16 planes, head_dim 128): the grid of a few query tiles
+// leaves most of the chip idle while each workgroup walks the whole context, so the context is cut into shares of
+// split_tiles key tiles, one workgroup per (query tile, head, share), and the decode step's combine kernel merges the
+// partials.  Shares are at least 16 tiles (512 keys) long and as many as it takes to reach two workgroups per CU.
+struct SplitChoice {
+    int n_splits, split_tiles;
+};
+SplitChoice plan_context_split(const vsp_kv_cache* cache, int64_t Hq, int64_t T, int64_t L) {
+    SplitChoice c{1, 0};
+    if (cache->format != VSP_KV_BF16 || cache->D != 128) return c;
+    const int64_t inner = ceil_div(T, kBM) * cache->B * Hq;
+    const int64_t slots = 2 * (int64_t)device_cu_count();
+    const int64_t tiles = ceil_div(L, kUnit);
+    if (inner <= 0 || inner * 2 > slots || tiles < 32) return c;
+    int64_t n = std::min<int64_t>(ceil_div(slots, inner), tiles / 16);
+    n = std::min<int64_t>(n, 64);
+    if (n <= 1) return c;
+    c.split_tiles = (int)ceil_div(tiles, n);
+    c.n_splits = (int)ceil_div(tiles, c.split_tiles);
+    return c;
+}
+}  // namespace
+
+extern "C" size_t vsp_attn_prefill_cached_split_workspace_bytes(const vsp_kv_cache* cache, int with_seq_lens, int32_t Hq, int32_t T) {
+    if (!cache || Hq <= 0 || T <= 0) return 0;
+    const int64_t L = with_seq_lens ? cache->S_max : cache->len;
+    const SplitChoice c = plan_context_split(cache, Hq, T, L);
+    if (c.n_splits <= 1) return 0;
+    return (size_t)cache->B * (size_t)Hq * (size_t)T * (size_t)c.n_splits * (size_t)(cache->D + 2) * sizeof(float);
+}
+
 extern "C" size_t vsp_attn_prefill_cached_workspace_bytes(const vsp_kv_cache* cache, int with_seq_lens) {
     if (!cache || cache->format != VSP_KV_Q8_0) return 0;
     const int64_t rows = with_seq_lens ? cache->S_max : cache->len;
@@ -1450,6 +1525,24 @@ extern "C" int vsp_attn_prefill_cached(const vsp_tensor* q, const vsp_kv_cache* 
     a.n_qtiles = (int)ceil_div(T, kBM);
     a.negate_q = (q->dtype == VSP_BF16 && scale < 0.0f) ? 1 : 0;
     a.scale_log2 = (q->dtype == VSP_BF16 ? fabsf(scale) : scale) * kLog2e;
+    // a caller that brings the workspace of vsp_attn_prefill_cached_split_workspace_bytes gets the context split over
+    // workgroups when the grid would otherwise leave the chip idle (no lse in that mode: the partials do not carry it)
+    if (!lse && workspace && is_aligned16(workspace)) {
+        const SplitChoice c = plan_context_split(cache, Hq, T, L);
+        const size_t rows = (size_t)B * (size_t)Hq * (size_t)T * (size_t)c.n_splits;
+        if (c.n_splits > 1 && workspace_bytes >= rows * (size_t)(D + 2) * sizeof(float)) {
+            a.n_splits = c.n_splits;
+            a.split_tiles = c.split_tiles;
+            a.ws_o = (float*)workspace;
+            a.ws_ml = a.ws_o + rows * (size_t)D;
+            const int64_t blocks = (int64_t)a.n_qtiles * B * Hq * c.n_splits;
+            if (blocks > INT32_MAX) return VSP_ERR_ARG;
+            hipLaunchKernelGGL(prefill_bf16_pipe_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, a);
+            if ((rc = check_launch()) != VSP_OK) return rc;
+            return launch_split_combine(a.ws_o, a.ws_ml, seq_lens, cache->len, c.split_tiles * kUnit, c.n_splits, B, Hq, T, D, (int)L, out,
+                                        (hipStream_t)stream);
+        }
+    }
     return launch_prefill(a, q->dtype, D, cache->format == VSP_KV_BF16, stream);
 }
 

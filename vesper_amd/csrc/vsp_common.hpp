@@ -51,6 +51,9 @@ __device__ inline uint32_t pack_bf16x2(float a, float b) {
 void set_hip_error(hipError_t e);
 int check_launch();  // VSP_OK or VSP_ERR_LAUNCH after a kernel launch
 int device_cu_count();  // compute units of the device that was current at the first call (256 if the query fails)
+// decode.hip: the split-K combine (decode step; context-split prefill over a cache)
+int launch_split_combine(const float* ws_o, const float* ws_ml, const int32_t* seq_lens, int32_t len, int32_t chunk, int32_t max_splits,
+                         int64_t B, int64_t Hq, int64_t T, int64_t D, int32_t L_cap, vsp_tensor* out, hipStream_t st);
 
 inline bool is_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
