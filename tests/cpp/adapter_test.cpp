@@ -471,6 +471,46 @@ static void test_multi_head_attention_core() {
     }
 }
 
+static void test_chunk_of_a_long_prompt_splits_the_context() {
+    // KVCache::attend with the last 96 tokens of a 4192-token context (bf16 cache, head_dim 128): 8 workgroups of queries
+    // for the whole chip, so attend() brings the split workspace and the library cuts the context into shares.  Expected:
+    // the rows of the causal forward over the whole context, in double precision on the values the cache holds.
+    std::printf("test_chunk_of_a_long_prompt_splits_the_context\n");
+    const int64_t B = 1, Hq = 8, Hkv = 2, D = 128, L = 4192, T = 96, S_max = 4224, n_rep = Hq / Hkv;
+    auto k = bf16_round(randn(B * Hkv * L * D, 71, 0.5f)), v = bf16_round(randn(B * Hkv * L * D, 72, 0.5f));
+    auto q = bf16_round(randn(B * Hq * T * D, 73, 0.5f));
+    nn::GQAKVCache cache(B, Hkv, S_max, D, Device::HIP, KVFormat::BFloat16);
+    cache.update(to_dev(k, {B, Hkv, L, D}, DType::BFloat16), to_dev(v, {B, Hkv, L, D}, DType::BFloat16), 0);
+    CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&cache.raw(), 0, (int32_t)Hq, (int32_t)T) > 0);
+    auto got = to_host(cache.attend(to_dev(q, {B, Hq, T, D}, DType::BFloat16), true));
+    const double scale = 1.0 / std::sqrt((double)D);
+    double worst = 0;
+    std::vector<double> s((size_t)L), o((size_t)D);
+    for (int64_t h = 0; h < Hq; ++h)
+        for (int64_t t = 0; t < T; t += 5) {  // every fifth row
+            const int64_t last = L - T + t;  // keys [0, last]
+            const float* qp = &q[(size_t)((h * T + t) * D)];
+            const float* kp = &k[(size_t)((h / n_rep) * L * D)];
+            const float* vp = &v[(size_t)((h / n_rep) * L * D)];
+            double m = -1e300, l = 0;
+            for (int64_t j = 0; j <= last; ++j) {
+                double d = 0;
+                for (int64_t e = 0; e < D; ++e) d += (double)qp[e] * kp[j * D + e];
+                s[(size_t)j] = d * scale;
+                m = std::fmax(m, s[(size_t)j]);
+            }
+            std::fill(o.begin(), o.end(), 0.0);
+            for (int64_t j = 0; j <= last; ++j) {
+                const double p = std::exp(s[(size_t)j] - m);
+                l += p;
+                for (int64_t e = 0; e < D; ++e) o[(size_t)e] += p * vp[j * D + e];
+            }
+            for (int64_t e = 0; e < D; ++e) worst = std::fmax(worst, std::fabs(o[(size_t)e] / l - (double)got[(size_t)((h * T + t) * D + e)]));
+        }
+    if (!(worst < 2e-2)) std::printf("  max-abs %.3g\n", worst);
+    CHECK(worst < 2e-2);
+}
+
 static void test_token_loop_allocates_nothing_and_keeps_pace() {
     // One decode step of the drop-in layer = forward_rope (RoPE + append, split-K decode + combine).  After warm-up the
     // step must not reach the driver's allocator and must not wait for the stream; its time per token is compared with
@@ -545,6 +585,7 @@ int main(int argc, char** argv) {
         test_sdpa_routing();
         test_backward_dispatch_seam();
         test_multi_head_attention_core();
+        test_chunk_of_a_long_prompt_splits_the_context();
         run_token_with_output_projection(KVFormat::Float32, DType::Float32, 1e-4, "f32");
         run_token_with_output_projection(KVFormat::BFloat16, DType::BFloat16, 1e-2, "bf16");
         test_token_loop_allocates_nothing_and_keeps_pace();
