@@ -191,10 +191,10 @@ class KVCache:
         cl = C.c_void_p(chunk_lens.data_ptr()) if chunk_lens is not None else None
         sc = float(scale) if scale is not None else 1.0 / math.sqrt(q.shape[-1])
         nws = lib.vsp_attn_prefill_cached_workspace_bytes(C.byref(self._c), int(seq_lens is not None))
-        if not return_lse and split:  # a few query tiles over a long context: the context is split over workgroups
-            nws = max(nws, lib.vsp_attn_prefill_cached_split_workspace_bytes(C.byref(self._c), int(seq_lens is not None),
-                                                                            q.shape[1], q.shape[2]))
         ws = torch.empty(nws, dtype=torch.uint8, device=q.device) if nws else None
+        if not nws and not return_lse and split:  # a few query tiles over a long context: the context is split over workgroups
+            nws = lib.vsp_attn_prefill_cached_split_workspace_bytes(C.byref(self._c), int(seq_lens is not None), q.shape[1], q.shape[2])
+            ws = _workspace(q.device, nws) if nws else None   # the per-stream block the decode step uses (bounded: <= 70 MB)
         check(lib.vsp_attn_prefill_cached(C.byref(dq), C.byref(self._c), sl, cl, C.byref(do),
                                           C.byref(dl) if dl is not None else None, sc, int(bool(is_causal)),
                                           C.c_void_p(ws.data_ptr()) if ws is not None else None, nws, _stream(q)))
