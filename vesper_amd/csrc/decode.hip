@@ -1067,10 +1067,11 @@ __global__ void __launch_bounds__(256) proj_f32_kernel(const float* __restrict__
 // (counted with the host's upper bound of the lengths).  Measured on small batches, where it matters (one sequence,
 // 32k context: 25.6 us with 1024-token splits against 34.6 us with 256-token ones); a large batch reaches the cap
 // whatever the threshold.  The quantised kernel has the heavier per-item cost and the lighter stream, hence its larger
-// cap.  Workspace sizing assumes >= 256.
-int pick_chunk(int format, int64_t B, int64_t Hkv, int64_t max_len) {
+// cap; a step of several tokens per sequence writes that many partial rows per split, hence its (+3 % at batch 32,
+// four tokens, contexts of 1k-32k).  Workspace sizing assumes >= 256.
+int pick_chunk(int format, int64_t B, int64_t Hkv, int64_t max_len, int64_t tokens) {
     const int64_t want = device_cu_count() / 2;
-    const int cap = format == VSP_KV_Q8_0 ? 8192 : 1024;
+    const int cap = format == VSP_KV_Q8_0 ? 8192 : (tokens > 1 ? 2048 : 1024);
     for (int chunk = cap; chunk > 256; chunk >>= 1) {
         if (B * Hkv * ceil_div(max_len, chunk) >= want) return chunk;
     }
@@ -1174,7 +1175,7 @@ int decode_impl(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* s
     if (max_len == 0) max_len = seq_lens ? cache->S_max : cache->len;
     hipStream_t st = (hipStream_t)stream;
 
-    const int chunk = max_len > 0 ? pick_chunk(cache->format, B, cache->Hkv, max_len) : 256;
+    const int chunk = max_len > 0 ? pick_chunk(cache->format, B, cache->Hkv, max_len, T) : 256;
     const int max_splits = max_len > 0 ? (int)ceil_div(max_len, chunk) : 1;
     const size_t need = (size_t)(B * Hq * T * max_splits * (D + 2) * 4);
     if (own_scratch) {
