@@ -249,7 +249,10 @@ int vsp_attn_prefill_backward_split(const vsp_tensor* dout, const vsp_tensor* q,
  * [L-T, L) of the reference's full causal forward over L tokens, src/ops/flash_attention.cpp:218-364):
  * q [B,Hq,T,D] holds the LAST T tokens of each context, whose K/V are already in the cache
  * (vsp_kv_append / vsp_rope_kv_append first).  Context length: cache->len, or seq_lens[b] (device int32[B],
- * T <= seq_lens[b] <= S_max; values are clamped to that range) for ragged batches.  Query t attends keys
+ * T <= seq_lens[b] <= max_len; values are clamped to that range) for ragged batches.  max_len: host-side upper
+ * bound of L_b, as in vsp_attn_decode (0 = cache->len if seq_lens is NULL, else S_max): the launch, the Q8_0 read-out
+ * and the context split are planned on it, so a batch whose longest row is far below the capacity should say so.
+ * max_len < 0 or > S_max, or cache->len > max_len > 0 with seq_lens NULL, is VSP_ERR_ARG.  Query t attends keys
  * j <= L_b - T + t when is_causal, all L_b keys otherwise.
  *   VSP_KV_F32 : q/out fp32, fp32 arithmetic.   VSP_KV_BF16 : q/out bf16; K rows and token-blocked V are
  *   consumed in place (V^T operands are plain 16-byte reads of the blocked plane).
@@ -260,15 +263,17 @@ int vsp_attn_prefill_backward_split(const vsp_tensor* dout, const vsp_tensor* q,
  * Tokens past L_b in the planes are never used, whatever they hold.  lse as in vsp_attn_prefill.
  * chunk_lens (nullable): device int32[B], n_b <= T valid query rows per sequence (ragged chunks in one call):
  * query t < n_b sits at position L_b - n_b + t; rows t >= n_b of `out` are unspecified.
- * Context split (VSP_KV_BF16, D = 128, lse == NULL): a chunk of a few query tiles over a long context leaves most of
+ * Context split (VSP_KV_BF16, D = 128): a chunk of a few query tiles over a long context leaves most of
  * the chip idle, each workgroup walking the whole context.  A caller that passes a 16-byte aligned workspace of at
- * least vsp_attn_prefill_cached_split_workspace_bytes(cache, with_seq_lens, Hq, T) bytes (0 when the grid fills the chip
- * anyway, or the context is short) gets the context cut into shares of at least 512 keys, one workgroup per (query
- * tile, head, share), and the partials merged by the decode step's combine kernel in a fixed order.  Without that
- * workspace the call runs unsplit; the results agree within bf16 rounding either way. */
-size_t vsp_attn_prefill_cached_workspace_bytes(const vsp_kv_cache* cache, int with_seq_lens);
-size_t vsp_attn_prefill_cached_split_workspace_bytes(const vsp_kv_cache* cache, int with_seq_lens, int32_t Hq, int32_t T);
-int vsp_attn_prefill_cached(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens,
+ * least vsp_attn_prefill_cached_split_workspace_bytes(cache, with_seq_lens, max_len, Hq, T) bytes (0 when the grid fills
+ * the chip anyway, or the context is short) gets the context cut into shares of at least 512 keys, one workgroup per
+ * (query tile, head, share), and the partials merged by the decode step's combine kernel in a fixed order (lse
+ * included: the partials carry (m, l)).  Without that workspace the call runs unsplit; the results agree within bf16
+ * rounding either way.  The two size functions take the same with_seq_lens (seq_lens != NULL) and max_len as the call. */
+size_t vsp_attn_prefill_cached_workspace_bytes(const vsp_kv_cache* cache, int with_seq_lens, int32_t max_len);
+size_t vsp_attn_prefill_cached_split_workspace_bytes(const vsp_kv_cache* cache, int with_seq_lens, int32_t max_len, int32_t Hq,
+                                                     int32_t T);
+int vsp_attn_prefill_cached(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, int32_t max_len,
                             const int32_t* chunk_lens, vsp_tensor* out, vsp_tensor* lse, float scale, int is_causal,
                             void* workspace, size_t workspace_bytes, void* stream);
 
@@ -315,6 +320,8 @@ int vsp_attn_decode_multi(const vsp_tensor* q, const vsp_kv_cache* cache, const 
  * validation, kernels and results (bit for bit) as vsp_attn_decode, minus the workspace: the split-K
  * partials go to a fixed 32 MiB array that is part of the library's code object (one copy per GPU, held
  * until the process ends), located on the first call on each device.  The call allocates and frees nothing.
+ * The first call on a device looks the array's address up (a lock and two runtime queries, no launch of its own):
+ * make that call outside any stream capture; every later call on that device may be captured.
  * Calls whose partials need more than that -- B * Hq * ceil(max_len / chunk) * (D + 2) * 4 bytes, chunk being
  * the split length the library picks (>= 256 tokens) -- return VSP_ERR_WORKSPACE: config 4 (B 32, 32 heads,
  * D 128, max_len 32768) needs 17 MiB.  Every call on one GPU shares that GPU's array: calls that overlap in

@@ -481,7 +481,7 @@ static void test_chunk_of_a_long_prompt_splits_the_context() {
     auto q = bf16_round(randn(B * Hq * T * D, 73, 0.5f));
     nn::GQAKVCache cache(B, Hkv, S_max, D, Device::HIP, KVFormat::BFloat16);
     cache.update(to_dev(k, {B, Hkv, L, D}, DType::BFloat16), to_dev(v, {B, Hkv, L, D}, DType::BFloat16), 0);
-    CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&cache.raw(), 0, (int32_t)Hq, (int32_t)T) > 0);
+    CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&cache.raw(), 0, 0, (int32_t)Hq, (int32_t)T) > 0);
     auto got = to_host(cache.attend(to_dev(q, {B, Hq, T, D}, DType::BFloat16), true));
     const double scale = 1.0 / std::sqrt((double)D);
     double worst = 0;

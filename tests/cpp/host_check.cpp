@@ -295,10 +295,14 @@ static void test_validation() {
     }
     // cached prefill: the chunk is part of the context, so T = 8 over a context of 4 is a shape error
     c.len = 4;
-    CHECK(vsp_attn_prefill_cached(&q, &c, nullptr, nullptr, &out, nullptr, 0.1f, 1, nullptr, 0, nullptr) == VSP_ERR_SHAPE);
+    CHECK(vsp_attn_prefill_cached(&q, &c, nullptr, 0, nullptr, &out, nullptr, 0.1f, 1, nullptr, 0, nullptr) == VSP_ERR_SHAPE);
     vsp_tensor qf32 = tensor4(mem, VSP_F32, 1, 4, 8, 64);
     c.len = 40;
-    CHECK(vsp_attn_prefill_cached(&qf32, &c, nullptr, nullptr, &qf32, nullptr, 0.1f, 1, nullptr, 0, nullptr) == VSP_ERR_DTYPE);
+    CHECK(vsp_attn_prefill_cached(&qf32, &c, nullptr, 0, nullptr, &qf32, nullptr, 0.1f, 1, nullptr, 0, nullptr) == VSP_ERR_DTYPE);
+    // a host-side length above the caller's own bound, a negative bound, a bound beyond the capacity
+    CHECK(vsp_attn_prefill_cached(&q, &c, nullptr, 39, nullptr, &out, nullptr, 0.1f, 1, nullptr, 0, nullptr) == VSP_ERR_ARG);
+    CHECK(vsp_attn_prefill_cached(&q, &c, nullptr, -1, nullptr, &out, nullptr, 0.1f, 1, nullptr, 0, nullptr) == VSP_ERR_ARG);
+    CHECK(vsp_attn_prefill_cached(&q, &c, nullptr, c.S_max + 1, nullptr, &out, nullptr, 0.1f, 1, nullptr, 0, nullptr) == VSP_ERR_ARG);
     // the context split is offered for bf16 planes at head_dim 128 when a short grid meets a long context, and only then
     {
         vsp_kv_cache big = c;
@@ -307,19 +311,22 @@ static void test_validation() {
         big.D = 128;
         big.S_max = 4096;
         big.len = 4096;
-        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&big, 0, 8, 100) == (size_t)1 * 8 * 100 * 8 * 130 * 4);  // 128 tiles / 16
+        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&big, 0, 0, 8, 100) == (size_t)1 * 8 * 100 * 8 * 130 * 4);  // 128 tiles / 16
         big.len = 900;
-        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&big, 0, 8, 100) == 0);   // under 32 key tiles
-        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&big, 1, 8, 100) > 0);    // device lengths: the bound is S_max
+        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&big, 0, 0, 8, 100) == 0);   // under 32 key tiles
+        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&big, 1, 0, 8, 100) > 0);    // device lengths: the bound is S_max
+        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&big, 1, 900, 8, 100) == 0); // ... unless the caller gives a tighter one
+        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&big, 1, 2048, 8, 100) == (size_t)1 * 8 * 100 * 4 * 130 * 4);  // 64 tiles / 16
+        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&big, 1, -1, 8, 100) == 0);
         big.len = 4096;
-        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&big, 0, 64, 1024) == 0); // 512 workgroups already
+        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&big, 0, 0, 64, 1024) == 0); // 512 workgroups already
         big.D = 64;
-        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&big, 0, 8, 100) == 0);
+        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&big, 0, 0, 8, 100) == 0);
         big.D = 128;
         big.format = VSP_KV_Q8_0;
-        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&big, 0, 8, 100) == 0);
-        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(nullptr, 0, 8, 100) == 0);
-        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&big, 0, 0, 100) == 0);
+        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&big, 0, 0, 8, 100) == 0);
+        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(nullptr, 0, 0, 8, 100) == 0);
+        CHECK(vsp_attn_prefill_cached_split_workspace_bytes(&big, 0, 0, 0, 100) == 0);
     }
 }
 

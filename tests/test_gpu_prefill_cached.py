@@ -142,7 +142,7 @@ def test_q8_0_cache(va):
     qd = G.to_bf16_dev(q[:, :, L - T:])
     od = torch.empty_like(qd)
     dq, do = _desc(qd), _desc(od)
-    rc = _ffi.lib.vsp_attn_prefill_cached(C.byref(dq), C.byref(c._c), None, None, C.byref(do), None, 0.1, 1, None, 0, _stream(qd))
+    rc = _ffi.lib.vsp_attn_prefill_cached(C.byref(dq), C.byref(c._c), None, 0, None, C.byref(do), None, 0.1, 1, None, 0, _stream(qd))
     assert rc == _ffi.ERR_WORKSPACE
 
 
@@ -168,11 +168,12 @@ def test_module_level_prefill_reads_the_planes_in_place(va, fmt, monkeypatch):
         va.attention_core(G.to_bf16_dev(q), G.to_bf16_dev(k), G.to_bf16_dev(v), va.KVCache(B, Hkv, 200, D, fmt=fmt), 5)
 
 
-def _chunk_rows64(q, k, v, L, causal):
+def _chunk_rows64(q, k, v, L, causal, with_lse=False):
     """float64 attention of the chunk rows q [B,Hq,T,D] (the last T of L tokens) over k, v [B,Hkv,>=L,D]."""
     B, Hq, T, D = q.shape
     n = Hq // k.shape[1]
     out = np.empty((B, Hq, T, D))
+    lse = np.empty((B, Hq, T))
     for b in range(B):
         for h in range(Hq):
             kk, vv = k[b, h // n, :L].astype(np.float64), v[b, h // n, :L].astype(np.float64)
@@ -181,7 +182,8 @@ def _chunk_rows64(q, k, v, L, causal):
                 s = np.where(np.arange(L)[None, :] <= (L - T + np.arange(T))[:, None], s, -np.inf)
             p = np.exp(s - s.max(-1, keepdims=True))
             out[b, h] = (p / p.sum(-1, keepdims=True)) @ vv
-    return out
+            lse[b, h] = s.max(-1) + np.log(p.sum(-1))
+    return (out, lse) if with_lse else out
 
 
 @pytest.mark.parametrize("B,Hq,Hkv,T,L,causal", [(1, 8, 2, 100, 3000, True), (1, 8, 2, 100, 3000, False), (2, 8, 2, 300, 5000, True),
@@ -195,7 +197,7 @@ def test_bf16_context_split_over_workgroups(va, B, Hq, Hkv, T, L, causal):
     c.update(G.to_bf16_dev(k), G.to_bf16_dev(v), 0, return_views=False)
     from vesper_amd import _ffi
     import ctypes as C
-    assert _ffi.lib.vsp_attn_prefill_cached_split_workspace_bytes(C.byref(c._c), 0, Hq, T) > 0
+    assert _ffi.lib.vsp_attn_prefill_cached_split_workspace_bytes(C.byref(c._c), 0, 0, Hq, T) > 0
     tq = G.to_bf16_dev(q)
     got = c.prefill(tq, is_causal=causal)
     G.assert_bf16_close(G.bf16_to_np(got), _chunk_rows64(q, k, v, L, causal).astype(np.float32), "split")
@@ -203,9 +205,13 @@ def test_bf16_context_split_over_workgroups(va, B, Hq, Hkv, T, L, causal):
     whole = c.prefill(tq, is_causal=causal, split=False)
     d = (got.float() - whole.float()).abs()
     assert d.max().item() <= 1.6e-2 and d.mean().item() <= 1e-3
-    # with lse requested the call runs unsplit (the partials do not carry it)
+    # lse = m + log l comes out of the merge of the partials' (m, l): against float64 and against the unsplit kernel
     o2, lse = c.prefill(tq, is_causal=causal, return_lse=True)
-    assert torch.equal(o2, whole) and torch.isfinite(lse).all()
+    assert torch.equal(o2, got)
+    _, lse64 = _chunk_rows64(q, k, v, L, causal, with_lse=True)
+    assert np.abs(lse.cpu().numpy() - lse64).max() <= 2e-3     # bf16 P in the row sum: 2^-9 relative on l
+    o3, lse3 = c.prefill(tq, is_causal=causal, return_lse=True, split=False)
+    assert torch.equal(o3, whole) and (lse - lse3).abs().max().item() <= 2e-3
 
 
 def test_bf16_context_split_ragged_rows_and_stale_tokens(va):
@@ -228,6 +234,39 @@ def test_bf16_context_split_ragged_rows_and_stale_tokens(va):
         want = _chunk_rows64(q[b:b + 1, :, :n], k[b:b + 1], v[b:b + 1], L, True).astype(np.float32)
         G.assert_bf16_close(G.bf16_to_np(got[b:b + 1, :, :n]), want, f"row {b}")
         assert (got[b, :, :n].float() - whole[b, :, :n].float()).abs().max().item() <= 1.6e-2
+
+
+def test_bf16_context_split_rows_shorter_than_their_chunk_and_a_host_bound(va):
+    # (i) device lengths below the chunk length (an idle or short row of a ragged batch, chunk_lens NULL): a chunk is part
+    # of its context, so producer and merge both take such a row as T tokens long: split == unsplit on every row.
+    # (ii) the longest row far below the capacity: with max_len the shares are planned on the real bound (8 shares of
+    # 16 tiles over 4096 tokens) instead of on S_max (16 shares of 32 tiles, of which such rows would fill 4).
+    from vesper_amd import _ffi
+    import ctypes as C
+    B, Hq, Hkv, T, D, S_max = 4, 8, 2, 64, 128, 16384
+    lens = np.array([4096, 10, 0, 1500], dtype=np.int32)       # rows 1 and 2 are shorter than the chunk
+    q, k, v = [O.bf16_round(x * np.float32(0.5)) for x in I.qkv(3450, B, Hq, Hkv, T, 4096, D)]
+    c = va.KVCache(B, Hkv, S_max, D, fmt="bf16")
+    c.update(G.to_bf16_dev(k), G.to_bf16_dev(v), 0, return_views=False)
+    f = _ffi.lib.vsp_attn_prefill_cached_split_workspace_bytes
+    per_share = B * Hq * T * 130 * 4
+    assert f(C.byref(c._c), 1, 0, Hq, T) == 16 * per_share and f(C.byref(c._c), 1, 4096, Hq, T) == 8 * per_share
+    sl = torch.from_numpy(lens).to(G.dev())
+    tq = G.to_bf16_dev(q)
+    for max_len in (0, 4096):
+        got, lse = c.prefill(tq, seq_lens=sl, max_len=max_len, return_lse=True)
+        whole, lse_w = c.prefill(tq, seq_lens=sl, max_len=max_len, return_lse=True, split=False)
+        assert (got.float() - whole.float()).abs().max().item() <= 1.6e-2, max_len
+        assert (lse - lse_w).abs().max().item() <= 2e-3, max_len
+        for b in range(B):
+            L = max(int(lens[b]), T)
+            want, lse64 = _chunk_rows64(q[b:b + 1], k[b:b + 1], v[b:b + 1], L, True, with_lse=True)
+            G.assert_bf16_close(G.bf16_to_np(got[b:b + 1]), want.astype(np.float32), f"row {b} max_len {max_len}")
+            assert np.abs(lse[b:b + 1].cpu().numpy() - lse64).max() <= 2e-3
+    # a device length above the host bound is clamped to it, by both kernels alike
+    got = c.prefill(tq, seq_lens=sl, max_len=2048)
+    want = _chunk_rows64(q[:1], k[:1], v[:1], 2048, True).astype(np.float32)
+    G.assert_bf16_close(G.bf16_to_np(got[:1]), want, "clamped to max_len")
 
 
 def test_bf16_context_split_over_pages(va):
@@ -253,17 +292,18 @@ def test_context_split_is_not_offered_where_it_cannot_help(va):
     f = _ffi.lib.vsp_attn_prefill_cached_split_workspace_bytes
     c = va.KVCache(1, 2, 4096, 128, fmt="bf16")
     c.set_len(4096)
-    assert f(C.byref(c._c), 0, 8, 100) == 1 * 8 * 100 * 8 * 130 * 4      # 128 tiles, 8 workgroups: 8 shares of 16 tiles
+    assert f(C.byref(c._c), 0, 0, 8, 100) == 1 * 8 * 100 * 8 * 130 * 4      # 128 tiles, 8 workgroups: 8 shares of 16 tiles
     c.set_len(900)
-    assert f(C.byref(c._c), 0, 8, 100) == 0                              # under 32 tiles
-    assert f(C.byref(c._c), 1, 8, 100) > 0                               # with device lengths the bound is S_max
+    assert f(C.byref(c._c), 0, 0, 8, 100) == 0                           # under 32 tiles
+    assert f(C.byref(c._c), 1, 0, 8, 100) > 0                            # with device lengths the bound is S_max
+    assert f(C.byref(c._c), 1, 900, 8, 100) == 0                         # or the caller's own
     big = va.KVCache(4, 8, 4096, 128, fmt="bf16")
     big.set_len(4096)
-    assert f(C.byref(big._c), 0, 32, 512) == 0                           # 512 workgroups already
+    assert f(C.byref(big._c), 0, 0, 32, 512) == 0                           # 512 workgroups already
     for fmt, D in (("q8_0", 128), ("bf16", 64)):
         o = va.KVCache(1, 2, 4096, D, fmt=fmt)
         o.set_len(4096)
-        assert f(C.byref(o._c), 0, 8, 100) == 0
+        assert f(C.byref(o._c), 0, 0, 8, 100) == 0
 
 
 def test_argument_errors(va):

@@ -70,3 +70,45 @@ def test_noalloc_decode_rejects_oversized_requests(va):
         va.api.check(_ffi.lib.vsp_attn_decode_noalloc(C.byref(va.api._desc(q)), C.byref(c), None, 0,
                                                       C.byref(va.api._desc(out)), 0.1, None))
     assert e.value.status == _ffi.ERR_WORKSPACE
+
+
+def test_noalloc_decode_with_an_empty_context_skips_the_size_check(va):
+    # nothing is attended to and no partial is written, so the 32 MiB bound does not apply: zeros, as vsp_attn_decode
+    B, Hq, Hkv, S, D = 64, 128, 8, 65536, 128
+    import ctypes as C
+    from vesper_amd import _ffi
+    c = _ffi.VspKVCache()
+    c.format, c.B, c.Hkv, c.S_max, c.D = _ffi.KV_BF16, B, Hkv, S, D
+    dummy = torch.zeros(1024, dtype=torch.uint8, device=G.dev())
+    c.k = c.v = dummy.data_ptr()
+    c.len = 0
+    q = torch.ones(B, Hq, 1, D, dtype=torch.bfloat16, device=G.dev())
+    out = torch.full_like(q, float("nan"))
+    va.api.check(_ffi.lib.vsp_attn_decode_noalloc(C.byref(va.api._desc(q)), C.byref(c), None, 0,
+                                                  C.byref(va.api._desc(out)), 0.1, None))
+    torch.cuda.synchronize()
+    assert torch.count_nonzero(out.float()).item() == 0
+
+
+def test_noalloc_decode_replays_from_a_graph_after_one_eager_call(va):
+    # the first call on a device looks the array up and must be eager; after it the entry point can be captured
+    c, qd, sl, _ = _case(va, "bf16", 81, 3, 16, 4, 640, 128, [640, 200, 33])
+    q2 = G.to_bf16_dev(O.bf16_round(I.normal(82, tuple(qd.shape))))
+    eager = []
+    for q in (qd, q2, qd):
+        o = torch.empty_like(q)
+        va.decode_attention_noalloc(q, c, o, seq_lens=sl, max_len=640)
+        eager.append(o)
+    torch.cuda.synchronize()
+    sq, out = torch.empty_like(qd), torch.empty_like(qd)
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            va.decode_attention_noalloc(sq, c, out, seq_lens=sl, max_len=640)
+    torch.cuda.synchronize()
+    for i, q in enumerate((qd, q2, qd)):
+        sq.copy_(q)  # eager work between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager[i]), f"replay {i}"

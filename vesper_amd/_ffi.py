@@ -50,9 +50,9 @@ SYMBOLS = {
     "vsp_attn_prefill_backward": (C.c_int, [_TP] * 9 + [C.c_float, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]),
     "vsp_attn_backward_split_workspace_bytes": (C.c_size_t, [C.c_int32] * 5),
     "vsp_attn_prefill_backward_split": (C.c_int, [_TP] * 9 + [C.c_float, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]),
-    "vsp_attn_prefill_cached_workspace_bytes": (C.c_size_t, [_KP, C.c_int]),
-    "vsp_attn_prefill_cached_split_workspace_bytes": (C.c_size_t, [_KP, C.c_int, C.c_int32, C.c_int32]),
-    "vsp_attn_prefill_cached": (C.c_int, [_TP, _KP, C.c_void_p, C.c_void_p, _TP, _TP, C.c_float, C.c_int, C.c_void_p,
+    "vsp_attn_prefill_cached_workspace_bytes": (C.c_size_t, [_KP, C.c_int, C.c_int32]),
+    "vsp_attn_prefill_cached_split_workspace_bytes": (C.c_size_t, [_KP, C.c_int, C.c_int32, C.c_int32, C.c_int32]),
+    "vsp_attn_prefill_cached": (C.c_int, [_TP, _KP, C.c_void_p, C.c_int32, C.c_void_p, _TP, _TP, C.c_float, C.c_int, C.c_void_p,
                                           C.c_size_t, C.c_void_p]),
     "vsp_seq_lens_advance": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p]),
     "vsp_attn_decode_workspace_bytes": (C.c_size_t, [C.c_int32] * 4),

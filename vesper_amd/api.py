@@ -179,10 +179,11 @@ class KVCache:
                                      C.c_void_p(rope.table.data_ptr()), rope.length, int(start_pos), sp, _stream(q)))
         return (q_out, self.views()) if return_views else q_out
 
-    def prefill(self, q, seq_lens=None, is_causal=True, scale=None, return_lse=False, chunk_lens=None, split=True):
+    def prefill(self, q, seq_lens=None, is_causal=True, scale=None, return_lse=False, chunk_lens=None, split=True, max_len=0):
         """Attention of the last T tokens (q [B,Hq,T,D]) over the cached context, read in place from the planes:
         chunked prefill.  seq_lens: device int32[B] per-row context lengths (default: the cache's one length).
-        split=False withholds the workspace that lets the library split a long context over workgroups."""
+        split=False withholds the workspace that lets the library split a long context over workgroups.
+        max_len: host-side bound of the device-side lengths (0: the cache's capacity), which the split is planned on."""
         out = torch.empty_like(q)
         lse = torch.empty(q.shape[:3], dtype=torch.float32, device=q.device) if return_lse else None
         dq, do = _desc(q), _desc(out)
@@ -190,12 +191,12 @@ class KVCache:
         sl = C.c_void_p(seq_lens.data_ptr()) if seq_lens is not None else None
         cl = C.c_void_p(chunk_lens.data_ptr()) if chunk_lens is not None else None
         sc = float(scale) if scale is not None else 1.0 / math.sqrt(q.shape[-1])
-        nws = lib.vsp_attn_prefill_cached_workspace_bytes(C.byref(self._c), int(seq_lens is not None))
+        nws = lib.vsp_attn_prefill_cached_workspace_bytes(C.byref(self._c), int(seq_lens is not None), int(max_len))
         ws = torch.empty(nws, dtype=torch.uint8, device=q.device) if nws else None
-        if not nws and not return_lse and split:  # a few query tiles over a long context: the context is split over workgroups
-            nws = lib.vsp_attn_prefill_cached_split_workspace_bytes(C.byref(self._c), int(seq_lens is not None), q.shape[1], q.shape[2])
+        if not nws and split:  # a few query tiles over a long context: the context is split over workgroups
+            nws = lib.vsp_attn_prefill_cached_split_workspace_bytes(C.byref(self._c), int(seq_lens is not None), int(max_len), q.shape[1], q.shape[2])
             ws = _workspace(q.device, nws) if nws else None   # the per-stream block the decode step uses (bounded: <= 70 MB)
-        check(lib.vsp_attn_prefill_cached(C.byref(dq), C.byref(self._c), sl, cl, C.byref(do),
+        check(lib.vsp_attn_prefill_cached(C.byref(dq), C.byref(self._c), sl, int(max_len), cl, C.byref(do),
                                           C.byref(dl) if dl is not None else None, sc, int(bool(is_causal)),
                                           C.c_void_p(ws.data_ptr()) if ws is not None else None, nws, _stream(q)))
         return (out, lse) if return_lse else out
@@ -280,7 +281,7 @@ class RaggedKVCache(KVCache):
         T, D = q.shape[2], q.shape[3]
         if n_new is None and T > 1 and T * (q.shape[1] // self._c.Hkv) <= 16 and D in (64, 128):
             return decode_attention_multi(q, self, seq_lens=self.seq_lens, max_len=max(self.upper, 1), scale=scale)
-        return self.prefill(q, seq_lens=self.seq_lens, chunk_lens=n_new, scale=scale)
+        return self.prefill(q, seq_lens=self.seq_lens, chunk_lens=n_new, scale=scale, max_len=max(self.upper, 1))
 
 
 _WS = {}

@@ -348,12 +348,12 @@ public:
             return out;
         }
         // the Q8_0 read-out, or the partials of a context split over workgroups (a few query tiles over a long context)
-        const size_t ws_bytes = std::max(vsp_attn_prefill_cached_workspace_bytes(&st_->c, 0),
-                                         q.ndim() == 4 ? vsp_attn_prefill_cached_split_workspace_bytes(&st_->c, 0, (int32_t)q.shape()[1], (int32_t)T)
+        const size_t ws_bytes = std::max(vsp_attn_prefill_cached_workspace_bytes(&st_->c, 0, 0),
+                                         q.ndim() == 4 ? vsp_attn_prefill_cached_split_workspace_bytes(&st_->c, 0, 0, (int32_t)q.shape()[1], (int32_t)T)
                                                        : size_t{0});
         std::shared_ptr<Storage> ws = ws_bytes ? std::make_shared<Storage>(ws_bytes) : nullptr;
         const float scale = 1.0f / std::sqrt(static_cast<float>(q.shape()[3]));
-        throw_status(vsp_attn_prefill_cached(&dq, &st_->c, nullptr, nullptr, &dout, nullptr, scale, is_causal ? 1 : 0,
+        throw_status(vsp_attn_prefill_cached(&dq, &st_->c, nullptr, 0, nullptr, &dout, nullptr, scale, is_causal ? 1 : 0,
                                              ws ? ws->data() : nullptr, ws_bytes, current_stream()));
         return out;  // the scratch block goes back to the cache; its next user is ordered behind this call on the stream
     }

@@ -86,7 +86,7 @@ __global__ void __launch_bounds__(256) bwd_dq_kernel(BwdArgs a) {
     const int n_qtiles = (a.N + kBQ - 1) / kBQ;
     const int bid = blockIdx.x;
     const int qt = n_qtiles - 1 - bid / (a.B * a.Hq);
-    const int bh = bid % (a.B * a.Hq);
+    const int bh = xcd_grouped_head(bid % (a.B * a.Hq), a.B * a.Hkv, a.n_rep);  // a kv group's query heads share one XCD's L2
     const int b = bh / a.Hq, hq = bh % a.Hq, kvh = hq / a.n_rep;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int ql = lane & 31, h = lane >> 5;
@@ -377,7 +377,7 @@ __global__ void __launch_bounds__(256, SPLIT ? 1 : 2) bwd_dq_bf16_kernel(BwdArgs
     const int n_qtiles = (a.N + kBQ - 1) / kBQ;
     const int bid = blockIdx.x;
     const int qt = n_qtiles - 1 - bid / (a.B * a.Hq);
-    const int bh = bid % (a.B * a.Hq);
+    const int bh = xcd_grouped_head(bid % (a.B * a.Hq), a.B * a.Hkv, a.n_rep);  // a kv group's query heads share one XCD's L2
     const int b = bh / a.Hq, hq = bh % a.Hq, kvh = hq / a.n_rep;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int ql = lane & 31, h = lane >> 5;

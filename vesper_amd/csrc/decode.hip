@@ -831,9 +831,13 @@ template <typename OutT, int BLK>
 __global__ void __launch_bounds__(256) decode_combine_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
                                                              const int32_t* __restrict__ seq_lens, int32_t len, int32_t chunk,
                                                              int32_t max_splits, int32_t Hq, int32_t D, OutT* __restrict__ out,
-                                                             int64_t so_b, int64_t so_h, int32_t L_cap, int32_t T, int64_t so_t) {
+                                                             int64_t so_b, int64_t so_h, int32_t L_cap, int32_t T, int64_t so_t,
+                                                             CombineExtra x) {
     const int hq = blockIdx.x / T, t = blockIdx.x % T, b = blockIdx.y, d = threadIdx.x;
-    const int L = min(max(seq_lens ? seq_lens[b] : len, 0), L_cap);  // the producers' clamp (locate_work)
+    // the producers' clamp: [0, L_cap] in the decode step (locate_work); a chunk of a prompt is part of its context, so
+    // there a row is at least as long as its chunk (prefill_bf16_pipe_kernel)
+    const int len_floor = x.chunk_lens ? min(max(x.chunk_lens[b], 0), x.len_floor) : x.len_floor;
+    const int L = min(max(seq_lens ? seq_lens[b] : len, len_floor), L_cap);
     const int ns = min((L + chunk - 1) / chunk, max_splits);
     const int64_t row0 = (((int64_t)b * Hq + hq) * T + t) * max_splits;
     // One pass over blocks of BLK splits (8, 16 or 32, the smallest that covers the launch's split count): everything a block needs (maxima, sums, partial rows) is requested before any of
@@ -872,6 +876,9 @@ __global__ void __launch_bounds__(256) decode_combine_kernel(const float* __rest
         if constexpr (sizeof(OutT) == 4) *p = r;
         else *p = f32_to_bf16_bits(r);
     }
+    // LSE = m + log l (src/ops/flash_attention.cpp:359), here from the merged (M, l) in the log2 domain; a row that met
+    // no key has l = 0 and reads -inf, as the unsplit kernels write it
+    if (x.lse && d == 0) x.lse[(int64_t)b * x.sl[0] + (int64_t)hq * x.sl[1] + (int64_t)t * x.sl[2]] = (M + __builtin_amdgcn_logf(l)) * 0.6931471805599453f;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1084,14 +1091,15 @@ int pick_chunk(int format, int64_t B, int64_t Hkv, int64_t max_len, int64_t toke
 // combine of the decode step, also used by the context-split prefill over a cache.  A row's split count is
 // ceil(its length / chunk), its length seq_lens[b] (or len) clamped to [0, L_cap].
 int launch_split_combine(const float* ws_o, const float* ws_ml, const int32_t* seq_lens, int32_t len, int32_t chunk, int32_t max_splits,
-                         int64_t B, int64_t Hq, int64_t T, int64_t D, int32_t L_cap, vsp_tensor* out, hipStream_t st) {
+                         int64_t B, int64_t Hq, int64_t T, int64_t D, int32_t L_cap, vsp_tensor* out, hipStream_t st,
+                         const CombineExtra& extra) {
     dim3 cgrid((unsigned)(Hq * T), (unsigned)B);
     const int cthreads = D <= 64 ? 64 : (D <= 128 ? 128 : 256);
     auto combine = [&](auto out_tag, auto blk) {
         using OutT = decltype(out_tag);
         hipLaunchKernelGGL((decode_combine_kernel<OutT, decltype(blk)::value>), cgrid, dim3(cthreads), 0, st, ws_o, ws_ml, seq_lens, len,
                            chunk, max_splits, (int)Hq, (int)D, (OutT*)out->data, out->stride[0], out->stride[1], L_cap, (int)T,
-                           out->stride[2]);
+                           out->stride[2], extra);
     };
     auto combine_blk = [&](auto out_tag) {
         if (max_splits <= 8) combine(out_tag, std::integral_constant<int, 8>{});
@@ -1179,7 +1187,7 @@ int decode_impl(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* s
     const int max_splits = max_len > 0 ? (int)ceil_div(max_len, chunk) : 1;
     const size_t need = (size_t)(B * Hq * T * max_splits * (D + 2) * 4);
     if (own_scratch) {
-        if (need > kScratchBytes) return VSP_ERR_WORKSPACE;
+        if (max_len > 0 && need > kScratchBytes) return VSP_ERR_WORKSPACE;  // an empty context writes no partials
         rc = scratch_for_current_device(&workspace);
         if (rc != VSP_OK) return rc;
     } else if (max_len > 0) {
@@ -1314,11 +1322,13 @@ int vsp_attn_decode_proj(const vsp_tensor* q, const vsp_kv_cache* cache, const i
         if (!wo->data || !y->data || (bias && !bias->data)) return VSP_ERR_NULL;
         if (!is_aligned16(wo->data) || (wo->stride[0] * esz) % 16) return VSP_ERR_ALIGN;
     }
-    if (B <= 0 || Hq <= 0 || D <= 0 || B > INT32_MAX || N > INT32_MAX || K > INT32_MAX) {
-        // shapes the attention step rejects are reported by it; an empty batch has nothing to project
+    if (B <= 0 || Hq <= 0 || D <= 0) {
+        // shapes the attention step rejects are reported by it (it launches nothing for them); an empty batch has
+        // nothing to project
         vsp_tensor none = *q;
         return decode_impl(q, cache, seq_lens, max_len, &none, scale, workspace, workspace_bytes, false, stream);
     }
+    if (B > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return VSP_ERR_ARG;  // the projection kernels index with 32 bits
     // the attention step writes the merged heads x [B][Hq][D] (= [B][K]) to the head of the workspace
     const size_t pb_bytes = proj_part_bytes(B, N);
     const size_t xb = proj_x_bytes(B, Hq, D) + pb_bytes;

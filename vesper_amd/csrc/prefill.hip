@@ -175,14 +175,7 @@ __global__ void __launch_bounds__(256, 3) prefill_bf16_kernel(PrefillArgs a) {
     const int bid = blockIdx.x;
     const int nbh = a.B * a.Hq;
     const int qt = a.n_qtiles - 1 - bid / nbh;
-    const int pos = bid % nbh;
-    int bh = pos;
-    const int ngroups = a.B * a.Hkv;
-    if ((ngroups & 7) == 0) {
-        const int xcd = pos & 7, slot = pos >> 3;
-        const int grp = xcd + 8 * (slot / a.n_rep);
-        bh = grp * a.n_rep + slot % a.n_rep;  // == b * Hq + hq, because groups are numbered b * Hkv + kvh
-    }
+    const int bh = xcd_grouped_head(bid % nbh, a.B * a.Hkv, a.n_rep);
     const int b = bh / a.Hq, hq = bh % a.Hq, kvh = hq / a.n_rep;
     int L = a.L;
     // cache mode: per-row context length (clamped to the bound a.L) and per-row chunk length n <= T:
@@ -530,7 +523,7 @@ __global__ void __launch_bounds__(256, 2) prefill_split_kernel(PrefillArgs a) {
     const int bid = blockIdx.x;
     const int nbh = a.B * a.Hq;
     const int qt = a.n_qtiles - 1 - bid / nbh;  // heaviest query tiles first
-    const int bh = bid % nbh;
+    const int bh = xcd_grouped_head(bid % nbh, a.B * a.Hkv, a.n_rep);  // a kv group's query heads share one XCD's L2
     const int b = bh / a.Hq, hq = bh % a.Hq, kvh = hq / a.n_rep;
     const int L = a.L;
     const int tid = threadIdx.x, lane = tid & 63;
@@ -826,14 +819,7 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_pipe_kernel(PrefillArgs a
         }
     }
     const int qt = a.n_qtiles - 1 - bid / nbh;
-    const int pos = bid % nbh;
-    int bh = pos;
-    const int ngroups = a.B * a.Hkv;
-    if ((ngroups & 7) == 0) {
-        const int xcd = pos & 7, slot = pos >> 3;
-        const int grp = xcd + 8 * (slot / a.n_rep);
-        bh = grp * a.n_rep + slot % a.n_rep;
-    }
+    const int bh = xcd_grouped_head(bid % nbh, a.B * a.Hkv, a.n_rep);
     const int b = bh / a.Hq, hq = bh % a.Hq, kvh = hq / a.n_rep;
     int L = a.L;
     // cache mode: per-row context length (clamped to the bound a.L) and per-row chunk length n <= T: query t < n sits
@@ -1246,7 +1232,7 @@ __global__ void __launch_bounds__(256) prefill_f32_kernel(PrefillArgs a) {
 
     const int bid = blockIdx.x;
     const int qt = a.n_qtiles - 1 - bid / (a.B * a.Hq);
-    const int bh = bid % (a.B * a.Hq);
+    const int bh = xcd_grouped_head(bid % (a.B * a.Hq), a.B * a.Hkv, a.n_rep);
     const int b = bh / a.Hq, hq = bh % a.Hq, kvh = hq / a.n_rep;
     const int n_chunk = a.chunk_lens ? min(max(a.chunk_lens[b], 0), a.T) : a.T;  // cache mode, as in the bf16 kernel
     const int L = a.seq_lens ? min(max(a.seq_lens[b], n_chunk), a.L) : a.L;
@@ -1420,26 +1406,34 @@ SplitChoice plan_context_split(const vsp_kv_cache* cache, int64_t Hq, int64_t T,
     c.n_splits = (int)ceil_div(tiles, c.split_tiles);
     return c;
 }
+
+// The host-side bound of the context lengths a cached-prefill call is planned on: max_len when given, else the
+// cache's own length, or its capacity when the lengths live on the device.
+int64_t cached_len_bound(const vsp_kv_cache* cache, bool with_seq_lens, int32_t max_len) {
+    if (max_len > 0) return std::min<int64_t>(max_len, cache->S_max);
+    return with_seq_lens ? cache->S_max : cache->len;
+}
 }  // namespace
 
-extern "C" size_t vsp_attn_prefill_cached_split_workspace_bytes(const vsp_kv_cache* cache, int with_seq_lens, int32_t Hq, int32_t T) {
-    if (!cache || Hq <= 0 || T <= 0) return 0;
-    const int64_t L = with_seq_lens ? cache->S_max : cache->len;
+extern "C" size_t vsp_attn_prefill_cached_split_workspace_bytes(const vsp_kv_cache* cache, int with_seq_lens, int32_t max_len,
+                                                                int32_t Hq, int32_t T) {
+    if (!cache || Hq <= 0 || T <= 0 || max_len < 0) return 0;
+    const int64_t L = cached_len_bound(cache, with_seq_lens != 0, max_len);
     const SplitChoice c = plan_context_split(cache, Hq, T, L);
     if (c.n_splits <= 1) return 0;
     return (size_t)cache->B * (size_t)Hq * (size_t)T * (size_t)c.n_splits * (size_t)(cache->D + 2) * sizeof(float);
 }
 
-extern "C" size_t vsp_attn_prefill_cached_workspace_bytes(const vsp_kv_cache* cache, int with_seq_lens) {
-    if (!cache || cache->format != VSP_KV_Q8_0) return 0;
-    const int64_t rows = with_seq_lens ? cache->S_max : cache->len;
+extern "C" size_t vsp_attn_prefill_cached_workspace_bytes(const vsp_kv_cache* cache, int with_seq_lens, int32_t max_len) {
+    if (!cache || cache->format != VSP_KV_Q8_0 || max_len < 0) return 0;
+    const int64_t rows = cached_len_bound(cache, with_seq_lens != 0, max_len);
     return (size_t)2 * (size_t)cache->B * (size_t)cache->Hkv * (size_t)rows * (size_t)cache->D * 2;  // K and V, bf16
 }
 
 extern "C" int vsp_kv_read(const vsp_kv_cache* cache, int64_t start, int64_t count, vsp_tensor* k_out, vsp_tensor* v_out,
                            void* stream);
 
-extern "C" int vsp_attn_prefill_cached(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens,
+extern "C" int vsp_attn_prefill_cached(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* seq_lens, int32_t max_len,
                                        const int32_t* chunk_lens, vsp_tensor* out, vsp_tensor* lse, float scale,
                                        int is_causal, void* workspace, size_t workspace_bytes, void* stream) {
     if (!q || !out) return VSP_ERR_NULL;
@@ -1450,7 +1444,11 @@ extern "C" int vsp_attn_prefill_cached(const vsp_tensor* q, const vsp_kv_cache* 
     const int64_t Hkv = cache->Hkv;
     if (B != cache->B || D != cache->D) return VSP_ERR_SHAPE;
     if (Hkv <= 0 ? Hq != 0 : (Hq % Hkv != 0)) return VSP_ERR_SHAPE;
-    const int64_t L = seq_lens ? cache->S_max : cache->len;  // with seq_lens: the bound the device values are clamped to
+    // the bound every plan below is made on; device-side lengths are clamped to it inside the kernels, a host-side
+    // length above it is a caller error (as in vsp_attn_decode)
+    if (max_len < 0 || max_len > cache->S_max) return VSP_ERR_ARG;
+    if (!seq_lens && max_len > 0 && cache->len > max_len) return VSP_ERR_ARG;
+    const int64_t L = cached_len_bound(cache, seq_lens != nullptr, max_len);
     if (T > L) return VSP_ERR_SHAPE;                          // the chunk is part of the context
     for (int i = 0; i < 4; ++i)
         if (out->shape[i] != q->shape[i]) return VSP_ERR_SHAPE;
@@ -1484,7 +1482,7 @@ extern "C" int vsp_attn_prefill_cached(const vsp_tensor* q, const vsp_kv_cache* 
         // Compute-bound path: dequantising inside the MFMA loop would add vector-ALU work to a kernel that is
         // already short of it, while reading the context out once costs ~0.2 % of the attention time.  The rows
         // [0, L) are dequantised to dense bf16 in the workspace and the dense kernel runs over that.
-        const size_t need = vsp_attn_prefill_cached_workspace_bytes(cache, seq_lens != nullptr);
+        const size_t need = vsp_attn_prefill_cached_workspace_bytes(cache, seq_lens != nullptr, max_len);
         if (!workspace || workspace_bytes < need) return VSP_ERR_WORKSPACE;
         if (!is_aligned16(workspace)) return VSP_ERR_ALIGN;
         vsp_tensor kt{}, vt{};
@@ -1526,8 +1524,8 @@ extern "C" int vsp_attn_prefill_cached(const vsp_tensor* q, const vsp_kv_cache* 
     a.negate_q = (q->dtype == VSP_BF16 && scale < 0.0f) ? 1 : 0;
     a.scale_log2 = (q->dtype == VSP_BF16 ? fabsf(scale) : scale) * kLog2e;
     // a caller that brings the workspace of vsp_attn_prefill_cached_split_workspace_bytes gets the context split over
-    // workgroups when the grid would otherwise leave the chip idle (no lse in that mode: the partials do not carry it)
-    if (!lse && workspace && is_aligned16(workspace)) {
+    // workgroups when the grid would otherwise leave the chip idle; the combine kernel finishes the rows (and their lse)
+    if (workspace && is_aligned16(workspace)) {
         const SplitChoice c = plan_context_split(cache, Hq, T, L);
         const size_t rows = (size_t)B * (size_t)Hq * (size_t)T * (size_t)c.n_splits;
         if (c.n_splits > 1 && workspace_bytes >= rows * (size_t)(D + 2) * sizeof(float)) {
@@ -1539,8 +1537,13 @@ extern "C" int vsp_attn_prefill_cached(const vsp_tensor* q, const vsp_kv_cache* 
             if (blocks > INT32_MAX) return VSP_ERR_ARG;
             hipLaunchKernelGGL(prefill_bf16_pipe_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, a);
             if ((rc = check_launch()) != VSP_OK) return rc;
+            CombineExtra x;
+            x.chunk_lens = chunk_lens;
+            x.len_floor = (int)T;
+            x.lse = a.lse;
+            for (int i = 0; i < 3; ++i) x.sl[i] = a.sl[i];
             return launch_split_combine(a.ws_o, a.ws_ml, seq_lens, cache->len, c.split_tiles * kUnit, c.n_splits, B, Hq, T, D, (int)L, out,
-                                        (hipStream_t)stream);
+                                        (hipStream_t)stream, x);
         }
     }
     return launch_prefill(a, q->dtype, D, cache->format == VSP_KV_BF16, stream);

@@ -47,13 +47,32 @@ __device__ inline uint32_t pack_bf16x2(float a, float b) {
     return (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(b) << 16);
 }
 
+// Workgroup ids are dealt round-robin to the 8 XCDs (id % 8), each with an L2 of its own.  Position `pos` of a row of
+// B * Hq workgroups is mapped to (batch, query head) = bh so that, when the number of (batch, kv head) groups is a
+// multiple of 8, the n_rep query heads of one kv group all get positions of the same residue mod 8: the group's K/V
+// tiles are then fetched into one XCD's L2 instead of up to n_rep of them.  Groups are numbered b * Hkv + kvh, so
+// grp * n_rep + r == b * Hq + hq.  The map is a permutation of [0, B * Hq).
+__device__ inline int xcd_grouped_head(int pos, int n_groups, int n_rep) {
+    if ((n_groups & 7) != 0) return pos;
+    const int xcd = pos & 7, slot = pos >> 3;
+    return (xcd + 8 * (slot / n_rep)) * n_rep + slot % n_rep;
+}
+
 // per-thread last HIP error text (vsp_last_hip_error)
 void set_hip_error(hipError_t e);
 int check_launch();  // VSP_OK or VSP_ERR_LAUNCH after a kernel launch
 int device_cu_count();  // compute units of the device that was current at the first call (256 if the query fails)
-// decode.hip: the split-K combine (decode step; context-split prefill over a cache)
+// decode.hip: the split-K combine (decode step; context-split prefill over a cache).  What the latter adds to the
+// decode step's merge: the lower clamp of a row's length (a chunk is part of its context) and the LSE.
+struct CombineExtra {
+    const int32_t* chunk_lens = nullptr;  // per-row number of valid query rows (device), clamped to [0, len_floor]
+    int32_t len_floor = 0;                // a row's length is at least this (its chunk length when chunk_lens is null)
+    float* lse = nullptr;                 // lse[b][hq][t] = ln sum_j exp(score_j), or null
+    int64_t sl[3] = {0, 0, 0};            // its strides (elements)
+};
 int launch_split_combine(const float* ws_o, const float* ws_ml, const int32_t* seq_lens, int32_t len, int32_t chunk, int32_t max_splits,
-                         int64_t B, int64_t Hq, int64_t T, int64_t D, int32_t L_cap, vsp_tensor* out, hipStream_t st);
+                         int64_t B, int64_t Hq, int64_t T, int64_t D, int32_t L_cap, vsp_tensor* out, hipStream_t st,
+                         const CombineExtra& extra = CombineExtra{});
 
 inline bool is_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
