@@ -209,9 +209,9 @@ def test_bf16_context_split_over_workgroups(va, B, Hq, Hkv, T, L, causal):
     o2, lse = c.prefill(tq, is_causal=causal, return_lse=True)
     assert torch.equal(o2, got)
     _, lse64 = _chunk_rows64(q, k, v, L, causal, with_lse=True)
-    assert np.abs(lse.cpu().numpy() - lse64).max() <= 2e-3     # bf16 P in the row sum: 2^-9 relative on l
+    assert np.abs(lse.cpu().numpy() - lse64).max() <= 5e-3     # the row sum is taken from the bf16 P: up to 2^-8 relative on l
     o3, lse3 = c.prefill(tq, is_causal=causal, return_lse=True, split=False)
-    assert torch.equal(o3, whole) and (lse - lse3).abs().max().item() <= 2e-3
+    assert torch.equal(o3, whole) and (lse - lse3).abs().max().item() <= 5e-3
 
 
 def test_bf16_context_split_ragged_rows_and_stale_tokens(va):
@@ -257,12 +257,12 @@ def test_bf16_context_split_rows_shorter_than_their_chunk_and_a_host_bound(va):
         got, lse = c.prefill(tq, seq_lens=sl, max_len=max_len, return_lse=True)
         whole, lse_w = c.prefill(tq, seq_lens=sl, max_len=max_len, return_lse=True, split=False)
         assert (got.float() - whole.float()).abs().max().item() <= 1.6e-2, max_len
-        assert (lse - lse_w).abs().max().item() <= 2e-3, max_len
+        assert (lse - lse_w).abs().max().item() <= 5e-3, max_len
         for b in range(B):
             L = max(int(lens[b]), T)
             want, lse64 = _chunk_rows64(q[b:b + 1], k[b:b + 1], v[b:b + 1], L, True, with_lse=True)
             G.assert_bf16_close(G.bf16_to_np(got[b:b + 1]), want.astype(np.float32), f"row {b} max_len {max_len}")
-            assert np.abs(lse[b:b + 1].cpu().numpy() - lse64).max() <= 2e-3
+            assert np.abs(lse[b:b + 1].cpu().numpy() - lse64).max() <= 5e-3
     # a device length above the host bound is clamped to it, by both kernels alike
     got = c.prefill(tq, seq_lens=sl, max_len=2048)
     want = _chunk_rows64(q[:1], k[:1], v[:1], 2048, True).astype(np.float32)
