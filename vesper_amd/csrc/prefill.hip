@@ -28,7 +28,6 @@
 // softmax, without a rescale per tile.  Key tiles entirely above the causal diagonal are skipped;
 // the mask is evaluated only on tiles that straddle it.
 #include <math.h>
-#include <stdlib.h>
 
 #include <algorithm>
 #include <utility>
@@ -1219,8 +1218,6 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_pipe_kernel(PrefillArgs a
 #endif
 }
 
-#include "prefill_wide.hpp"
-
 // ---------------------------------------------------------------------------------------------
 // fp32 kernel (fp32 inputs, fp32 MFMA 32x32x2, fp32 softmax): the precision the reference computes
 // in.  One wavefront owns 32 queries, a workgroup 128; key tiles of 32 through LDS.
@@ -1354,14 +1351,6 @@ int launch_prefill(const PrefillArgs& a, int dtype, int64_t D, bool cache_planes
     if (blocks > INT32_MAX) return VSP_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
     dim3 grid((unsigned)blocks), block(256);
-    if (dtype == VSP_BF16 && D == 128 && getenv("VSP_PREFILL_WIDE") && !(!cache_planes && (a.seq_lens || a.chunk_lens))) {
-        PrefillArgs w = a;
-        w.n_qtiles = (int)ceil_div(a.T, kBMW);
-        const dim3 wgrid((unsigned)((int64_t)w.n_qtiles * a.B * a.Hq));
-        if (cache_planes) hipLaunchKernelGGL(prefill_bf16_wide_kernel<true>, wgrid, block, 0, st, w);
-        else hipLaunchKernelGGL(prefill_bf16_wide_kernel<false>, wgrid, block, 0, st, w);
-        return check_launch();
-    }
     if (dtype == VSP_BF16) {
         // head_dim 128 has two kernels.  The software-pipelined one (two workgroups per CU) has the faster steady state;
         // the general one (three per CU, no pipeline to fill and drain) has the cheaper workgroup and wins while contexts
