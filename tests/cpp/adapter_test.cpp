@@ -461,6 +461,29 @@ static void test_multi_head_attention_core() {
         };
         step(0, 16);
         for (int64_t t = 16; t < T; ++t) step(t, t + 1);
+        // forward(x, nullptr, start_pos) with RoPE and no cache (:187-191): rotated as positions start_pos.., attention
+        // over exactly these T tokens; and what the call takes from the allocator does not grow with the position
+        {
+            const int64_t T2 = 16;
+            auto check_at = [&](int64_t pos) {
+                std::vector<float> a2((size_t)(T2 * D / 2)), q2(B * H * T2 * D), k2(q2.size()), w2(q2.size());
+                auto qs = slice(q, 0, T2), ks = slice(k, 0, T2), vs = slice(v, 0, T2);
+                orc_rope_angles((int)T2, (int)D, (int)pos, 10000.0f, a2.data());
+                orc_rope_apply_f32(qs.data(), B, H, T2, D, a2.data(), q2.data());
+                orc_rope_apply_f32(ks.data(), B, H, T2, D, a2.data(), k2.data());
+                orc_sdpa_f32(q2.data(), k2.data(), vs.data(), w2.data(), B, H, T2, T2, D, 1);
+                const size_t before = BlockCache::instance().bytes_taken();
+                Tensor out = mha.forward(to_dev(qs, {B, H, T2, D}, DType::Float32), to_dev(ks, {B, H, T2, D}, DType::Float32),
+                                         to_dev(vs, {B, H, T2, D}, DType::Float32), (nn::KVCache*)nullptr, (int)pos);
+                const size_t taken = BlockCache::instance().bytes_taken() - before;
+                CHECK(max_abs_diff(to_host(out), w2.data(), w2.size()) < 1e-4);
+                return taken;
+            };
+            check_at(3000);  // (builds the RoPE table that covers every position used below)
+            const size_t at0 = check_at(0), at3000 = check_at(3000), at7 = check_at(7);
+            if (!(at0 == at3000 && at0 == at7)) std::printf("  bytes taken at 0 / 7 / 3000: %zu %zu %zu\n", at0, at7, at3000);
+            CHECK(at0 == at3000 && at0 == at7);
+        }
         // training-mode attention dropout is not implemented on this path
         nn::MultiHeadAttentionCore drop((int)(H * D), (int)H, 0.1f, false);
         drop.train();
@@ -571,6 +594,35 @@ static void test_token_loop_allocates_nothing_and_keeps_pace() {
     (void)hipEventDestroy(e1);
 }
 
+static void test_gqa_configurations_of_the_reference() {
+    // tests/test_gqa_chapter33.cpp:600-627: embed_dim 256 with 8, 16 and 32 query heads (head_dim 32, 16, 8) at every
+    // head ratio the reference lists, T = 8; the attention core against the oracle's matmul / softmax route
+    std::printf("test_gqa_configurations_of_the_reference\n");
+    const int64_t configs[6][2] = {{8, 8}, {8, 4}, {8, 2}, {8, 1}, {16, 4}, {32, 8}};
+    const int64_t C = 256, B = 1, T = 8;
+    for (auto& cfg : configs) {
+        const int64_t Hq = cfg[0], Hkv = cfg[1], D = C / Hq;
+        nn::GroupedQueryAttentionCore attn(C, Hq, Hkv, 64);
+        CHECK(attn.head_dim() == D && attn.num_rep() == Hq / Hkv);
+        auto q = randn(B * Hq * T * D, 500 + (int)Hq, 1.0f), k = randn(B * Hkv * T * D, 501 + (int)Hkv, 1.0f), v = randn(B * Hkv * T * D, 502, 1.0f);
+        std::vector<float> want(q.size());
+        int64_t st[4] = {Hkv * T * D, T * D, D, 1};
+        CHECK(orc_gqa_attention_f32(q.data(), k.data(), st, v.data(), st, want.data(), B, Hq, T, T, D, Hq / Hkv, 1) == 0);
+        Tensor out = attn.forward(to_dev(q, {B, Hq, T, D}, DType::Float32), to_dev(k, {B, Hkv, T, D}, DType::Float32),
+                                  to_dev(v, {B, Hkv, T, D}, DType::Float32));
+        CHECK((out.shape() == std::vector<int64_t>{B, Hq, T, D}));
+        auto got = to_host(out);
+        const double err = max_abs_diff(got, want.data(), want.size());
+        if (!(err < 1e-4)) std::printf("  %lldQ/%lldKV head_dim %lld: max-abs %.3g\n", (long long)Hq, (long long)Hkv, (long long)D, err);
+        CHECK(err < 1e-4);
+        // and through a cache: prompt of 8, then one token
+        nn::KVCache cache((int)B, (int)Hkv, 64, (int)D, Device::HIP);
+        Tensor o2 = attn.forward(to_dev(q, {B, Hq, T, D}, DType::Float32), to_dev(k, {B, Hkv, T, D}, DType::Float32),
+                                 to_dev(v, {B, Hkv, T, D}, DType::Float32), &cache, 0);
+        CHECK(max_abs_diff(to_host(o2), want.data(), want.size()) < 1e-4);
+    }
+}
+
 int main(int argc, char** argv) {
     const bool cpu_only = argc > 1 && std::string(argv[1]) == "--cpu-only";
     test_gqa_constructor_validation();
@@ -585,6 +637,7 @@ int main(int argc, char** argv) {
         test_sdpa_routing();
         test_backward_dispatch_seam();
         test_multi_head_attention_core();
+        test_gqa_configurations_of_the_reference();
         test_chunk_of_a_long_prompt_splits_the_context();
         run_token_with_output_projection(KVFormat::Float32, DType::Float32, 1e-4, "f32");
         run_token_with_output_projection(KVFormat::BFloat16, DType::BFloat16, 1e-2, "bf16");

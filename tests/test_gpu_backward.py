@@ -68,6 +68,27 @@ def test_f32_gqa_against_oracle_through_repeat_kv(va, B, Hq, Hkv, N, D, causal):
     G.assert_f32_close(dk.cpu().numpy(), ck.reshape(B, Hkv, n, N, D).sum(2).astype(np.float32), "dk closed form")
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,N,D,causal", [(1, 16, 4, 8, 16, True), (1, 32, 8, 8, 8, True), (2, 4, 2, 70, 24, True),
+                                                 (1, 3, 1, 45, 5, False), (1, 2, 2, 33, 100, True)])
+def test_f32_any_head_dim(va, B, Hq, Hkv, N, D, causal):
+    # the reference's backward takes any head_dim (src/ops/flash_attention.cpp:366-482); 16 and 8 are what its own GQA
+    # configurations have at embed_dim 256 (tests/test_gqa_chapter33.cpp:600-627)
+    q, k, v = I.qkv(800 + D, B, Hq, Hkv, N, N, D)
+    dout = I.normal(805 + D, (B, Hq, N, D))
+    scale = float(np.float32(1.0 / np.sqrt(D)))
+    n = Hq // Hkv
+    kr, vr = O.repeat_kv(k, n), O.repeat_kv(v, n)
+    out, lse = O.flash_attention(q, kr, vr, scale, causal, return_lse=True)
+    wq, wk, wv = O.flash_attention_backward(dout, q, kr, vr, out, lse, scale, causal)
+    dq, dk, dv = _forward_then_backward(va, q, k, v, dout, scale, causal)
+    G.assert_f32_close(dq.cpu().numpy(), wq, "dq")
+    G.assert_f32_close(dk.cpu().numpy(), wk.reshape(B, Hkv, n, N, D).sum(2), "dk")
+    G.assert_f32_close(dv.cpu().numpy(), wv.reshape(B, Hkv, n, N, D).sum(2), "dv")
+    cq, ck, cv = closed_form_grads(dout, q, kr, vr, scale, causal)
+    G.assert_f32_close(dq.cpu().numpy(), cq.astype(np.float32), "dq closed form")
+    G.assert_f32_close(dv.cpu().numpy(), cv.reshape(B, Hkv, n, N, D).sum(2).astype(np.float32), "dv closed form")
+
+
 def test_single_token(va):
     # N = 1: P = 1, so dS = dP - Di = 0 and dq = dk = 0 exactly in exact arithmetic, dv = dout
     q, k, v = I.qkv(750, 1, 2, 2, 1, 1, 64)
@@ -182,11 +203,11 @@ def test_argument_errors(va):
     q = torch.zeros(1, 4, 8, 64, device=d)
     k = torch.zeros(1, 2, 8, 64, device=d)
     lse = torch.zeros(1, 4, 8, device=d)
-    with pytest.raises(va.VspError):   # head dim 32 exists in fp32 only; head dim 48 not at all
+    with pytest.raises(va.VspError):   # bf16: head dim 64 or 128 only
         z = torch.zeros(1, 2, 8, 32, device=d, dtype=torch.bfloat16)
         va.flash_attention_backward(z, z, z, z, z, torch.zeros(1, 2, 8, device=d), 0.1)
-    with pytest.raises(va.VspError):
-        z = torch.zeros(1, 2, 8, 48, device=d)
+    with pytest.raises(va.VspError):   # fp32: any head dim up to 128
+        z = torch.zeros(1, 2, 8, 160, device=d)
         va.flash_attention_backward(z, z, z, z, z, torch.zeros(1, 2, 8, device=d), 0.1)
     with pytest.raises(va.VspError):   # 3 query heads over 2 kv heads
         q3 = torch.zeros(1, 3, 8, 64, device=d)

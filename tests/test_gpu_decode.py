@@ -65,6 +65,36 @@ def test_q8_0_decode_against_oracle_over_dequantised_cache(va, B, Hq, Hkv, S, D,
     G.assert_bf16_close(G.bf16_to_np(out), oracle_decode(q, kd, vd, lens), f"q8_0 lens={lens}")
 
 
+@pytest.mark.parametrize("fmt", ["bf16", "q8_0"])
+@pytest.mark.parametrize("B,Hq,Hkv,S,D,lens", [
+    (2, 32, 1, 700, 128, [700, 129]),        # multi-query attention: 32 query heads on one kv head (two groups of 16)
+    (1, 128, 2, 1300, 128, [1211]),          # 64 per kv head (four groups)
+    (3, 40, 2, 300, 64, [300, 0, 65]),       # 20 per kv head: a full group and one of four heads
+    (9, 17, 1, 130, 128, [130, 1, 64, 65, 2, 130, 99, 17, 33])])   # nine (item, kv head) pairs: the grid is padded to 16
+def test_more_than_16_query_heads_per_kv_head(va, fmt, B, Hq, Hkv, S, D, lens):
+    # ops::repeat_kv takes any n_rep (src/ops/attention_ops.cpp:92-155): beyond the 16 columns of the matrix
+    # instructions the heads of a kv head are served in groups of 16, one workgroup per group
+    q, k, v = I.qkv(48, B, Hq, Hkv, 1, S, D)
+    q = O.bf16_round(q)
+    if fmt == "bf16":
+        k, v = O.bf16_round(k), O.bf16_round(v)
+        kd, vd = k, v
+    else:
+        kd, vd = O.q8_0_dequantize(*O.q8_0_quantize(k)), O.q8_0_dequantize(*O.q8_0_quantize(v))
+    c = fill_cache(va, fmt, k, v)
+    sl = torch.tensor(lens, dtype=torch.int32, device=G.dev())
+    out = va.decode_attention(G.to_bf16_dev(q), c, seq_lens=sl)
+    G.assert_bf16_close(G.bf16_to_np(out), oracle_decode(q, kd, vd, lens), f"{fmt} lens={lens}")
+    assert torch.equal(out, va.decode_attention(G.to_bf16_dev(q), c, seq_lens=sl))   # fixed merge order
+    # the same heads 16 at a time through the one-group path give the same bits: a group is a pure partition of the work
+    n = Hq // Hkv
+    if n % 16 == 0:
+        qd = G.to_bf16_dev(q).view(B, Hkv, n // 16, 16, 1, D)
+        for gi in range(n // 16):
+            part = va.decode_attention(qd[:, :, gi].reshape(B, Hkv * 16, 1, D).contiguous(), c, seq_lens=sl)
+            assert torch.equal(part.view(B, Hkv, 16, 1, D), out.view(B, Hkv, n // 16, 16, 1, D)[:, :, gi])
+
+
 # D 64 / 128 with up to 16 query heads per kv head run on the fp32 matrix instructions, everything else (D 32: the
 # reference's own test shapes; 32 query heads on one kv head) on the plain-FMA kernel
 @pytest.mark.parametrize("B,Hq,Hkv,S,D,lens", [

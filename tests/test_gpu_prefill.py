@@ -73,6 +73,39 @@ def test_f32_against_oracle_and_closed_form(va, B, Hq, Hkv, T, L, D, causal):
         G.assert_f32_close(out, want, "oracle")
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,T,L,D,causal", [
+    (1, 16, 4, 8, 8, 16, True), (1, 32, 8, 8, 8, 8, True),          # embed_dim 256 with 16 and 32 heads: the reference's
+    (1, 8, 1, 8, 8, 32, True),                                      # own GQA configurations, tests/test_gqa_chapter33.cpp:600-627
+    (2, 4, 2, 70, 70, 24, True), (1, 3, 1, 40, 90, 5, False), (1, 2, 2, 33, 33, 100, True), (1, 4, 2, 65, 65, 1, True),
+    (1, 2, 1, 50, 50, 129, True), (1, 2, 2, 37, 80, 200, False), (1, 1, 1, 20, 20, 256, True)])
+def test_f32_any_head_dim(va, B, Hq, Hkv, T, L, D, causal):
+    # the reference's forward takes any head_dim (src/ops/flash_attention.cpp:235-238); here the fp32 kernel pads the
+    # tile to the next of 32 / 64 / 128 / 256 inside the kernel, rows of any length are read element by element
+    q, k, v = I.qkv(1200 + D, B, Hq, Hkv, T, L, D)
+    scale = 1.0 / math.sqrt(D)
+    out, lse = va.flash_attention(G.f32_dev(q), G.f32_dev(k), G.f32_dev(v), scale, causal, return_lse=True)
+    out = out.cpu().numpy()
+    G.assert_f32_close(out, closed_form64(q, k, v, scale, causal).astype(np.float32), "closed form")
+    if T == L:
+        want, want_lse = oracle_gqa_flash(q, k, v, float(np.float32(scale)), causal)
+        G.assert_f32_close(out, want, "oracle")
+        assert np.abs(lse.cpu().numpy() - want_lse).max() < 1e-4
+    # a strided view (rows of a wider buffer): nothing about the row pitch is assumed
+    wide = torch.zeros(B, Hkv, L, D + 3, device=G.dev())
+    wide[..., :D] = G.f32_dev(k)
+    out2 = va.flash_attention(G.f32_dev(q), wide[..., :D], G.f32_dev(v), scale, causal).cpu().numpy()
+    assert np.array_equal(out, out2)
+
+
+def test_head_dims_that_stay_unsupported(va):
+    z = lambda *s: torch.zeros(*s, device=G.dev())
+    with pytest.raises(va.VspError):      # fp32 beyond 256
+        va.flash_attention(z(1, 1, 4, 257), z(1, 1, 4, 257), z(1, 1, 4, 257), 0.1, True)
+    b = lambda *s: torch.zeros(*s, device=G.dev(), dtype=torch.bfloat16)
+    with pytest.raises(va.VspError):      # bf16 keeps its two tile widths
+        va.flash_attention(b(1, 1, 4, 32), b(1, 1, 4, 32), b(1, 1, 4, 32), 0.1, True)
+
+
 def test_f32_known_answers_of_the_reference_tests(va):
     # causal structure, tests/test_attention_chapter32.cpp:168-203 (padded to D=64: extra dims are zero)
     q = np.ones((1, 1, 4, 64), np.float32)

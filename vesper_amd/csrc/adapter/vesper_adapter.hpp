@@ -75,6 +75,7 @@ public:
         const size_t want = round_size(bytes);
         {
             std::lock_guard<std::mutex> lock(mu_);
+            bytes_taken_ += want;
             auto range = free_.equal_range(Key{stream, want});
             if (range.first != range.second) {
                 void* p = range.first->second;
@@ -83,7 +84,13 @@ public:
             }
         }
         void* p = nullptr;
-        hip_check(hipMalloc(&p, want), "hipMalloc");
+        if (hipMalloc(&p, want) != hipSuccess) {
+            // out of memory: give the cached free blocks back to the driver and try once more, as the reference's
+            // CachingAllocator::allocate does (src/core/allocator.cpp:190-198)
+            (void)hipGetLastError();
+            empty_cache();
+            hip_check(hipMalloc(&p, want), "hipMalloc");
+        }
         std::lock_guard<std::mutex> lock(mu_);
         size_[p] = want;
         return p;
@@ -106,6 +113,11 @@ public:
         std::lock_guard<std::mutex> lock(mu_);
         return size_.size();
     }
+    // bytes handed out so far, recycled blocks included: what the calls in between asked for
+    size_t bytes_taken() const {
+        std::lock_guard<std::mutex> lock(mu_);
+        return bytes_taken_;
+    }
 
 private:
     using Key = std::pair<hipStream_t, size_t>;
@@ -118,6 +130,7 @@ private:
     mutable std::mutex mu_;
     std::multimap<Key, void*> free_;
     std::unordered_map<void*, size_t> size_;
+    size_t bytes_taken_ = 0;
 };
 
 class Storage {
@@ -213,8 +226,16 @@ public:
     // set by ops::repeat_kv: logically [B, H*head_rep, S, D], physically the un-repeated tensor
     int64_t head_rep = 1;
     // set by KVCache::update: this tensor is the K (is_v == false) or V side of that cache's context
+    // (the cache's state is shared, not copied: cache_len is the context length as of that update, and cache_desc()
+    // the descriptor a kernel should see for this handle)
     std::shared_ptr<KVCacheState> cache;
+    int32_t cache_len = 0;
     bool is_v = false;
+    vsp_kv_cache cache_desc() const {
+        vsp_kv_cache c = cache->c;
+        c.len = cache_len;
+        return c;
+    }
 
 private:
     void host_copy(void* host, bool to_device) {
@@ -287,6 +308,15 @@ class KVCacheT {
 public:
     KVCacheT(LenT batch_size, LenT num_heads, LenT max_seq_len, LenT head_dim, Device device = Device::HIP,
              KVFormat format = KVFormat::Float32)
+        : KVCacheT(batch_size, num_heads, max_seq_len, head_dim, device, format, /*zero=*/true) {}
+    // A cache whose planes are left as allocated (no zero fill: one pass over memory saved): for a caller that writes
+    // every row before reading it, such as the scratch of a single forward call.
+    static KVCacheT uninitialized(LenT batch_size, LenT num_heads, LenT max_seq_len, LenT head_dim, KVFormat format) {
+        return KVCacheT(batch_size, num_heads, max_seq_len, head_dim, Device::HIP, format, /*zero=*/false);
+    }
+
+private:
+    KVCacheT(LenT batch_size, LenT num_heads, LenT max_seq_len, LenT head_dim, Device device, KVFormat format, bool zero)
         : st_(std::make_shared<KVCacheState>()) {
         if (device != Device::HIP) throw std::runtime_error("KVCache: only Device::HIP is implemented here");
         auto& c = st_->c;
@@ -304,8 +334,10 @@ public:
         c.k_scale = st_->planes[2] ? st_->planes[2]->data() : nullptr;
         c.v_scale = st_->planes[3] ? st_->planes[3]->data() : nullptr;
         c.len = 0;
-        throw_status(vsp_kv_cache_reset(&c, current_stream()));  // vesper::zeros in the reference constructor
+        if (zero) throw_status(vsp_kv_cache_reset(&c, current_stream()));  // vesper::zeros in the reference constructor
     }
+
+public:
 
     // Writes [:, :, start_pos:start_pos+T, :], then returns the active context [:, :, 0:len, :].
     // Float32 storage: the pair are true strided views of the cache planes, as in the reference.
@@ -321,10 +353,16 @@ public:
     // (`q_dtype`: what the attention kernels should receive).
     std::pair<Tensor, Tensor> rope_update(Tensor& q, const Tensor& new_k, const Tensor& new_v, LenT start_pos,
                                           const RopeTable& rope, DType q_dtype) {
+        return rope_update(q, new_k, new_v, start_pos, rope.data(), rope.length(), q_dtype);
+    }
+    // The same with the table given as rows: row r of `table` rotates the token written at position r, so a table pointer
+    // advanced by p rows places tokens at 0.. while rotating them as positions p.. (a scratch cache of T tokens for a
+    // call at start_pos > 0).
+    std::pair<Tensor, Tensor> rope_update(Tensor& q, const Tensor& new_k, const Tensor& new_v, LenT start_pos, const float* table,
+                                          int64_t table_rows, DType q_dtype) {
         Tensor q_out = empty(q.shape(), q_dtype);
         vsp_tensor dq = q.desc(), dk = new_k.desc(), dv = new_v.desc(), dout = q_out.desc();
-        throw_status(vsp_rope_kv_append(&st_->c, &dq, &dk, &dv, &dout, rope.data(), rope.length(), (int64_t)start_pos,
-                                        nullptr, current_stream()));
+        throw_status(vsp_rope_kv_append(&st_->c, &dq, &dk, &dv, &dout, table, table_rows, (int64_t)start_pos, nullptr, current_stream()));
         q = q_out;
         return {view(false), view(true)};
     }
@@ -378,7 +416,8 @@ private:
             std::vector<int64_t> shape = {c.B, c.Hkv, c.len, c.D};
             t = Tensor::over(nullptr, DType::BFloat16, shape, Tensor::contiguous_strides(shape));
         }
-        t.cache = std::make_shared<KVCacheState>(*st_);  // snapshot of the descriptor (len as of this update)
+        t.cache = st_;          // shared state, no copy: the handle keeps the planes alive
+        t.cache_len = c.len;    // the context length as of this update
         t.is_v = is_v;
         return t;
     }
@@ -391,7 +430,7 @@ using GQAKVCache = KVCacheT<int64_t>;
 // [:, :, 0:len, :] of a cache handle as a real tensor of `dtype` (copy; Q8_0 is dequantised).
 inline Tensor materialize(const Tensor& handle, DType dtype) {
     if (!handle.cache || handle.defined()) return handle;
-    const auto& c = handle.cache->c;
+    const vsp_kv_cache c = handle.cache_desc();
     Tensor out = empty({c.B, c.Hkv, c.len, c.D}, dtype);
     vsp_tensor d = out.desc();
     throw_status(vsp_kv_read(&c, 0, c.len, handle.is_v ? nullptr : &d, handle.is_v ? &d : nullptr, current_stream()));
@@ -523,6 +562,14 @@ namespace functional {
 
 // include/vesper/nn/functional.h:132-136, src/nn/functional.cpp:370-422.  One kernel family serves
 // every sequence length (the reference's switch at 512 is a speed heuristic of its own back ends):
+// The length a per-call decode workspace is sized for: the next power of two at or above the context length, capped
+// at the cache's capacity.
+inline int32_t ws_len_bound(int32_t len, int32_t s_max) {
+    int64_t p = 256;
+    while (p < len) p *= 2;
+    return (int32_t)std::min<int64_t>(p, std::max<int32_t>(s_max, 1));
+}
+
 // T == 1 over a cache handle -> split-K decode; everything else -> the prefill kernel.
 inline Tensor scaled_dot_product_attention(const Tensor& query, const Tensor& key, const Tensor& value, bool is_causal = false,
                                            double dropout_p = 0.0) {
@@ -533,9 +580,11 @@ inline Tensor scaled_dot_product_attention(const Tensor& query, const Tensor& ke
     const float scale = 1.0f / std::sqrt(static_cast<float>(D));
     if (T == 1 && key.cache && value.cache && !key.is_v && value.is_v) {
         Tensor out = empty(query.shape(), query.dtype());
-        const vsp_kv_cache& c = key.cache->c;
+        const vsp_kv_cache c = key.cache_desc();
+        // (sized for the next power of two of the context length: a token loop then keeps taking the same block
+        // instead of walking through a bin per 2 MiB of growth)
         const size_t ws_bytes = vsp_attn_decode_workspace_bytes((int32_t)query.shape()[0], (int32_t)query.shape()[1], (int32_t)D,
-                                                               c.len > 0 ? c.len : 1);
+                                                               ws_len_bound(c.len, c.S_max));
         Storage ws(ws_bytes);  // a recycled block after the first call; released without waiting (see BlockCache)
         vsp_tensor dq = query.desc(), dout = out.desc();
         throw_status(vsp_attn_decode(&dq, &c, nullptr, 0, &dout, scale, ws.data(), ws_bytes, current_stream()));
@@ -554,10 +603,10 @@ inline Tensor decode_attention_proj(const Tensor& query, const Tensor& key, cons
     if (!(key.cache && value.cache && !key.is_v && value.is_v)) throw std::runtime_error("decode_attention_proj: key/value must be cache handles");
     if (wo.ndim() != 2) throw_status(VSP_ERR_NDIM);
     const int64_t B = query.shape()[0], Hq = query.shape()[1], D = query.shape()[3];
-    const vsp_kv_cache& c = key.cache->c;
+    const vsp_kv_cache c = key.cache_desc();
     const float scale = 1.0f / std::sqrt(static_cast<float>(D));
     Tensor y = empty({B, 1, wo.shape()[0]}, query.dtype());
-    const size_t ws_bytes = vsp_attn_decode_proj_workspace_bytes((int32_t)B, (int32_t)Hq, (int32_t)D, c.len > 0 ? c.len : 1, (int32_t)wo.shape()[0]);
+    const size_t ws_bytes = vsp_attn_decode_proj_workspace_bytes((int32_t)B, (int32_t)Hq, (int32_t)D, ws_len_bound(c.len, c.S_max), (int32_t)wo.shape()[0]);
     Storage ws(ws_bytes);
     vsp_tensor dq = query.desc(), dw = wo.desc(), dy = y.desc(), db;
     if (bias) db = bias->desc();
@@ -573,8 +622,13 @@ inline Tensor decode_attention_proj(const Tensor& query, const Tensor& key, cons
 // produced.  The constructor performs the reference constructor's checks and arithmetic.
 class GroupedQueryAttentionCore {
 public:
-    GroupedQueryAttentionCore(int64_t embed_dim, int64_t num_heads, int64_t num_kv_heads)
-        : embed_dim_(embed_dim), num_heads_(num_heads), num_kv_heads_(num_kv_heads) {
+    // the reference's parameter list (include/vesper/nn/gqa_attention.h:40-47); max_seq_len and rope_base size its RoPE
+    // table, which callers of this core bring themselves (RopeTable), dropout is refused at forward time when training,
+    // bias belongs to the projections
+    GroupedQueryAttentionCore(int64_t embed_dim, int64_t num_heads, int64_t num_kv_heads, int64_t max_seq_len = 4096,
+                              float rope_base = 10000.0f, float dropout = 0.0f, bool bias = false)
+        : embed_dim_(embed_dim), num_heads_(num_heads), num_kv_heads_(num_kv_heads), max_seq_len_(max_seq_len),
+          rope_base_(rope_base), dropout_(dropout), bias_(bias) {
         if (num_heads % num_kv_heads != 0)
             throw std::invalid_argument("GroupedQueryAttention: num_heads (" + std::to_string(num_heads) +
                                         ") must be divisible by num_kv_heads (" + std::to_string(num_kv_heads) + ")");
@@ -588,6 +642,10 @@ public:
     int64_t num_kv_heads() const { return num_kv_heads_; }
     int64_t head_dim() const { return head_dim_; }
     int64_t num_rep() const { return num_rep_; }
+    int64_t max_seq_len() const { return max_seq_len_; }
+    float rope_base() const { return rope_base_; }
+    float dropout() const { return dropout_; }
+    bool bias() const { return bias_; }
     float kv_cache_ratio() const { return static_cast<float>(num_kv_heads_) / num_heads_; }
 
     // forward(x, causal) core, src/nn/gqa_attention.cpp:91-96
@@ -643,6 +701,9 @@ public:
 
 private:
     int64_t embed_dim_, num_heads_, num_kv_heads_, head_dim_ = 0, num_rep_ = 0;
+    int64_t max_seq_len_;
+    float rope_base_, dropout_;
+    bool bias_;
 };
 
 // The attention core of MultiHeadAttention (include/vesper/nn/transformer.h:41-56, src/nn/transformer.cpp:96-216):
@@ -668,7 +729,8 @@ public:
         if (q.ndim() != 4) throw_status(VSP_ERR_NDIM);
         const int64_t B = q.shape()[0], H = k.shape()[1], T = q.shape()[2], D = q.shape()[3];
         const RopeTable& rope = rope_for(T, D);
-        KVCache scratch((int)B, (int)H, (int)T, (int)D, Device::HIP, q.dtype() == DType::Float32 ? KVFormat::Float32 : KVFormat::BFloat16);
+        // (every row of the scratch is written by the rotation before it is read: no zero fill)
+        KVCache scratch = KVCache::uninitialized((int)B, (int)H, (int)T, (int)D, q.dtype() == DType::Float32 ? KVFormat::Float32 : KVFormat::BFloat16);
         Tensor qr = q;
         auto kv = scratch.rope_update(qr, k, v, 0, rope, q.dtype());
         if (q.dtype() == DType::Float32) return functional::scaled_dot_product_attention(qr, kv.first, kv.second, causal, 0.0);
@@ -686,15 +748,17 @@ public:
             k = kv.first;
             v = kv.second;
         } else if (use_rope_) {
-            // no cache: rotate at start_pos.. through a cache of this call's own, as above
+            // no cache: rotate as positions start_pos.. through a scratch of this call's own that holds exactly these T
+            // tokens (the table enters advanced by start_pos rows, so the tokens are placed at 0..: what the call
+            // writes does not grow with the position), then SDPA over exactly these T keys (:187-191)
             const int64_t B = q.shape()[0], H = k.shape()[1];
-            KVCache scratch((int)B, (int)H, (int)(start_pos + T), (int)D, Device::HIP,
-                            q.dtype() == DType::Float32 ? KVFormat::Float32 : KVFormat::BFloat16);
-            // only rows [start_pos, start_pos + T) are written and read back: SDPA over exactly these T keys
-            scratch.rope_update(qq, k, v, start_pos, rope_for(start_pos + T, D), q.dtype());
+            KVCache scratch = KVCache::uninitialized((int)B, (int)H, (int)T, (int)D,
+                                                     q.dtype() == DType::Float32 ? KVFormat::Float32 : KVFormat::BFloat16);
+            const RopeTable& rope = rope_for(start_pos + T, D);
+            scratch.rope_update(qq, k, v, 0, rope.data() + (int64_t)start_pos * D, rope.length() - start_pos, q.dtype());
             Tensor kr = empty(k.shape(), q.dtype()), vr = empty(v.shape(), q.dtype());
             vsp_tensor dk = kr.desc(), dv = vr.desc();
-            throw_status(vsp_kv_read(&scratch.raw(), start_pos, T, &dk, &dv, current_stream()));
+            throw_status(vsp_kv_read(&scratch.raw(), 0, T, &dk, &dv, current_stream()));
             k = kr;
             v = vr;
         }

@@ -35,6 +35,7 @@ struct BwdArgs {
     int32_t causal;
     float scale;
     int64_t lo_q, lo_kv;                   // split operands: elements from a hi plane to its lo plane (q-shaped, kv-shaped)
+    int32_t D_true;                        // fp32 kernels: the tensors' head_dim (<= the kernel's tile width; columns past it are zero)
 };
 
 template <typename T>
@@ -99,10 +100,11 @@ __global__ void __launch_bounds__(256) bwd_dq_kernel(BwdArgs a) {
     const T* Kp = (const T*)a.k + (int64_t)b * a.s_k[0] + (int64_t)kvh * a.s_k[1];
     const T* Vp = (const T*)a.v + (int64_t)b * a.s_v[0] + (int64_t)kvh * a.s_v[1];
     float qf[D / 2], dof[D / 2];
+    const int Dt = a.D_true;  // the reference's backward takes any head_dim (src/ops/flash_attention.cpp:366-482)
 #pragma unroll
     for (int ks = 0; ks < D / 2; ++ks) {
-        qf[ks] = ld<T>(Qp + 2 * ks + h);
-        dof[ks] = ld<T>(Op + 2 * ks + h);
+        qf[ks] = 2 * ks + h < Dt ? ld<T>(Qp + 2 * ks + h) : 0.f;
+        dof[ks] = 2 * ks + h < Dt ? ld<T>(Op + 2 * ks + h) : 0.f;
     }
     const float lse_q = a.lse[(int64_t)b * a.s_l[0] + (int64_t)hq * a.s_l[1] + (int64_t)qrow * a.s_l[2]];
     const float di_q = a.delta[((int64_t)b * a.Hq + hq) * a.N + qrow];
@@ -122,8 +124,9 @@ __global__ void __launch_bounds__(256) bwd_dq_kernel(BwdArgs a) {
         __syncthreads();
         for (int id = tid; id < kBT * D; id += 256) {
             const int row = id / D, col = id % D, key = kt * kBT + row;
-            sK[row * PITCH + col] = key < a.N ? ld<T>(Kp + (int64_t)key * a.s_k[2] + col) : 0.f;
-            sV[row * PITCH + col] = key < a.N ? ld<T>(Vp + (int64_t)key * a.s_v[2] + col) : 0.f;
+            const bool ok = key < a.N && col < Dt;
+            sK[row * PITCH + col] = ok ? ld<T>(Kp + (int64_t)key * a.s_k[2] + col) : 0.f;
+            sV[row * PITCH + col] = ok ? ld<T>(Vp + (int64_t)key * a.s_v[2] + col) : 0.f;
         }
         __syncthreads();
         const int k0 = kt * kBT;
@@ -158,7 +161,10 @@ __global__ void __launch_bounds__(256) bwd_dq_kernel(BwdArgs a) {
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) st<T>(op + 32 * db + 8 * (v >> 2) + 4 * h + (v & 3), a.scale * acc[db][v]);
+            for (int v = 0; v < 16; ++v) {
+                const int d = 32 * db + 8 * (v >> 2) + 4 * h + (v & 3);
+                if (d < Dt) st<T>(op + d, a.scale * acc[db][v]);
+            }
     }
 }
 
@@ -191,10 +197,11 @@ __global__ void __launch_bounds__(256) bwd_dkdv_kernel(BwdArgs a) {
     const T* Kp = (const T*)a.k + (int64_t)b * a.s_k[0] + (int64_t)kvh * a.s_k[1] + (int64_t)krow * a.s_k[2];
     const T* Vp = (const T*)a.v + (int64_t)b * a.s_v[0] + (int64_t)kvh * a.s_v[1] + (int64_t)krow * a.s_v[2];
     float kf[D / 2], vf[D / 2];
+    const int Dt = a.D_true;
 #pragma unroll
     for (int ks = 0; ks < D / 2; ++ks) {
-        kf[ks] = ld<T>(Kp + 2 * ks + h);
-        vf[ks] = ld<T>(Vp + 2 * ks + h);
+        kf[ks] = 2 * ks + h < Dt ? ld<T>(Kp + 2 * ks + h) : 0.f;
+        vf[ks] = 2 * ks + h < Dt ? ld<T>(Vp + 2 * ks + h) : 0.f;
     }
     f32x16_t acck[DB], accv[DB];
 #pragma unroll
@@ -218,8 +225,9 @@ __global__ void __launch_bounds__(256) bwd_dkdv_kernel(BwdArgs a) {
             __syncthreads();
             for (int id = tid; id < kBT * D; id += 256) {
                 const int row = id / D, col = id % D, qi = qt * kBT + row;
-                sQ[row * PITCH + col] = qi < a.N ? ld<T>(Qp + (int64_t)qi * a.s_q[2] + col) : 0.f;
-                sO[row * PITCH + col] = qi < a.N ? ld<T>(Op + (int64_t)qi * a.s_do[2] + col) : 0.f;
+                const bool ok = qi < a.N && col < Dt;
+                sQ[row * PITCH + col] = ok ? ld<T>(Qp + (int64_t)qi * a.s_q[2] + col) : 0.f;
+                sO[row * PITCH + col] = ok ? ld<T>(Op + (int64_t)qi * a.s_do[2] + col) : 0.f;
             }
             if (tid < kBT) {
                 const int qi = qt * kBT + tid;
@@ -265,8 +273,10 @@ __global__ void __launch_bounds__(256) bwd_dkdv_kernel(BwdArgs a) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int d = 32 * db + 8 * (v >> 2) + 4 * h + (v & 3);
-                st<T>(pk + d, a.scale * acck[db][v]);
-                st<T>(pv + d, accv[db][v]);
+                if (d < Dt) {
+                    st<T>(pk + d, a.scale * acck[db][v]);
+                    st<T>(pv + d, accv[db][v]);
+                }
             }
     }
 }
@@ -871,10 +881,10 @@ int launch_backward(const BwdArgs& a, int64_t D, hipStream_t st) {
         }
         return check_launch();
     }
-    if (D == 128) {
+    if (D > 64) {  // the fp32 kernels take any head_dim up to their tile width (a.D_true)
         hipLaunchKernelGGL((bwd_dq_kernel<128, T>), gq, dim3(256), 0, st, a);
         hipLaunchKernelGGL((bwd_dkdv_kernel<128, T>), gk, dim3(256), 0, st, a);
-    } else if (D == 64) {
+    } else if (D > 32) {
         hipLaunchKernelGGL((bwd_dq_kernel<64, T>), gq, dim3(256), 0, st, a);
         hipLaunchKernelGGL((bwd_dkdv_kernel<64, T>), gk, dim3(256), 0, st, a);
     } else {
@@ -933,7 +943,8 @@ extern "C" int vsp_attn_prefill_backward(const vsp_tensor* dout, const vsp_tenso
     if (lse->dtype != VSP_F32) return VSP_ERR_DTYPE;
     if (B * Hq * N * D == 0) return VSP_OK;
     if (!lse->data) return VSP_ERR_NULL;
-    if (D != 64 && D != 128 && !(D == 32 && dt == VSP_F32)) return VSP_ERR_UNSUPPORTED;  // fp32 also takes head_dim 32
+    // bf16: head_dim 64 or 128; fp32: any head_dim up to 128, as the reference's backward takes any
+    if (dt == VSP_BF16 ? (D != 64 && D != 128) : D > 128) return VSP_ERR_UNSUPPORTED;
     if (!(fabsf(scale) < INFINITY)) return VSP_ERR_ARG;
     if (N > INT32_MAX / 2) return VSP_ERR_ARG;
     if (!workspace || workspace_bytes < vsp_attn_backward_workspace_bytes((int32_t)B, (int32_t)Hq, (int32_t)N)) return VSP_ERR_WORKSPACE;
@@ -978,6 +989,7 @@ extern "C" int vsp_attn_prefill_backward(const vsp_tensor* dout, const vsp_tenso
     a.N = (int)N;
     a.causal = is_causal ? 1 : 0;
     a.scale = scale;
+    a.D_true = (int)D;
     return dt == VSP_F32 ? launch_backward<float>(a, D, (hipStream_t)stream) : launch_backward<uint16_t>(a, D, (hipStream_t)stream);
 }
 

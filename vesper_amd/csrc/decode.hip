@@ -54,6 +54,9 @@ struct DecodeArgs {
     // page size.  nullptr for a contiguous cache.
     const int32_t* page_table;
     int32_t page_tokens, pages_per_seq;
+    // More than 16 query heads per kv head (one token per sequence): the heads are cut into n_cgroups groups of 16
+    // columns, one workgroup per (item, kv head, group); col0 is the group's first head (set by each workgroup).
+    int32_t n_cgroups, col0;
 };
 
 // Index of the [S][D] slab that holds the 64-key group at token `kbase` of (sequence b, kv head), and the
@@ -87,9 +90,27 @@ struct Column {
     int t, r;
     bool live;
 };
+// Columns this workgroup owns: all (token, head) pairs, or its group of up to 16 heads.
+__device__ inline int column_count(const DecodeArgs& a) { return a.n_cgroups > 1 ? min(16, a.n_rep - a.col0) : a.n_rep * a.T; }
 __device__ inline Column column_of(const DecodeArgs& a, int c) {
-    const int n = a.n_rep * a.T, cc = min(c, n - 1);
+    const int n = column_count(a), cc = min(c, n - 1);
+    if (a.n_cgroups > 1) return Column{0, a.col0 + cc, c < n};
     return Column{cc / a.n_rep, cc % a.n_rep, c < n};
+}
+// Which (work item, kv head) a workgroup serves.  kv head fastest: every item that exists comes before the first
+// surplus workgroup of the grid (which is sized for the longest possible batch), so the surplus ones start, find
+// nothing and exit under the tail of the real work.  With column groups, the groups of one (item, kv head) get block
+// ids 8 apart: the same XCD (ids are dealt round-robin to the 8 XCDs), so the K/V stream they share is fetched into
+// one L2, once, and read from there by the others.
+__device__ inline void block_coords(DecodeArgs& a, int& kvh, int& item) {
+    int ik = blockIdx.x;
+    if (a.n_cgroups > 1) {  // id = ((ik / 8) * n_cgroups + group) * 8 + ik % 8
+        const int rest = blockIdx.x >> 3;
+        a.col0 = 16 * (rest % a.n_cgroups);
+        ik = (rest / a.n_cgroups) * 8 + (blockIdx.x & 7);
+    }
+    kvh = ik % a.Hkv;
+    item = ik / a.Hkv;
 }
 // Keys [0, limit) are visible to column col: token t of T sits at position L - T + t and attends up to itself.
 __device__ inline int column_limit(const DecodeArgs& a, const Column& col, int L, int chunk_end) {
@@ -160,11 +181,10 @@ __global__ void __launch_bounds__(256, 2) decode_bf16_kernel(DecodeArgs a) {
     constexpr int KS = D / 32;   // MFMA k-steps over the head dim
     constexpr int DB = D / 16;   // 16-row tiles of O^T
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    // kv head fastest: every item that exists comes before the first surplus workgroup of the grid (which is sized for
-    // the longest possible batch), so the surplus ones start, find nothing and exit under the tail of the real work
-    const int kvh = blockIdx.x % a.Hkv;
+    int kvh, item;
+    block_coords(a, kvh, item);
     int b, split, L;
-    if (!locate_work(a, blockIdx.x / a.Hkv, lane, b, split, L)) return;
+    if (!locate_work(a, item, lane, b, split, L)) return;
     const int chunk_start = split * a.chunk;
     const int chunk_end = min(L, chunk_start + a.chunk);
 
@@ -296,7 +316,7 @@ __global__ void __launch_bounds__(256, 2) decode_bf16_kernel(DecodeArgs a) {
         }
     }
     __syncthreads();
-    for (int i = tid; i < a.n_rep * a.T * D; i += 256) {
+    for (int i = tid; i < column_count(a) * D; i += 256) {
         const int hc = i / D, d = i % D;
         float mm = sm_m[0][hc];
 #pragma unroll
@@ -340,11 +360,10 @@ __global__ void __launch_bounds__(256, 2) decode_q8_kernel(DecodeArgs a) {
     constexpr int NH = D / 64;  // 16-byte K loads per row per lane
     constexpr int NQ = D / kQBlock;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    // kv head fastest: every item that exists comes before the first surplus workgroup of the grid (which is sized for
-    // the longest possible batch), so the surplus ones start, find nothing and exit under the tail of the real work
-    const int kvh = blockIdx.x % a.Hkv;
+    int kvh, item;
+    block_coords(a, kvh, item);
     int b, split, L;
-    if (!locate_work(a, blockIdx.x / a.Hkv, lane, b, split, L)) return;
+    if (!locate_work(a, item, lane, b, split, L)) return;
     const int chunk_start = split * a.chunk;
     const int chunk_end = min(L, chunk_start + a.chunk);
 
@@ -515,7 +534,7 @@ __global__ void __launch_bounds__(256, 2) decode_q8_kernel(DecodeArgs a) {
         }
     }
     __syncthreads();
-    for (int i = tid; i < a.n_rep * a.T * D; i += 256) {
+    for (int i = tid; i < column_count(a) * D; i += 256) {
         const int hc = i / D, d = i % D;
         float mm = sm_m[0][hc];
 #pragma unroll
@@ -672,11 +691,10 @@ __global__ void __launch_bounds__(256, 2) decode_f32_mfma_kernel(DecodeArgs a) {
     constexpr int KT = 2;       // 16-key tiles per wavefront iteration
     constexpr int GROUP = 16 * KT;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    // kv head fastest: every item that exists comes before the first surplus workgroup of the grid (which is sized for
-    // the longest possible batch), so the surplus ones start, find nothing and exit under the tail of the real work
-    const int kvh = blockIdx.x % a.Hkv;
+    int kvh, item;
+    block_coords(a, kvh, item);
     int b, split, L;
-    if (!locate_work(a, blockIdx.x / a.Hkv, lane, b, split, L)) return;
+    if (!locate_work(a, item, lane, b, split, L)) return;
     const int chunk_start = split * a.chunk;
     const int chunk_end = min(L, chunk_start + a.chunk);
     const int c = lane & 15, g = lane >> 4;
@@ -802,7 +820,7 @@ __global__ void __launch_bounds__(256, 2) decode_f32_mfma_kernel(DecodeArgs a) {
         }
     }
     __syncthreads();
-    for (int i = tid; i < a.n_rep * a.T * D; i += 256) {
+    for (int i = tid; i < column_count(a) * D; i += 256) {
         const int hc = i / D, d = i % D;
         float mm = sm_m[0][hc];
 #pragma unroll
@@ -1166,7 +1184,8 @@ int decode_impl(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* s
     const int want_dtype = cache->format == VSP_KV_F32 ? VSP_F32 : VSP_BF16;
     if (q->dtype != out->dtype) return VSP_ERR_DTYPE;
     if (q->dtype != want_dtype) return VSP_ERR_UNSUPPORTED;
-    if (cache->format != VSP_KV_F32 && n_rep > 16) return VSP_ERR_UNSUPPORTED;
+    // bf16 / Q8_0: the query heads of a kv head ride in the 16 columns of the matrix instructions; more than 16 are
+    // served in groups of 16 (one token per sequence; ops::repeat_kv takes any n_rep, src/ops/attention_ops.cpp:92-155)
     if (cache->format == VSP_KV_F32 && D > 256) return VSP_ERR_UNSUPPORTED;
     // several tokens per sequence: they and the query heads of a kv head share the 16 columns of the matrix instructions
     if (T > 1 && (n_rep * T > 16 || (D != 64 && D != 128))) return VSP_ERR_UNSUPPORTED;
@@ -1221,10 +1240,17 @@ int decode_impl(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* s
     a.scale_log2 = scale * kLog2e;
     a.ws_o = (float*)workspace;
     a.ws_ml = a.ws_o ? a.ws_o + (size_t)B * Hq * T * max_splits * D : nullptr;
+    a.n_cgroups = (cache->format != VSP_KV_F32 && n_rep > 16) ? (n_rep + 15) / 16 : 1;
+    a.col0 = 0;
+    // (item, kv head) pairs in the grid, and the grid with one workgroup per pair and column group (pairs padded to a
+    // multiple of 8 when there are groups: see block_coords)
+    const int64_t pairs = (int64_t)max_splits * B * cache->Hkv;
+    const int64_t wgs = a.n_cgroups > 1 ? round_up(pairs, 8) * a.n_cgroups : pairs;
+    if (wgs > INT32_MAX) return VSP_ERR_ARG;
 
     if (max_len > 0) {
         if (cache->format == VSP_KV_BF16) {
-            dim3 grid((unsigned)(max_splits * B * cache->Hkv));
+            dim3 grid((unsigned)wgs);
             if (cache->page_table) {
                 if (D == 128) hipLaunchKernelGGL((decode_bf16_kernel<128, true>), grid, dim3(256), 0, st, a);
                 else hipLaunchKernelGGL((decode_bf16_kernel<64, true>), grid, dim3(256), 0, st, a);
@@ -1233,7 +1259,7 @@ int decode_impl(const vsp_tensor* q, const vsp_kv_cache* cache, const int32_t* s
                 else hipLaunchKernelGGL((decode_bf16_kernel<64, false>), grid, dim3(256), 0, st, a);
             }
         } else if (cache->format == VSP_KV_Q8_0) {
-            dim3 grid((unsigned)(max_splits * B * cache->Hkv));
+            dim3 grid((unsigned)wgs);
             if (cache->page_table) {
                 if (D == 128) hipLaunchKernelGGL((decode_q8_kernel<128, true>), grid, dim3(256), 0, st, a);
                 else hipLaunchKernelGGL((decode_q8_kernel<64, true>), grid, dim3(256), 0, st, a);

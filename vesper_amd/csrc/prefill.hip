@@ -66,6 +66,8 @@ struct PrefillArgs {
     int32_t n_splits, split_tiles;
     float* ws_o;
     float* ws_ml;
+    int32_t D_true;  // fp32 kernel: the tensors' head_dim when the kernel's tile is wider (columns past it read as zeros)
+    int32_t elementwise;  // fp32 kernel: rows are read element by element (any head_dim, any 4-byte aligned pitch)
 };
 
 constexpr int kBM = 128;       // queries per workgroup
@@ -1221,14 +1223,19 @@ __global__ void __launch_bounds__(256, 2) prefill_bf16_pipe_kernel(PrefillArgs a
 // ---------------------------------------------------------------------------------------------
 // fp32 kernel (fp32 inputs, fp32 MFMA 32x32x2, fp32 softmax): the precision the reference computes
 // in.  One wavefront owns 32 queries, a workgroup 128; key tiles of 32 through LDS.
+// GEN: the tensors' head_dim a.D_true is any value up to the tile width D (the reference's forward takes any
+// head_dim, src/ops/flash_attention.cpp:235-238): columns past it are zero in the operands (they add nothing to a
+// score) and are not stored; rows are read element by element, so they need no 16-byte alignment.
 // ---------------------------------------------------------------------------------------------
-template <int D>
+template <int D, bool GEN>
 __global__ void __launch_bounds__(256) prefill_f32_kernel(PrefillArgs a) {
     constexpr int BN = 32;
     constexpr int PITCH = D + 1;  // odd pitch: a column walk hits 32 different banks
     constexpr int DB = D / 32;
-    __shared__ float sK[BN * PITCH];
-    __shared__ float sV[BN * PITCH];
+    extern __shared__ float smem_f32[];  // K tile | V tile (2 * BN * PITCH floats, sized by the launch)
+    float* sK = smem_f32;
+    float* sV = smem_f32 + BN * PITCH;
+    const int Dt = GEN ? a.D_true : D;
 
     const int bid = blockIdx.x;
     const int qt = a.n_qtiles - 1 - bid / (a.B * a.Hq);
@@ -1249,7 +1256,7 @@ __global__ void __launch_bounds__(256) prefill_f32_kernel(PrefillArgs a) {
     // Q^T operands: column ql, contraction slot d = 2*ks + h
     float qf[D / 2];
 #pragma unroll
-    for (int ks = 0; ks < D / 2; ++ks) qf[ks] = Qp[2 * ks + h];
+    for (int ks = 0; ks < D / 2; ++ks) qf[ks] = (!GEN || 2 * ks + h < Dt) ? Qp[2 * ks + h] : 0.f;
 
     const int wg_qmax = min(qt * kBM + kBM - 1, a.T - 1);
     const int kv_end_wg = a.causal ? min(L, wg_qmax + off + 1) : L;
@@ -1266,6 +1273,14 @@ __global__ void __launch_bounds__(256) prefill_f32_kernel(PrefillArgs a) {
 
     for (int kt = 0; kt < n_tiles; ++kt) {
         __syncthreads();
+        if constexpr (GEN) {
+            for (int id = tid; id < BN * D; id += 256) {
+                const int row = id / D, col = id % D, key = kt * BN + row;
+                const bool ok = key < L && col < Dt;
+                sK[row * PITCH + col] = ok ? Kp[(int64_t)key * a.sk[2] + col] : 0.f;
+                sV[row * PITCH + col] = ok ? Vp[(int64_t)key * a.sv[2] + col] : 0.f;
+            }
+        } else
         for (int id = tid; id < BN * (D / 4); id += 256) {  // 16-byte loads (rows are 16-byte aligned), padded LDS rows
             const int row = id / (D / 4), col = 4 * (id % (D / 4)), key = kt * BN + row;
             float4 kk = {0.f, 0.f, 0.f, 0.f}, vv = kk;
@@ -1331,7 +1346,10 @@ __global__ void __launch_bounds__(256) prefill_f32_kernel(PrefillArgs a) {
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) op[32 * db + 8 * (v >> 2) + 4 * h + (v & 3)] = acc[db][v] * inv_l;
+            for (int v = 0; v < 16; ++v) {
+                const int d = 32 * db + 8 * (v >> 2) + 4 * h + (v & 3);
+                if (!GEN || d < Dt) op[d] = acc[db][v] * inv_l;
+            }
         if (a.lse && h == 0)
             a.lse[(int64_t)b * a.sl[0] + (int64_t)hq * a.sl[1] + (int64_t)qi * a.sl[2]] = (m_run + log2f(l)) * 0.6931471805599453f;
     }
@@ -1344,6 +1362,34 @@ int check_tensor4(const vsp_tensor* t, int esz) {
     for (int i = 0; i < 3; ++i)
         if ((t->stride[i] * esz) % 16 != 0) return VSP_ERR_ALIGN;
     return VSP_OK;
+}
+
+// fp32 tensors whose head_dim is not one of the native tiles: element-wise access, so 4-byte alignment is all it takes
+int check_tensor4_any_d(const vsp_tensor* t) {
+    if (t->stride[3] != 1) return VSP_ERR_STRIDE;
+    if (!t->data) return VSP_ERR_NULL;
+    if ((reinterpret_cast<uintptr_t>(t->data) & 3u) != 0) return VSP_ERR_ALIGN;
+    return VSP_OK;
+}
+bool native_head_dim(int dtype, int64_t D) { return D == 64 || D == 128 || (D == 32 && dtype == VSP_F32); }
+// the fp32 kernels' tile width for a head_dim they do not hold natively (0: none)
+int64_t padded_head_dim(int dtype, int64_t D) {
+    if (dtype != VSP_F32 || D < 1 || D > 256) return 0;
+    return D <= 32 ? 32 : D <= 64 ? 64 : D <= 128 ? 128 : 256;
+}
+
+template <int DP, bool GEN>
+int launch_prefill_f32(const PrefillArgs& a, dim3 grid, hipStream_t st) {
+    constexpr size_t lds = 2 * 32 * (DP + 1) * sizeof(float);
+    if constexpr (lds > 65536) {  // beyond the default limit of a launch: raised once per process
+        static const hipError_t e = hipFuncSetAttribute((const void*)prefill_f32_kernel<DP, GEN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) {
+            set_hip_error(e);
+            return VSP_ERR_LAUNCH;
+        }
+    }
+    hipLaunchKernelGGL((prefill_f32_kernel<DP, GEN>), grid, dim3(256), lds, st, a);
+    return check_launch();
 }
 
 int launch_prefill(const PrefillArgs& a, int dtype, int64_t D, bool cache_planes, void* stream) {
@@ -1369,9 +1415,18 @@ int launch_prefill(const PrefillArgs& a, int dtype, int64_t D, bool cache_planes
             else hipLaunchKernelGGL((prefill_bf16_kernel<64, false>), grid, block, 0, st, a);
         }
     } else {
-        if (D == 128) hipLaunchKernelGGL(prefill_f32_kernel<128>, grid, block, 0, st, a);
-        else if (D == 64) hipLaunchKernelGGL(prefill_f32_kernel<64>, grid, block, 0, st, a);
-        else hipLaunchKernelGGL(prefill_f32_kernel<32>, grid, block, 0, st, a);
+        if (!a.elementwise) {
+            if (D == 128) return launch_prefill_f32<128, false>(a, grid, st);
+            if (D == 64) return launch_prefill_f32<64, false>(a, grid, st);
+            if (D == 32) return launch_prefill_f32<32, false>(a, grid, st);
+        }
+        switch (padded_head_dim(dtype, D)) {  // a.D_true == D
+            case 32: return launch_prefill_f32<32, true>(a, grid, st);
+            case 64: return launch_prefill_f32<64, true>(a, grid, st);
+            case 128: return launch_prefill_f32<128, true>(a, grid, st);
+            case 256: return launch_prefill_f32<256, true>(a, grid, st);
+            default: return VSP_ERR_UNSUPPORTED;
+        }
     }
     return check_launch();
 }
@@ -1459,14 +1514,23 @@ extern "C" int vsp_attn_prefill_cached(const vsp_tensor* q, const vsp_kv_cache* 
         if (lse->dtype != VSP_F32) return VSP_ERR_DTYPE;
     }
     if (B * Hq * T * D == 0) return VSP_OK;
-    if (D != 64 && D != 128 && !(D == 32 && q->dtype == VSP_F32)) return VSP_ERR_UNSUPPORTED;  // fp32 also takes head_dim 32
+    // bf16: head_dim 64 or 128; fp32: any head_dim up to 256 (the native tiles 32 / 64 / 128, or the next one padded)
+    const bool native = native_head_dim(q->dtype, D);
+    if (!native && !padded_head_dim(q->dtype, D)) return VSP_ERR_UNSUPPORTED;
     if (!(fabsf(scale) > 0.0f) || !(fabsf(scale) < INFINITY)) return VSP_ERR_ARG;
     const int esz = q->dtype == VSP_F32 ? 4 : 2;
-    if ((rc = check_tensor4(q, esz)) != VSP_OK || (rc = check_tensor4(out, esz)) != VSP_OK) return rc;
+    bool elementwise = !native;
+    if (native && ((rc = check_tensor4(q, esz)) != VSP_OK || (rc = check_tensor4(out, esz)) != VSP_OK)) {
+        if (q->dtype != VSP_F32 || rc != VSP_ERR_ALIGN) return rc;
+        elementwise = true;  // fp32 rows that are not 16-byte aligned: the element-wise kernel takes them
+    }
+    if (elementwise && ((rc = check_tensor4_any_d(q)) != VSP_OK || (rc = check_tensor4_any_d(out)) != VSP_OK)) return rc;
     if (lse && !lse->data) return VSP_ERR_NULL;
     if (T > INT32_MAX / 2) return VSP_ERR_ARG;
 
     PrefillArgs a{};
+    a.D_true = (int)D;
+    a.elementwise = elementwise ? 1 : 0;
     a.q = q->data;
     a.k = cache->k;
     a.v = cache->v;
@@ -1601,13 +1665,22 @@ int prefill_entry(const vsp_tensor* q, const vsp_tensor* k, const vsp_tensor* v,
         if (lse->dtype != VSP_F32) return VSP_ERR_DTYPE;
     }
     if (B * Hq * T * D == 0) return VSP_OK;
-    if (D != 64 && D != 128 && !(D == 32 && q->dtype == VSP_F32)) return VSP_ERR_UNSUPPORTED;  // fp32 also takes head_dim 32
+    // bf16: head_dim 64 or 128; fp32: any head_dim up to 256, as the reference's forward takes any (:235-238): the native
+    // tiles 32 / 64 / 128, or the next one with the columns past head_dim padded with zeros inside the kernel
+    const bool native = native_head_dim(q->dtype, D);
+    if (!native && (split || !padded_head_dim(q->dtype, D))) return VSP_ERR_UNSUPPORTED;
     if (L == 0) return VSP_ERR_SHAPE;  // softmax over an empty context is undefined
     if (!(fabsf(scale) > 0.0f) || !(fabsf(scale) < INFINITY)) return VSP_ERR_ARG;
     const int esz = q->dtype == VSP_F32 ? 4 : 2;
     int rc;
-    if ((rc = check_tensor4(q, esz)) != VSP_OK || (rc = check_tensor4(k, esz)) != VSP_OK ||
-        (rc = check_tensor4(v, esz)) != VSP_OK || (rc = check_tensor4(out, esz)) != VSP_OK)
+    bool elementwise = !native;
+    if (native && ((rc = check_tensor4(q, esz)) != VSP_OK || (rc = check_tensor4(k, esz)) != VSP_OK ||
+                   (rc = check_tensor4(v, esz)) != VSP_OK || (rc = check_tensor4(out, esz)) != VSP_OK)) {
+        if (q->dtype != VSP_F32 || split || rc != VSP_ERR_ALIGN) return rc;
+        elementwise = true;  // fp32 rows that are not 16-byte aligned: the element-wise kernel takes them
+    }
+    if (elementwise && ((rc = check_tensor4_any_d(q)) != VSP_OK || (rc = check_tensor4_any_d(k)) != VSP_OK ||
+                        (rc = check_tensor4_any_d(v)) != VSP_OK || (rc = check_tensor4_any_d(out)) != VSP_OK))
         return rc;
     if (lse && !lse->data) return VSP_ERR_NULL;
     if (T > INT32_MAX / 2 || L > INT32_MAX / 2) return VSP_ERR_ARG;
@@ -1616,6 +1689,8 @@ int prefill_entry(const vsp_tensor* q, const vsp_tensor* k, const vsp_tensor* v,
     if (q->dtype == VSP_BF16 && (L * k->stride[2] * 2 > INT32_MAX || L * v->stride[2] * 2 > INT32_MAX)) return VSP_ERR_STRIDE;
 
     PrefillArgs a{};
+    a.D_true = (int)D;
+    a.elementwise = elementwise ? 1 : 0;
     a.q = q->data;
     a.k = k->data;
     a.v = v->data;
