@@ -355,14 +355,24 @@ def cpu_baseline(key):
 # they read for a 1 GiB read + 1 GiB write elementwise kernel launched by --copy-calibration in the same run.  Counters
 # cannot be collected inside a timed run, so these are properties of the workload shapes, not live values.
 PROFILE_OF = {
-    "c2": ("prefill_bf16_config2.txt", "prefill_bf16", 96 * 2**20 + 65 * 2**20),
-    "p4k": ("prefill_bf16_4k.txt", "prefill_bf16", 96 * 2**20 + 65 * 2**20),
-    "c3": ("prefill_bf16_config3.txt", "prefill_bf16", 96 * 2**20 + 65 * 2**20),
-    "c2c": ("prefill_bf16_cache_planes_config2.txt", "prefill_bf16", 96 * 2**20 + 65 * 2**20),
-    "r2": ("rope_append_bf16_config2.txt", "append_bf16_tile_kernel<unsigned short, true", 202375168),
-    "c4": ("decode_bf16_config4.txt", "decode_bf16_kernel", 2614935552),
-    "c5": ("decode_q8_0_config5.txt", "decode_q8_kernel", 2282225664),
-    "c4f": ("decode_f32_config4.txt", "decode_f32_mfma_kernel", 5229871104),
+    # workload: (summary under profiles/, name fragments of the step's kernels (their counters are added up), algorithmic
+    # bytes of a step: every input read once and every output written once)
+    "c2": ("prefill_bf16_config2.txt", ("prefill_bf16",), 96 * 2**20 + 65 * 2**20),
+    "p4k": ("prefill_bf16_4k.txt", ("prefill_bf16",), 96 * 2**20 + 65 * 2**20),
+    "c3": ("prefill_bf16_config3.txt", ("prefill_bf16",), 96 * 2**20 + 65 * 2**20),
+    "c2c": ("prefill_bf16_cache_planes_config2.txt", ("prefill_bf16",), 96 * 2**20 + 65 * 2**20),
+    "c3c": ("prefill_bf16_cache_planes_config3.txt", ("prefill_bf16",), 96 * 2**20 + 65 * 2**20),
+    "k512": ("prefill_bf16_chunk512_context32k.txt", ("prefill_bf16", "decode_combine_kernel"), 2 * 4194304 + 2 * 67108864),
+    "c2f": ("prefill_split_f32_config2.txt", ("prefill_split_kernel", "split_f32_kernel"), 2 * 134217728 + 2 * 33554432),
+    "r2": ("rope_append_bf16_config2.txt", ("append_bf16_tile_kernel<unsigned short, true",), 202375168),
+    "c4": ("decode_bf16_config4.txt", ("decode_bf16_kernel", "decode_combine_kernel"), 2614935552),
+    "c4m": ("decode_bf16_multi_config4.txt", ("decode_bf16_kernel", "decode_combine_kernel"), 2614935552 + 3 * 524288),
+    "c4w": ("decode_bf16_proj_config4.txt", ("decode_bf16_kernel", "decode_combine_kernel", "proj_bf16_partial_kernel", "proj_reduce_kernel"),
+            2614935552 + 33554432),
+    "c5": ("decode_q8_0_config5.txt", ("decode_q8_kernel", "decode_combine_kernel"), 2282225664),
+    "c4f": ("decode_f32_config4.txt", ("decode_f32_mfma_kernel", "decode_combine_kernel"), 5229871104),
+    # backward: Q, dO, O, K, V, lse read; dQ, dK, dV written
+    "b2": ("backward_bf16_config2.txt", ("bwd_dq_bf16_kernel", "bwd_dkdv_bf16_kernel"), 4 * 67108864 + 4 * 16777216 + 1048576),
 }
 CALIBRATION_KERNEL, CALIBRATION_KIB = "CUDAFunctorOnSelf_add<int>", 1048576.0
 
@@ -371,7 +381,7 @@ def traffic_from_profile(key):
     """{"fetch_bytes", "write_bytes", "algorithmic_bytes", "source"} parsed from profiles/<file>, or None."""
     if key not in PROFILE_OF:
         return None
-    fname, kernel, algorithmic = PROFILE_OF[key]
+    fname, kernels, algorithmic = PROFILE_OF[key]
     path = os.path.join(ROOT, "profiles", fname)
     if not os.path.exists(path):
         return None
@@ -385,9 +395,11 @@ def traffic_from_profile(key):
             left, right = line.rsplit(section, 1)
             cols = right.split()
             if len(cols) >= 2:
-                name = "calibration" if CALIBRATION_KERNEL in left else ("kernel" if kernel in left else None)
-                if name and name not in raw[section]:
-                    raw[section][name] = float(cols[1])  # columns after the counter name: n, avg, min, max
+                value = float(cols[1])  # columns after the counter name: n, avg, min, max
+                if CALIBRATION_KERNEL in left:
+                    raw[section].setdefault("calibration", value)
+                elif any(k in left for k in kernels):
+                    raw[section]["kernel"] = raw[section].get("kernel", 0.0) + value  # one line per kernel and counter
     try:
         for section, field in (("FETCH_SIZE", "fetch_bytes"), ("WRITE_SIZE", "write_bytes")):
             scale = CALIBRATION_KIB / raw[section]["calibration"]

@@ -41,6 +41,18 @@ def assert_bf16_close(got_f32, want_f32, what=""):
     assert err.mean() <= BF16_MEAN_ABS, f"{what}: mean-abs {err.mean():.4g} > {BF16_MEAN_ABS}"
 
 
+def assert_bf16_close_wide_range(got_f32, want_f32, what=""):
+    """The bf16 bar for outputs that are not of order one: max-abs 2e-2 plus one bf16 step of the expected value itself
+    (storing an exact result of magnitude 4 as bf16 already moves it by up to 0.0156), elementwise; mean-abs as usual."""
+    assert np.isfinite(got_f32).all(), what
+    want = want_f32.astype(np.float64)
+    err = np.abs(got_f32.astype(np.float64) - want)
+    ulp = np.exp2(np.floor(np.log2(np.maximum(np.abs(want), 2.0 ** -126))) - 7)   # spacing of bf16 numbers at |want|
+    over = err - (BF16_MAX_ABS + ulp)
+    assert over.max() <= 0, f"{what}: error {err.flat[over.argmax()]:.4g} where 2e-2 + one bf16 step is {BF16_MAX_ABS + ulp.flat[over.argmax()]:.4g}"
+    assert err.mean() <= BF16_MEAN_ABS, f"{what}: mean-abs {err.mean():.4g} > {BF16_MEAN_ABS}"
+
+
 def assert_f32_close(got, want, what=""):
     """1e-4 relative, measured against the magnitude of the reference output (elementwise relative error
     is meaningless where the output crosses zero)."""
