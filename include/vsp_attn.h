@@ -221,8 +221,14 @@ int vsp_attn_prefill_split(const vsp_tensor* q, const vsp_tensor* k, const vsp_t
  * accumulation, P and dS rounded to bf16 between the products, gradients rounded to nearest even; base pointers and
  * strides multiples of 16 bytes (VSP_ERR_ALIGN), stride[2] >= D (VSP_ERR_STRIDE).  D in {64,128}, fp32 also 32.  dq/dk/dv are
  * overwritten.  No atomics: results are bitwise reproducible (the reference's
- * HIP kernel accumulates dQ with atomicAdd).  workspace: vsp_attn_backward_workspace_bytes(B, Hq, N) bytes. */
+ * HIP kernel accumulates dQ with atomicAdd).  workspace: vsp_attn_backward_workspace_bytes(B, Hq, N) bytes.
+ * bf16 with a workspace of at least vsp_attn_backward_fast_workspace_bytes(B, Hq, N) bytes (16-byte aligned; about
+ * 2 N^2 bytes per query head on top of the former): dS is computed once instead of twice - the dK / dV pass leaves
+ * every 32 x 32 tile of it in the workspace as bf16 and dQ is one product over those tiles - five tile products
+ * instead of seven for the price of writing and reading the tiles, which the matrix-core-bound passes have the memory
+ * bandwidth for.  Same rounding points (dS enters both of its products as the same bf16 values); still no atomics. */
 size_t vsp_attn_backward_workspace_bytes(int32_t B, int32_t Hq, int32_t N);
+size_t vsp_attn_backward_fast_workspace_bytes(int32_t B, int32_t Hq, int32_t N);
 int vsp_attn_prefill_backward(const vsp_tensor* dout, const vsp_tensor* q, const vsp_tensor* k, const vsp_tensor* v,
                               const vsp_tensor* out, const vsp_tensor* lse, vsp_tensor* dq, vsp_tensor* dk,
                               vsp_tensor* dv, float scale, int is_causal, void* workspace, size_t workspace_bytes,

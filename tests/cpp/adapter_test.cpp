@@ -401,6 +401,25 @@ static void test_backward_dispatch_seam() {
     // the front end with the reference's defaults (is_causal = true, dropout_p = 0, no mask)
     auto g = ops::flash_attention_backward(tdo, tq, tk, tv, o, l, scale);
     CHECK(max_abs_diff(to_host(std::get<0>(g)), wq.data(), wq.size()) < 2e-4);
+    // bf16 tensors: with the larger workspace (the default while it stays under backward_fast_workspace_limit()) dS is
+    // computed once, with the limit at 0 twice; both inside the bf16 bar against the fp32 oracle, and dK / dV the same
+    {
+        Tensor bq = to_dev(q, {B, Hq, N, D}, DType::BFloat16), bk = to_dev(k, {B, Hkv, N, D}, DType::BFloat16);
+        Tensor bv = to_dev(v, {B, Hkv, N, D}, DType::BFloat16), bdo = to_dev(dout, {B, Hq, N, D}, DType::BFloat16);
+        Tensor bo = empty({B, Hq, N, D}, DType::BFloat16), bl = empty({B, Hq, N}, DType::Float32);
+        ops::flash_attention_hip_dispatch(bq, ops::repeat_kv(bk, n), ops::repeat_kv(bv, n), bo, bl, scale, true, 0.0f, false, nullptr);
+        auto once = ops::flash_attention_backward(bdo, bq, bk, bv, bo, bl, scale);
+        const size_t keep = ops::backward_fast_workspace_limit();
+        ops::backward_fast_workspace_limit() = 0;
+        auto twice = ops::flash_attention_backward(bdo, bq, bk, bv, bo, bl, scale);
+        ops::backward_fast_workspace_limit() = keep;
+        CHECK(max_abs_diff(to_host(std::get<0>(once)), wq.data(), wq.size()) < 3e-2);
+        CHECK(max_abs_diff(to_host(std::get<0>(twice)), wq.data(), wq.size()) < 3e-2);
+        CHECK(max_abs_diff(to_host(std::get<1>(once)), wk.data(), wk.size()) < 5e-2);
+        CHECK(max_abs_diff(to_host(std::get<2>(once)), wv.data(), wv.size()) < 5e-2);
+        auto dk1 = to_host(std::get<1>(once)), dk2 = to_host(std::get<1>(twice));
+        CHECK(max_abs_diff(dk1, dk2.data(), dk2.size()) < 1e-2);
+    }
 }
 
 static void test_multi_head_attention_core() {

@@ -277,6 +277,11 @@ static void test_validation() {
     CHECK(vsp_attn_prefill_backward(&q, &q, &k, &k, &q, &lse, &q, &k, &k, 0.1f, 1, nullptr, 0, nullptr) == VSP_ERR_WORKSPACE);
     CHECK(vsp_attn_prefill_backward(&q, &q, &k5, &k5, &q, &lse, &q, &k5, &k5, 0.1f, 1, mem, 1 << 16, nullptr) == VSP_ERR_SHAPE);
     CHECK(vsp_attn_backward_workspace_bytes(1, 4, 8) == 2u * 4 * 8 * 4);
+    // the larger one: the former rounded up to 256 bytes, then one 2 KB tile per (32 queries, 32 keys), key tiles in pairs
+    CHECK(vsp_attn_backward_fast_workspace_bytes(1, 4, 8) == 256u + 4u * 1 * 2 * 2048);
+    CHECK(vsp_attn_backward_fast_workspace_bytes(2, 4, 100) == 6400u + 2u * 4 * 4 * 4 * 2048);
+    CHECK(vsp_attn_backward_fast_workspace_bytes(1, 32, 8192) == 2u * 32 * 8192 * 4 + (size_t)32 * 256 * 256 * 2048);
+    CHECK(vsp_attn_backward_fast_workspace_bytes(0, 4, 8) == 0 && vsp_attn_backward_fast_workspace_bytes(1, 4, 0) == 0);
     // backward with split operands: fp32 only, head_dim 64 / 128, workspace for Di, lse and the eight planes
     {
         vsp_tensor qf = tensor4(mem, VSP_F32, 1, 4, 8, 64), kf = tensor4(mem, VSP_F32, 1, 2, 8, 64), k3 = tensor4(mem, VSP_F32, 1, 3, 8, 64);

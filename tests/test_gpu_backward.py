@@ -24,11 +24,12 @@ def va():
     return vesper_amd
 
 
-def _forward_then_backward(va, q, k, v, dout, scale, causal, bf16=False):
+def _forward_then_backward(va, q, k, v, dout, scale, causal, bf16=False, fast=False):
+    # fast: the larger workspace, with which the bf16 path computes dS once (vsp_attn_backward_fast_workspace_bytes)
     cv = G.to_bf16_dev if bf16 else G.f32_dev
     dq_, dk_, dv_, dd_ = cv(q), cv(k), cv(v), cv(dout)
     out, lse = va.flash_attention(dq_, dk_, dv_, scale, causal, return_lse=True)
-    return va.flash_attention_backward(dd_, dq_, dk_, dv_, out, lse, scale, causal)
+    return va.flash_attention_backward(dd_, dq_, dk_, dv_, out, lse, scale, causal, workspace=va.backward_workspace(dq_, fast=fast))
 
 
 def test_fixture_written_from_the_reference(va):
@@ -98,13 +99,14 @@ def test_single_token(va):
     G.assert_f32_close(dv.cpu().numpy(), dout, "dv")
 
 
-def test_bf16_inputs_and_determinism(va):
+@pytest.mark.parametrize("fast", [False, True])
+def test_bf16_inputs_and_determinism(va, fast):
     B, Hq, Hkv, N, D = 2, 8, 2, 300, 128
     q, k, v = [O.bf16_round(x * np.float32(0.5)) for x in I.qkv(800, B, Hq, Hkv, N, N, D)]
     dout = O.bf16_round(I.normal(805, (B, Hq, N, D)))
     scale = 1.0 / math.sqrt(D)
-    dq, dk, dv = _forward_then_backward(va, q, k, v, dout, scale, True, bf16=True)
-    again = _forward_then_backward(va, q, k, v, dout, scale, True, bf16=True)
+    dq, dk, dv = _forward_then_backward(va, q, k, v, dout, scale, True, bf16=True, fast=fast)
+    again = _forward_then_backward(va, q, k, v, dout, scale, True, bf16=True, fast=fast)
     for a, b in zip((dq, dk, dv), again):
         assert torch.equal(a, b)          # no atomics: bitwise reproducible
     kr, vr = O.repeat_kv(k, 4), O.repeat_kv(v, 4)
@@ -121,8 +123,9 @@ def test_bf16_inputs_and_determinism(va):
 
 @pytest.mark.parametrize("B,Hq,Hkv,N,D,causal", [(1, 4, 2, 100, 64, True), (2, 8, 2, 257, 128, True), (1, 4, 4, 64, 128, False),
                                                  (1, 6, 1, 33, 64, True), (1, 2, 1, 129, 128, False), (1, 8, 8, 1, 64, True),
-                                                 (1, 4, 1, 512, 128, True)])
-def test_bf16_against_oracle(va, B, Hq, Hkv, N, D, causal):
+                                                 (1, 4, 1, 512, 128, True), (1, 2, 2, 96, 64, True), (2, 4, 2, 200, 128, False)])
+@pytest.mark.parametrize("fast", [False, True])
+def test_bf16_against_oracle(va, B, Hq, Hkv, N, D, causal, fast):
     q, k, v = [O.bf16_round(x) for x in I.qkv(820 + N, B, Hq, Hkv, N, N, D)]
     dout = O.bf16_round(I.normal(825 + N, (B, Hq, N, D)))
     scale = float(np.float32(1.0 / np.sqrt(D)))
@@ -132,7 +135,7 @@ def test_bf16_against_oracle(va, B, Hq, Hkv, N, D, causal):
     wq, wk, wv = O.flash_attention_backward(dout, q, kr, vr, out, lse, scale, causal)
     wk = wk.reshape(B, Hkv, n, N, D).sum(2)
     wv = wv.reshape(B, Hkv, n, N, D).sum(2)
-    dq, dk, dv = _forward_then_backward(va, q, k, v, dout, scale, causal, bf16=True)
+    dq, dk, dv = _forward_then_backward(va, q, k, v, dout, scale, causal, bf16=True, fast=fast)
     for got, want, name in ((dq, wq, "dq"), (dk, wk, "dk"), (dv, wv, "dv")):
         g = G.bf16_to_np(got)
         err = np.abs(g - want)
@@ -141,8 +144,31 @@ def test_bf16_against_oracle(va, B, Hq, Hkv, N, D, causal):
         assert err.mean() <= 2e-3 * ref, (name, err.mean(), ref)
 
 
-@pytest.mark.parametrize("bf16", [False, True])
-def test_strided_operands(va, bf16):
+def test_bf16_dS_once_against_dS_twice(va):
+    # The two bf16 paths differ in where dQ's dS comes from: recomputed from the fp32 P in the dQ pass, or the tiles the
+    # dK / dV pass left behind (P rounded to bf16 first: one more rounding of 2^-9 relative per element of dS), and in
+    # the summation order of Di.  dK and dV go through the same arithmetic in both.
+    B, Hq, Hkv, N, D = 2, 8, 2, 1000, 128
+    g = torch.Generator(device="cuda").manual_seed(23)
+    mk = lambda h: (torch.randn(B, h, N, D, device=G.dev(), generator=g) * 0.7).to(torch.bfloat16)
+    q, k, v, dout = mk(Hq), mk(Hkv), mk(Hkv), mk(Hq)
+    scale = 1.0 / math.sqrt(D)
+    for causal in (True, False):
+        out, lse = va.flash_attention(q, k, v, scale, causal, return_lse=True)
+        two = va.flash_attention_backward(dout, q, k, v, out, lse, scale, causal)
+        ws = va.backward_workspace(q, fast=True)
+        ws.fill_(0xff)            # stale tiles would show as NaNs
+        one = va.flash_attention_backward(dout, q, k, v, out, lse, scale, causal, workspace=ws)
+        for a, b, name in zip(one, two, ("dq", "dk", "dv")):
+            a, b = a.float(), b.float()
+            assert torch.isfinite(a).all(), name
+            ref = max(1.0, b.abs().max().item())
+            assert (a - b).abs().max().item() <= (2e-2 if name == "dq" else 8e-3) * ref, (name, causal, (a - b).abs().max().item())
+            assert (a - b).abs().mean().item() <= (1e-3 if name == "dq" else 1e-4) * ref, (name, causal, (a - b).abs().mean().item())
+
+
+@pytest.mark.parametrize("bf16,fast", [(False, False), (True, False), (True, True)])
+def test_strided_operands(va, bf16, fast):
     # [B, N, H, D] storage viewed as [B, H, N, D] (what a fused qkv projection hands over): the strides of every
     # operand and of every gradient are honoured
     B, Hq, Hkv, N, D = 2, 4, 2, 70, 64
@@ -153,8 +179,9 @@ def test_strided_operands(va, bf16):
     strided = [t.transpose(1, 2).contiguous().transpose(1, 2) for t in dense]
     assert not strided[0].is_contiguous()
     out, lse = va.flash_attention(dense[1], dense[2], dense[3], 0.125, True, return_lse=True)
-    want = va.flash_attention_backward(*dense, out, lse, 0.125, True)
-    got = va.flash_attention_backward(*strided, out.transpose(1, 2).contiguous().transpose(1, 2), lse, 0.125, True)
+    ws = lambda: va.backward_workspace(dense[1], fast=fast)
+    want = va.flash_attention_backward(*dense, out, lse, 0.125, True, workspace=ws())
+    got = va.flash_attention_backward(*strided, out.transpose(1, 2).contiguous().transpose(1, 2), lse, 0.125, True, workspace=ws())
     for g, w in zip(got, want):
         assert g.stride() != w.stride() and torch.equal(g, w)
 
@@ -168,7 +195,8 @@ def test_bf16_rows_must_be_16_byte_aligned(va):
         va.flash_attention_backward(ok, off, ok, ok, ok, torch.zeros(1, 2, 8, device=d), 0.1)
 
 
-def test_bf16_config3_shape_causal_truncation(va):
+@pytest.mark.parametrize("fast", [False, True])
+def test_bf16_config3_shape_causal_truncation(va, fast):
     # benchmark config 3's shape (B1, 32/8 heads, D128, N8192).  With dO = 0 from row n on, causal attention makes the
     # first n rows of dq / dk / dv those of the n-token problem - bit for bit, because the later query tiles add exact
     # zeros (dP = 0, Di = 0, so dS = 0, and P * 0 = 0) in between the same partial sums - and the rest exactly zero.
@@ -179,9 +207,10 @@ def test_bf16_config3_shape_causal_truncation(va):
     dout[:, :, n:] = 0
     scale = 1.0 / math.sqrt(D)
     out, lse = va.flash_attention(q, k, v, scale, True, return_lse=True)
-    dq, dk, dv = va.flash_attention_backward(dout, q, k, v, out, lse, scale, True)
+    dq, dk, dv = va.flash_attention_backward(dout, q, k, v, out, lse, scale, True, workspace=va.backward_workspace(q, fast=fast))
     cut = lambda t: t[:, :, :n].contiguous()
-    sq, sk, sv = va.flash_attention_backward(cut(dout), cut(q), cut(k), cut(v), cut(out), lse[:, :, :n].contiguous(), scale, True)
+    sq, sk, sv = va.flash_attention_backward(cut(dout), cut(q), cut(k), cut(v), cut(out), lse[:, :, :n].contiguous(), scale, True,
+                                             workspace=va.backward_workspace(cut(q), fast=fast))
     for big, small, name in ((dq, sq, "dq"), (dk, sk, "dk"), (dv, sv, "dv")):
         assert torch.isfinite(big.float()).all(), name
         assert torch.equal(big[:, :, :n], small), name

@@ -75,16 +75,16 @@ def test_backward_random_shapes(va, seed):
     out, lse = O.flash_attention(q, kr, vr, scale, causal, return_lse=True)
     wq, wk, wv = O.flash_attention_backward(dout, q, kr, vr, out, lse, scale, causal)
     wk, wv = wk.reshape(B, Hkv, n, N, D).sum(2), wv.reshape(B, Hkv, n, N, D).sum(2)
-    for bf16 in (False, True):
+    for bf16, fast in ((False, False), (True, False), (True, True)):   # fast: the workspace that keeps dS (bf16 only)
         cv = G.to_bf16_dev if bf16 else G.f32_dev
         tq, tk, tv, td = cv(q), cv(k), cv(v), cv(dout)
         o, l = va.flash_attention(tq, tk, tv, scale, causal, return_lse=True)
-        got = va.flash_attention_backward(td, tq, tk, tv, o, l, scale, causal)
+        got = va.flash_attention_backward(td, tq, tk, tv, o, l, scale, causal, workspace=va.backward_workspace(tq, fast=fast))
         for g, w, name in zip(got, (wq, wk, wv), ("dq", "dk", "dv")):
             if bf16:
                 err = np.abs(G.bf16_to_np(g) - w)
                 ref = max(1.0, float(np.abs(w).max()))
-                assert err.max() <= 2e-2 * ref and err.mean() <= 2e-3 * ref, (name, c, err.max(), ref)
+                assert err.max() <= 2e-2 * ref and err.mean() <= 2e-3 * ref, (name, c, fast, err.max(), ref)
             else:   # 1e-4 of the gradient's scale; a gradient that is exactly zero (N = 1: dS = P (dP - Di) with
                     # dP = Di up to rounding) has no scale of its own and gets 1e-5 absolute
                 err = np.abs(g.cpu().numpy() - w)

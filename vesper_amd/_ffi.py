@@ -47,6 +47,7 @@ SYMBOLS = {
     "vsp_attn_prefill_split_workspace_bytes": (C.c_size_t, [C.c_int32] * 6),
     "vsp_attn_prefill_split": (C.c_int, [_TP] * 5 + [C.c_float, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]),
     "vsp_attn_backward_workspace_bytes": (C.c_size_t, [C.c_int32] * 3),
+    "vsp_attn_backward_fast_workspace_bytes": (C.c_size_t, [C.c_int32] * 3),
     "vsp_attn_prefill_backward": (C.c_int, [_TP] * 9 + [C.c_float, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]),
     "vsp_attn_backward_split_workspace_bytes": (C.c_size_t, [C.c_int32] * 5),
     "vsp_attn_prefill_backward_split": (C.c_int, [_TP] * 9 + [C.c_float, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]),

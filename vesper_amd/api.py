@@ -77,15 +77,21 @@ def flash_attention_split(q, k, v, scale, is_causal=True, return_lse=False, work
     return (out, lse) if return_lse else out
 
 
-def flash_attention_backward(grad_output, q, k, v, output, lse, scale, is_causal=True):
+def backward_workspace(q, fast=False):
+    """Workspace of flash_attention_backward for tensors of q's shape; fast: the larger one that lets the bf16 path
+    compute dS once (vsp_attn_backward_fast_workspace_bytes)."""
+    f = lib.vsp_attn_backward_fast_workspace_bytes if fast else lib.vsp_attn_backward_workspace_bytes
+    return torch.empty(max(f(q.shape[0], q.shape[1], q.shape[2]), 16), dtype=torch.uint8, device=q.device)
+
+
+def flash_attention_backward(grad_output, q, k, v, output, lse, scale, is_causal=True, workspace=None):
     """ops::flash_attention_backward: (dq, dk, dv); k, v may have fewer heads than q (their gradients then sum over
-    the query heads of each group)."""
+    the query heads of each group).  workspace: from backward_workspace(); its size selects the bf16 path."""
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     descs = [_desc(t) for t in (grad_output, q, k, v, output, lse, dq, dk, dv)]
-    nws = lib.vsp_attn_backward_workspace_bytes(q.shape[0], q.shape[1], q.shape[2])
-    ws = torch.empty(max(nws, 4), dtype=torch.uint8, device=q.device)
+    ws = workspace if workspace is not None else backward_workspace(q)
     check(lib.vsp_attn_prefill_backward(*[C.byref(d) for d in descs], float(scale), int(bool(is_causal)),
-                                        C.c_void_p(ws.data_ptr()), nws, _stream(q)))
+                                        C.c_void_p(ws.data_ptr()), ws.numel(), _stream(q)))
     return dq, dk, dv
 
 

@@ -515,6 +515,13 @@ inline Tensor flash_attention_split(const Tensor& q, const Tensor& k, const Tens
     return output;
 }
 
+// bf16 backward: the larger workspace, with which dS is computed once and kept as tiles (about 2 N^2 bytes per query
+// head, vsp_attn_backward_fast_workspace_bytes), is taken when it is no larger than this many bytes; 0 switches it off.
+inline size_t& backward_fast_workspace_limit() {
+    static size_t limit = (size_t)8 << 30;
+    return limit;
+}
+
 // include/vesper/ops/flash_attention.h:80-92 (defined src/ops/hip/flash_attention.hip:183-299): the gradients are
 // caller-allocated.  A dropout mask can only come from a training forward with dropout_p > 0, which this path
 // rejects, so a non-null mask with dropout_p > 0 is VSP_ERR_UNSUPPORTED here too.
@@ -535,7 +542,11 @@ inline void flash_attention_backward_hip_dispatch(const Tensor& grad_output, con
                                                      split_bytes, current_stream()));
         return;
     }
-    const size_t ws_bytes = q.ndim() == 4 ? vsp_attn_backward_workspace_bytes((int32_t)q.shape()[0], (int32_t)q.shape()[1], (int32_t)q.shape()[2]) : 0;
+    size_t ws_bytes = q.ndim() == 4 ? vsp_attn_backward_workspace_bytes((int32_t)q.shape()[0], (int32_t)q.shape()[1], (int32_t)q.shape()[2]) : 0;
+    if (q.ndim() == 4 && q.dtype() == DType::BFloat16) {   // dS kept instead of recomputed, when the tiles are affordable
+        const size_t fast = vsp_attn_backward_fast_workspace_bytes((int32_t)q.shape()[0], (int32_t)q.shape()[1], (int32_t)q.shape()[2]);
+        if (fast > 0 && fast <= backward_fast_workspace_limit()) ws_bytes = fast;
+    }
     Storage ws(ws_bytes ? ws_bytes : 4);
     throw_status(vsp_attn_prefill_backward(&d0, &d1, &d2, &d3, &d4, &d5, &o0, &o1, &o2, scale, is_causal ? 1 : 0, ws.data(), ws_bytes,
                                            current_stream()));

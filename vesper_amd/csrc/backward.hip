@@ -36,6 +36,10 @@ struct BwdArgs {
     float scale;
     int64_t lo_q, lo_kv;                   // split operands: elements from a hi plane to its lo plane (q-shaped, kv-shaped)
     int32_t D_true;                        // fp32 kernels: the tensors' head_dim (<= the kernel's tile width; columns past it are zero)
+    // bf16, one-pass dS: the dK / dV pass leaves every dS tile (32 keys x 32 queries, bf16, [key][query], 2 KB) in the
+    // workspace at [b][hq][query tile][key tile], and dQ is one product over those tiles
+    uint16_t* ds_tiles;
+    int32_t n_qt32, n_kt32;                // query tiles per head, key tiles per head (an even number: key blocks come in pairs)
 };
 
 template <typename T>
@@ -68,6 +72,35 @@ __global__ void __launch_bounds__(256) bwd_delta_kernel(BwdArgs a, int D) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
     if (lane == 0) a.delta[row] = s;
+}
+
+// bf16 operands: Di as above and lse * log2(e), the two per-row constants of the dK / dV pass, when no dQ pass has
+// run before it.  D / 8 lanes per row, 16 bytes of O and dO each.
+template <int D>
+__global__ void __launch_bounds__(256) bwd_rowstats_bf16_kernel(BwdArgs a) {
+    constexpr int LPR = D / 8, RPB = 256 / LPR;
+    const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / LPR;
+    const int piece = threadIdx.x % LPR;
+    const int64_t rows = (int64_t)a.B * a.Hq * a.N;
+    const int64_t rr = row < rows ? row : rows - 1;
+    const int i = (int)(rr % a.N);
+    const int64_t bh = rr / a.N;
+    const int h = (int)(bh % a.Hq), b = (int)(bh / a.Hq);
+    const uint4 wo = *(const uint4*)((const uint16_t*)a.out + (int64_t)b * a.s_o[0] + (int64_t)h * a.s_o[1] + (int64_t)i * a.s_o[2] + 8 * piece);
+    const uint4 wd = *(const uint4*)((const uint16_t*)a.dout + (int64_t)b * a.s_do[0] + (int64_t)h * a.s_do[1] + (int64_t)i * a.s_do[2] + 8 * piece);
+    const uint32_t o4[4] = {wo.x, wo.y, wo.z, wo.w}, d4[4] = {wd.x, wd.y, wd.z, wd.w};
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        s += __uint_as_float(o4[j] << 16) * __uint_as_float(d4[j] << 16);
+        s += __uint_as_float(o4[j] & 0xffff0000u) * __uint_as_float(d4[j] & 0xffff0000u);
+    }
+#pragma unroll
+    for (int o = LPR / 2; o > 0; o >>= 1) s += __shfl_xor(s, o);
+    if (row < rows && piece == 0) {
+        a.delta[row] = s;
+        a.lse2[row] = 1.4426950408889634f * a.lse[(int64_t)b * a.s_l[0] + (int64_t)h * a.s_l[1] + (int64_t)i * a.s_l[2]];
+    }
 }
 
 constexpr int kBQ = 128;  // rows (queries or keys) per workgroup, 32 per wavefront
@@ -556,7 +589,9 @@ constexpr int kBK = 64;   // key rows per workgroup in the bf16 dK / dV pass
 
 // SPLIT: as in bwd_dq_bf16_kernel; P crosses to the partner as fp32, and each wavefront splits what it feeds to its
 // own second product (P or dS) into two bf16 terms.
-template <int D, bool SPLIT = false>
+// SPILL: the D wavefront also leaves dS of every (query tile, key block) in the workspace (a.ds_tiles), from where
+// bwd_dq_stream_kernel takes dQ with one product instead of the three of bwd_dq_bf16_kernel.
+template <int D, bool SPLIT = false, bool SPILL = false>
 __global__ void __launch_bounds__(256, SPLIT ? 1 : 2) bwd_dkdv_bf16_kernel(BwdArgs a) {
     constexpr int KS = D / 16, DB = D / 32;
     // One variable per ring slot: the compiler then knows that a read of one slot does not touch the slot a
@@ -606,6 +641,15 @@ __global__ void __launch_bounds__(256, SPLIT ? 1 : 2) bwd_dkdv_bf16_kernel(BwdAr
     const int qt_begin = a.causal ? (kt * kBK) / kBT : 0;
     const int n_qt = (a.N + kBT - 1) / kBT - qt_begin;   // query tiles per head
     const int n_it = a.n_rep * n_qt;                     // the loop runs over (head of the group, query tile)
+    // SPILL: where the D wavefront leaves its next dS tile; query tiles of a head are n_kt32 tiles apart, heads
+    // n_qt32 * n_kt32
+    char* ds_tile = nullptr;
+    int64_t ds_step_t = 0, ds_step_r = 0;   // to the next query tile; from the last query tile of a head to the first of the next
+    if constexpr (SPILL) {
+        ds_step_t = (int64_t)a.n_kt32 * 2048;
+        ds_step_r = (int64_t)a.n_qt32 * ds_step_t - (int64_t)(n_qt - 1) * ds_step_t;
+        ds_tile = (char*)a.ds_tiles + ((((int64_t)b * a.Hq + kvh * a.n_rep) * a.n_qt32 + qt_begin) * a.n_kt32 + (key0 >> 5)) * 2048 + lane * 16;
+    }
     const float scale_log2 = a.scale * kLog2e;
 
     TileDma<D> dq_, do_;
@@ -613,7 +657,7 @@ __global__ void __launch_bounds__(256, SPLIT ? 1 : 2) bwd_dkdv_bf16_kernel(BwdAr
     do_.init(a.s_do[2], wave, lane);
     // (head of the group, query tile) of the tile being fetched and of the tile whose first products are due:
     // the loop index split without a division per step
-    int ld_r = 0, ld_t = 0, fi_r = 0, fi_t = 0;
+    int ld_r = 0, ld_t = 0, fi_r = 0, fi_t = 0, se_t = 0;
     auto advance = [&](int& r, int& t) {
         if (++t == n_qt) {
             t = 0;
@@ -722,6 +766,20 @@ __global__ void __launch_bounds__(256, SPLIT ? 1 : 2) bwd_dkdv_bf16_kernel(BwdAr
                 pw[v >> 3][(v & 7) >> 1] = w2;
                 if constexpr (SPLIT) pl[v >> 3][(v & 7) >> 1] = cvt_pk_bf16(d0 - __uint_as_float(w2 << 16), d1 - __uint_as_float(w2 & 0xffff0000u));
             }
+            if constexpr (SPILL) {
+                // the tile as this wavefront's registers hold it, [j][lane][4 words]: lane (key kl, half h) holds, in
+                // pw[j][2c], pw[j][2c + 1], the queries 16 j + 8 c + 4 h .. + 3.  Two instructions of 1 KB each, written once
+                // and read once: kept out of the way of the tiles the L2 is holding.
+                u32x4_t* tile = (u32x4_t*)ds_tile;
+                if (++se_t == n_qt) {
+                    se_t = 0;
+                    ds_tile += ds_step_r;
+                } else {
+                    ds_tile += ds_step_t;
+                }
+#pragma unroll
+                for (int j = 0; j < 2; ++j) __builtin_nontemporal_store(u32x4_t{pw[j][0], pw[j][1], pw[j][2], pw[j][3]}, tile + 64 * j);
+            }
         }
         const uint16_t *cols, *cols_lo;
         if constexpr (RD) cols = tq(buf), cols_lo = tql(buf);
@@ -757,7 +815,10 @@ __global__ void __launch_bounds__(256, SPLIT ? 1 : 2) bwd_dkdv_bf16_kernel(BwdAr
         using B1 = std::integral_constant<int, (buf.value + 1) % 3>;
         using B2 = std::integral_constant<int, (buf.value + 2) % 3>;
         // tile it + 1 and P(it) are in LDS; every wavefront has left tile it - 1, whose slot takes tile it + 2
-        dma_wait_all();
+        // (SPILL: the D wavefront's two dS stores of the previous iteration are younger than that tile's requests in
+        // its memory queue and need not have been acknowledged)
+        if constexpr (RD && SPILL) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+        else dma_wait_all();
         __syncthreads();
         if (it + 2 < n_it) load(it + 2, B2{});
         // the second products consume s / pw of this tile, then the first products of the next tile refill them
@@ -784,7 +845,139 @@ __global__ void __launch_bounds__(256, SPLIT ? 1 : 2) bwd_dkdv_bf16_kernel(BwdAr
     }
 }
 
+// ---- dQ from the dS tiles the dK / dV pass left behind (bf16) ----
+// A wavefront owns 32 query rows and walks the key tiles.  Its own dS tile (2 KB, consecutive key tiles consecutive in
+// the workspace) comes straight into registers, several tiles ahead; the workgroup's shared K tile comes through a
+// ring of four LDS slots.  The tile is the register image of the wavefront that wrote it (a lane = a key), and this
+// product contracts over keys, so it passes through a 2 KB patch of LDS of the wavefront's own: written as it came,
+// read back with the transposing read (a lane = a query).  Then dQ^T[d][q] += K^T . dS^T, A = the K tile read
+// column-wise.  One product instead of the three of bwd_dq_bf16_kernel: the pass runs at the rate the tiles stream in.
+// Masked positions hold zeros in the tiles, so no mask is applied here.
+template <int D>
+__global__ void __launch_bounds__(256, 2) bwd_dq_stream_kernel(BwdArgs a) {
+    constexpr int DB = D / 32;
+    constexpr int PER_STAGE = TileDma<D>::NLD + 2;   // memory instructions a wavefront issues per ring stage
+    __shared__ __attribute__((aligned(1024))) uint16_t sK0[kBT * D], sK1[kBT * D], sK2[kBT * D], sK3[kBT * D];
+    __shared__ __attribute__((aligned(1024))) char sT[4][2048];   // per wavefront
+    auto tk = [&](auto s) -> uint16_t* { if constexpr (s.value == 0) return sK0; else if constexpr (s.value == 1) return sK1; else if constexpr (s.value == 2) return sK2; else return sK3; };
+    const int n_qtiles = (a.N + kBQ - 1) / kBQ;
+    const int bid = blockIdx.x;
+    const int qt = n_qtiles - 1 - bid / (a.B * a.Hq);
+    const int bh = xcd_grouped_head(bid % (a.B * a.Hq), a.B * a.Hkv, a.n_rep);
+    const int b = bh / a.Hq, hq = bh % a.Hq, kvh = hq / a.n_rep;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ql = lane & 31, h = lane >> 5;
+    const int q0 = qt * kBQ + wave * 32;
+    const int qi = q0 + ql;
+
+    const int wg_qmax = min(qt * kBQ + kBQ - 1, a.N - 1);
+    const int n_tiles = ((a.causal ? wg_qmax + 1 : a.N) + kBT - 1) / kBT;          // key tiles the workgroup walks
+    const int nt_w = q0 < a.N ? ((a.causal ? min(q0 + 31, a.N - 1) + 1 : a.N) + kBT - 1) / kBT : 0;   // of which this wavefront uses
+
+    const uint16_t* Kp = (const uint16_t*)a.k + (int64_t)b * a.s_k[0] + (int64_t)kvh * a.s_k[1];
+    const u32x4_t* Sp = (const u32x4_t*)((const char*)a.ds_tiles + ((((int64_t)b * a.Hq + hq) * a.n_qt32 + min(q0 >> 5, a.n_qt32 - 1)) * a.n_kt32) * 2048) + lane;
+    TileDma<D> dk_;
+    dk_.init(a.s_k[2], wave, lane);
+    constexpr int NI = 8, AHEAD = 6;   // dS tiles: register ring, and how many tiles ahead they are requested
+    u32x4_t img[NI][2];
+    // Every step issues the same number of loads, so that the wait counts below hold: past the end the tile index is
+    // clamped (the tile is fetched again and not used).
+    auto load_k = [&](int t, auto slot) {
+        const int kt = min(t, n_tiles - 1);
+        dk_.load(tk(slot), Kp + (int64_t)kt * kBT * a.s_k[2], a.N - kt * kBT, a.s_k[2], wave);
+    };
+    auto load_s = [&](int t, auto islot) {
+        const u32x4_t* tile = Sp + (int64_t)min(t, max(nt_w - 1, 0)) * 128;
+        img[islot.value][0] = __builtin_nontemporal_load(tile);
+        img[islot.value][1] = __builtin_nontemporal_load(tile + 64);
+    };
+    f32x16_t acc[DB];
+#pragma unroll
+    for (int i = 0; i < DB; ++i)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) acc[i][j] = 0.f;
+    // The patch holds the image as [j][position of the writing lane][4 words], the lane (key kl, half hh) at position
+    // 2 kl + hh, rotated by 128 bytes for j = 1: the 16 lanes of a transposing read then fetch 4 keys x 32 bytes =
+    // 128 consecutive bytes, and the four such groups of an instruction fall in different banks.
+    char* patch = sT[wave];
+    const int wr_off = (2 * ql + h) * 16;
+    const int i16 = lane & 15, g4 = (lane >> 4) & 1;
+    // k-step j', keys 16 j' + 4 h + (i16 >> 2) (+ 8), queries 16 g4 + 4 (i16 & 3) .. + 3: words 2c, 2c + 1 of the lane
+    // (key, hh) with hh = i16 & 1, c = (i16 >> 1) & 1, in half j = g4 of the image
+    const int rd_off = 32 * (4 * h + (i16 >> 2)) + 16 * (i16 & 1) + 8 * ((i16 >> 1) & 1);
+    auto step = [&](int t, auto idx) {
+        using KS = std::integral_constant<int, idx.value % 4>;
+        using KL = std::integral_constant<int, (idx.value + 3) % 4>;
+        using IL = std::integral_constant<int, (idx.value + AHEAD) % NI>;
+        // This wavefront's share of K tile t has landed.  Younger in its memory queue, and possibly still in flight: the
+        // dS tile requested right behind it and the two steps' requests since.  No fence: it would drain them.
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 + 2 * PER_STAGE) : "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        const u32x4_t i0 = img[idx.value % NI][0], i1 = img[idx.value % NI][1];
+        load_k(t + 3, KL{});   // into the slot every wavefront left before this barrier
+        load_s(t + AHEAD, IL{});
+        if (t >= nt_w) return;
+        using slot_t = KS;
+        const slot_t slot{};
+        const uint16_t* tK = tk(slot);
+        *(u32x4_t*)(patch + wr_off) = i0;
+        *(u32x4_t*)(patch + 1024 + ((wr_off + 128) & 1023)) = i1;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const char* half = patch + 1024 * g4;
+            const uint2 lo = lds_tr16(half + ((rd_off + 512 * j + 128 * g4) & 1023));
+            const uint2 hi = lds_tr16(half + ((rd_off + 512 * j + 256 + 128 * g4) & 1023));
+            const bf16x8_t dsf = __builtin_bit_cast(bf16x8_t, uint4{lo.x, lo.y, hi.x, hi.y});
+#pragma unroll
+            for (int db = 0; db < DB; ++db) acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_transposed<D>(tK, j, db, lane), dsf, acc[db], 0, 0, 0);
+        }
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    using I3 = std::integral_constant<int, 3>;
+    using I4 = std::integral_constant<int, 4>;
+    using I5 = std::integral_constant<int, 5>;
+    using I6 = std::integral_constant<int, 6>;
+    using I7 = std::integral_constant<int, 7>;
+    // the order of the first requests gives every K tile at least as many younger requests as the steady state does
+    load_k(0, I0{});
+    load_s(0, I0{});
+    load_s(1, I1{});
+    load_s(2, I2{});
+    load_s(3, I3{});
+    load_k(1, I1{});
+    load_s(4, I4{});
+    load_k(2, I2{});
+    load_s(5, I5{});
+    for (int t = 0; t < n_tiles; t += 8) {
+        step(t, I0{});
+        if (t + 1 < n_tiles) step(t + 1, I1{});
+        if (t + 2 < n_tiles) step(t + 2, I2{});
+        if (t + 3 < n_tiles) step(t + 3, I3{});
+        if (t + 4 < n_tiles) step(t + 4, I4{});
+        if (t + 5 < n_tiles) step(t + 5, I5{});
+        if (t + 6 < n_tiles) step(t + 6, I6{});
+        if (t + 7 < n_tiles) step(t + 7, I7{});
+    }
+    dma_wait_all();   // the clamped requests of the last steps write LDS: they land before the workgroup gives it back
+    if (qi < a.N) {
+        const int64_t row = (int64_t)b * a.s_dq[0] + (int64_t)hq * a.s_dq[1] + (int64_t)qi * a.s_dq[2];
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int vq = 0; vq < 4; ++vq) store4<false>(a.dq, row + 32 * db + 8 * vq + 4 * h, a.scale, acc[db], 4 * vq);
+    }
+}
+
 // Instantiated explicitly: the host pass of this compiler drops the implicit instantiation of the launch stubs.
+template __global__ void bwd_dkdv_bf16_kernel<128, false, true>(BwdArgs);
+template __global__ void bwd_dkdv_bf16_kernel<64, false, true>(BwdArgs);
+template __global__ void bwd_dq_stream_kernel<128>(BwdArgs);
+template __global__ void bwd_dq_stream_kernel<64>(BwdArgs);
+template __global__ void bwd_rowstats_bf16_kernel<128>(BwdArgs);
+template __global__ void bwd_rowstats_bf16_kernel<64>(BwdArgs);
 template __global__ void bwd_dkdv_bf16_kernel<128, false>(BwdArgs);
 template __global__ void bwd_dkdv_bf16_kernel<64, false>(BwdArgs);
 template __global__ void bwd_dq_bf16_kernel<128, false>(BwdArgs);
@@ -872,6 +1065,18 @@ int launch_backward(const BwdArgs& a, int64_t D, hipStream_t st) {
     const dim3 gq((unsigned)(tiles * a.B * a.Hq)), gk((unsigned)(tiles * a.B * a.Hkv));
     if constexpr (sizeof(T) == 2) {
         const dim3 gk((unsigned)(ceil_div(a.N, kBK) * a.B * a.Hkv));
+        if (a.ds_tiles) {  // one-pass dS: row constants, dK / dV (leaving the dS tiles), dQ from the tiles
+            if (D == 128) {
+                hipLaunchKernelGGL((bwd_rowstats_bf16_kernel<128>), dim3((unsigned)ceil_div(rows, 16)), dim3(256), 0, st, a);
+                hipLaunchKernelGGL((bwd_dkdv_bf16_kernel<128, false, true>), gk, dim3(256), 0, st, a);
+                hipLaunchKernelGGL((bwd_dq_stream_kernel<128>), gq, dim3(256), 0, st, a);
+            } else {
+                hipLaunchKernelGGL((bwd_rowstats_bf16_kernel<64>), dim3((unsigned)ceil_div(rows, 32)), dim3(256), 0, st, a);
+                hipLaunchKernelGGL((bwd_dkdv_bf16_kernel<64, false, true>), gk, dim3(256), 0, st, a);
+                hipLaunchKernelGGL((bwd_dq_stream_kernel<64>), gq, dim3(256), 0, st, a);
+            }
+            return check_launch();
+        }
         if (D == 128) {
             hipLaunchKernelGGL((bwd_dq_bf16_kernel<128, false>), gq, dim3(256), 0, st, a);
             hipLaunchKernelGGL((bwd_dkdv_bf16_kernel<128, false>), gk, dim3(256), 0, st, a);
@@ -920,6 +1125,13 @@ using namespace vsp;
 extern "C" size_t vsp_attn_backward_workspace_bytes(int32_t B, int32_t Hq, int32_t N) {
     if (B <= 0 || Hq <= 0 || N <= 0) return 0;
     return 2 * (size_t)B * (size_t)Hq * (size_t)N * sizeof(float);   // Di and the rescaled log-sum-exp
+}
+
+extern "C" size_t vsp_attn_backward_fast_workspace_bytes(int32_t B, int32_t Hq, int32_t N) {
+    if (B <= 0 || Hq <= 0 || N <= 0) return 0;
+    const size_t base = (vsp_attn_backward_workspace_bytes(B, Hq, N) + 255) & ~(size_t)255;
+    const size_t n_qt32 = ((size_t)N + 31) / 32, n_kt32 = 2 * (((size_t)N + 63) / 64);
+    return base + (size_t)B * (size_t)Hq * n_qt32 * n_kt32 * 2048;   // one 32 x 32 bf16 dS tile per (query tile, key tile)
 }
 
 extern "C" int vsp_attn_prefill_backward(const vsp_tensor* dout, const vsp_tensor* q, const vsp_tensor* k,
@@ -990,6 +1202,12 @@ extern "C" int vsp_attn_prefill_backward(const vsp_tensor* dout, const vsp_tenso
     a.causal = is_causal ? 1 : 0;
     a.scale = scale;
     a.D_true = (int)D;
+    // bf16 with the larger workspace: dS is computed once (see include/vsp_attn.h)
+    if (dt == VSP_BF16 && workspace_bytes >= vsp_attn_backward_fast_workspace_bytes((int32_t)B, (int32_t)Hq, (int32_t)N) && is_aligned16(workspace)) {
+        a.ds_tiles = (uint16_t*)((char*)workspace + ((vsp_attn_backward_workspace_bytes((int32_t)B, (int32_t)Hq, (int32_t)N) + 255) & ~(size_t)255));
+        a.n_qt32 = (int)ceil_div(N, 32);
+        a.n_kt32 = (int)(2 * ceil_div(N, 64));
+    }
     return dt == VSP_F32 ? launch_backward<float>(a, D, (hipStream_t)stream) : launch_backward<uint16_t>(a, D, (hipStream_t)stream);
 }
 
