@@ -8,7 +8,9 @@
 // instead of scalar FMAs, D in {64, 128} (and 32 for fp32 operands), grouped-query heads folded in
 // (dK / dV of a kv head sum over its query heads, the gradient of ops::repeat_kv), and no atomics:
 // dQ is produced by one pass that owns query rows, dK / dV by a second pass that owns key rows, so the
-// result is bitwise reproducible (the reference accumulates dQ with atomicAdd).
+// result is bitwise reproducible (the reference accumulates dQ with atomicAdd).  Both passes compute dS; with the
+// larger of the two workspaces (bf16 operands) the dK / dV pass runs first and leaves dS behind as bf16 tiles, and dQ is
+// one product over those tiles (bwd_rowstats_bf16_kernel, bwd_dkdv_bf16_kernel<D, false, true>, bwd_dq_stream_kernel).
 //
 // fp32 operands: fp32 MFMA (32x32x2) throughout.  bf16 operands: bf16 MFMA (32x32x16) with fp32 accumulation
 // and fp32 softmax algebra; P and dS are rounded to bf16 (round-to-nearest-even) between the products, as P is
