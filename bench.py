@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on ONE MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|p4k|c3|c2f|c4|c5|c4f|c4p|c4w|c4m|c2c|c3c|k512|r2|b2|b3|b2r|b3r|b2f] [--no-cpu] [--no-extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|p4k|c3|c2f|c4|c5|c4f|c4p|c4w|c4m|c2c|c3c|k512|r2|b2|b3|b2s|b3r|b2f] [--no-cpu] [--no-extra]
 
 A "step" is one pass of the hot path over one batch of synthetic input that is already resident in
 HBM: one prefill launch (c2, p4k, c3) or one decode call = split-K kernel + combine kernel (c4, c5).
@@ -64,17 +64,17 @@ WORKLOADS = {
                  name="one chunk of a long prompt: the last 512 tokens of a 32768-token context read from the bf16 cache planes, "
                       "B1, 32 q / 8 kv heads, D128 (128 workgroups of queries: the context is split over workgroups and merged by "
                       "the decode step's combine kernel)"),
-    "b2": dict(kind="backward", B=4, Hq=32, Hkv=8, D=128, N=2048, fast=True,
+    "b2": dict(kind="backward", B=4, Hq=32, Hkv=8, D=128, N=2048, fast=False,
                name="attention backward at config 2's shape: causal GQA bf16 in/out, bf16 MFMA with fp32 accumulation, "
-                    "B4, 32 q / 8 kv heads, D128, N2048 (dq, dk, dv; 2.5 x the forward's FLOPs); dS computed once and kept as "
-                    "bf16 tiles in the workspace (vsp_attn_backward_fast_workspace_bytes)"),
+                    "B4, 32 q / 8 kv heads, D128, N2048 (dq, dk, dv; 2.5 x the forward's FLOPs); the small workspace: dS "
+                    "recomputed in the dQ pass, which is the faster path at this context length"),
     "b3": dict(kind="backward", B=1, Hq=32, Hkv=8, D=128, N=8192, fast=True,
                name="attention backward at config 3's shape: causal GQA bf16 in/out, bf16 MFMA with fp32 accumulation, "
                     "B1, 32 q / 8 kv heads, D128, N8192 (dq, dk, dv; 2.5 x the forward's FLOPs); dS computed once and kept as "
-                    "bf16 tiles in the workspace (vsp_attn_backward_fast_workspace_bytes)"),
-    "b2r": dict(kind="backward", B=4, Hq=32, Hkv=8, D=128, N=2048, fast=False,
-                name="attention backward at config 2's shape with the small workspace: dS recomputed in the dQ pass (seven tile "
-                     "products for five)"),
+                    "bf16 tiles in the workspace (vsp_attn_backward_fast_workspace_bytes), the faster path from 4096 tokens on"),
+    "b2s": dict(kind="backward", B=4, Hq=32, Hkv=8, D=128, N=2048, fast=True,
+                name="attention backward at config 2's shape with dS computed once and kept as bf16 tiles in the larger "
+                     "workspace (five tile products for five)"),
     "b3r": dict(kind="backward", B=1, Hq=32, Hkv=8, D=128, N=8192, fast=False,
                 name="attention backward at config 3's shape with the small workspace: dS recomputed in the dQ pass (seven tile "
                      "products for five)"),
@@ -384,9 +384,12 @@ PROFILE_OF = {
     "c5": ("decode_q8_0_config5.txt", ("decode_q8_kernel", "decode_combine_kernel"), 2282225664),
     "c4f": ("decode_f32_config4.txt", ("decode_f32_mfma_kernel", "decode_combine_kernel"), 5229871104),
     # backward: Q, dO, O, K, V, lse read; dQ, dK, dV written
-    "b2": ("backward_bf16_config2.txt", ("bwd_rowstats_bf16_kernel", "bwd_dkdv_bf16_kernel", "bwd_dq_stream_kernel"),
+    "b2": ("backward_bf16_config2.txt", ("bwd_dq_bf16_kernel", "bwd_dkdv_bf16_kernel"), 4 * 67108864 + 4 * 16777216 + 1048576),
+    "b3r": ("backward_bf16_config3.txt", ("bwd_dq_bf16_kernel", "bwd_dkdv_bf16_kernel"), 4 * 67108864 + 4 * 16777216 + 1048576),
+    "b2s": ("backward_bf16_stored_ds_config2.txt", ("bwd_rowstats_bf16_kernel", "bwd_dkdv_bf16_kernel", "bwd_dq_stream_kernel"),
+            4 * 67108864 + 4 * 16777216 + 1048576),
+    "b3": ("backward_bf16_stored_ds_config3.txt", ("bwd_rowstats_bf16_kernel", "bwd_dkdv_bf16_kernel", "bwd_dq_stream_kernel"),
            4 * 67108864 + 4 * 16777216 + 1048576),
-    "b2r": ("backward_bf16_recompute_config2.txt", ("bwd_dq_bf16_kernel", "bwd_dkdv_bf16_kernel"), 4 * 67108864 + 4 * 16777216 + 1048576),
 }
 CALIBRATION_KERNEL, CALIBRATION_KIB = "CUDAFunctorOnSelf_add<int>", 1048576.0
 
@@ -536,7 +539,7 @@ def main():
 
     if not args.no_extra:
         others = {}
-        for key in ("c2", "p4k", "c3", "c2f", "c4", "c5", "c4f", "c4p", "c4w", "c4m", "c2c", "c3c", "k512", "r2", "b2", "b3", "b2r", "b3r", "b2f"):
+        for key in ("c2", "p4k", "c3", "c2f", "c4", "c5", "c4f", "c4p", "c4w", "c4m", "c2c", "c3c", "k512", "r2", "b2", "b3", "b2s", "b3r", "b2f"):
             if key == args.workload:
                 continue
             r = Runner(key, torch, va)

@@ -401,14 +401,20 @@ static void test_backward_dispatch_seam() {
     // the front end with the reference's defaults (is_causal = true, dropout_p = 0, no mask)
     auto g = ops::flash_attention_backward(tdo, tq, tk, tv, o, l, scale);
     CHECK(max_abs_diff(to_host(std::get<0>(g)), wq.data(), wq.size()) < 2e-4);
-    // bf16 tensors: with the larger workspace (the default while it stays under backward_fast_workspace_limit()) dS is
-    // computed once, with the limit at 0 twice; both inside the bf16 bar against the fp32 oracle, and dK / dV the same
+    // bf16 tensors: with the larger workspace (taken from backward_fast_min_context() tokens on while it stays under
+    // backward_fast_workspace_limit()) dS is computed once, with the limit at 0 twice; both inside the bf16 bar against the
+    // fp32 oracle, and dK / dV the same
     {
         Tensor bq = to_dev(q, {B, Hq, N, D}, DType::BFloat16), bk = to_dev(k, {B, Hkv, N, D}, DType::BFloat16);
         Tensor bv = to_dev(v, {B, Hkv, N, D}, DType::BFloat16), bdo = to_dev(dout, {B, Hq, N, D}, DType::BFloat16);
         Tensor bo = empty({B, Hq, N, D}, DType::BFloat16), bl = empty({B, Hq, N}, DType::Float32);
         ops::flash_attention_hip_dispatch(bq, ops::repeat_kv(bk, n), ops::repeat_kv(bv, n), bo, bl, scale, true, 0.0f, false, nullptr);
+        const int64_t keep_n = ops::backward_fast_min_context();
+        ops::backward_fast_min_context() = 1;
+        const size_t taken = BlockCache::instance().bytes_taken();
         auto once = ops::flash_attention_backward(bdo, bq, bk, bv, bo, bl, scale);
+        CHECK(BlockCache::instance().bytes_taken() - taken >= vsp_attn_backward_fast_workspace_bytes((int32_t)B, (int32_t)Hq, (int32_t)N));
+        ops::backward_fast_min_context() = keep_n;
         const size_t keep = ops::backward_fast_workspace_limit();
         ops::backward_fast_workspace_limit() = 0;
         auto twice = ops::flash_attention_backward(bdo, bq, bk, bv, bo, bl, scale);

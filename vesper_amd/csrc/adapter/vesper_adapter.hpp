@@ -516,7 +516,13 @@ inline Tensor flash_attention_split(const Tensor& q, const Tensor& k, const Tens
 }
 
 // bf16 backward: the larger workspace, with which dS is computed once and kept as tiles (about 2 N^2 bytes per query
-// head, vsp_attn_backward_fast_workspace_bytes), is taken when it is no larger than this many bytes; 0 switches it off.
+// head, vsp_attn_backward_fast_workspace_bytes), is taken for contexts of at least backward_fast_min_context() tokens
+// (4096: below that recomputing dS measured as fast) when it is no larger than backward_fast_workspace_limit() bytes
+// (8 GiB; 0 switches the path off).
+inline int64_t& backward_fast_min_context() {
+    static int64_t n = 4096;
+    return n;
+}
 inline size_t& backward_fast_workspace_limit() {
     static size_t limit = (size_t)8 << 30;
     return limit;
@@ -543,7 +549,7 @@ inline void flash_attention_backward_hip_dispatch(const Tensor& grad_output, con
         return;
     }
     size_t ws_bytes = q.ndim() == 4 ? vsp_attn_backward_workspace_bytes((int32_t)q.shape()[0], (int32_t)q.shape()[1], (int32_t)q.shape()[2]) : 0;
-    if (q.ndim() == 4 && q.dtype() == DType::BFloat16) {   // dS kept instead of recomputed, when the tiles are affordable
+    if (q.ndim() == 4 && q.dtype() == DType::BFloat16 && q.shape()[2] >= backward_fast_min_context()) {   // dS kept instead of recomputed
         const size_t fast = vsp_attn_backward_fast_workspace_bytes((int32_t)q.shape()[0], (int32_t)q.shape()[1], (int32_t)q.shape()[2]);
         if (fast > 0 && fast <= backward_fast_workspace_limit()) ws_bytes = fast;
     }
