@@ -167,6 +167,29 @@ def test_bf16_dS_once_against_dS_twice(va):
             assert (a - b).abs().mean().item() <= (1e-3 if name == "dq" else 1e-4) * ref, (name, causal, (a - b).abs().mean().item())
 
 
+def test_the_workspace_size_selects_the_bf16_path(va):
+    # one byte short of vsp_attn_backward_fast_workspace_bytes(): the recomputing path, bit for bit; fp32 tensors ignore
+    # the extra room
+    B, Hq, Hkv, N, D = 1, 4, 2, 300, 64
+    g = torch.Generator(device="cuda").manual_seed(29)
+    mk = lambda h, dt: (torch.randn(B, h, N, D, device=G.dev(), generator=g) * 0.7).to(dt)
+    for dt in (torch.bfloat16, torch.float32):
+        q, k, v, dout = mk(Hq, dt), mk(Hkv, dt), mk(Hkv, dt), mk(Hq, dt)
+        out, lse = va.flash_attention(q, k, v, 0.125, True, return_lse=True)
+        small = va.flash_attention_backward(dout, q, k, v, out, lse, 0.125, True)
+        big = va.backward_workspace(q, fast=True)
+        short = va.flash_attention_backward(dout, q, k, v, out, lse, 0.125, True, workspace=big[:big.numel() - 1])
+        full = va.flash_attention_backward(dout, q, k, v, out, lse, 0.125, True, workspace=big)
+        for a, b in zip(short, small):
+            assert torch.equal(a, b)
+        if dt == torch.float32:
+            for a, b in zip(full, small):
+                assert torch.equal(a, b)
+        else:
+            assert not torch.equal(full[0], small[0])      # dQ from the stored tiles: P rounded before the multiply
+            assert (full[0].float() - small[0].float()).abs().max().item() <= 2e-2 * max(1.0, small[0].float().abs().max().item())
+
+
 @pytest.mark.parametrize("bf16,fast", [(False, False), (True, False), (True, True)])
 def test_strided_operands(va, bf16, fast):
     # [B, N, H, D] storage viewed as [B, H, N, D] (what a fused qkv projection hands over): the strides of every
