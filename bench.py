@@ -379,6 +379,7 @@ PROFILE_OF = {
     "r2": ("rope_append_bf16_config2.txt", ("append_bf16_tile_kernel<unsigned short, true",), 202375168),
     "c4": ("decode_bf16_config4.txt", ("decode_bf16_kernel", "decode_combine_kernel"), 2614935552),
     "c4m": ("decode_bf16_multi_config4.txt", ("decode_bf16_kernel", "decode_combine_kernel"), 2614935552 + 3 * 524288),
+    "c4p": ("decode_bf16_paged_config4.txt", ("decode_bf16_kernel", "decode_combine_kernel"), 2614935552),
     "c4w": ("decode_bf16_proj_config4.txt", ("decode_bf16_kernel", "decode_combine_kernel", "proj_bf16_partial_kernel", "proj_reduce_kernel"),
             2614935552 + 33554432),
     "c5": ("decode_q8_0_config5.txt", ("decode_q8_kernel", "decode_combine_kernel"), 2282225664),
