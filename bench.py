@@ -387,6 +387,9 @@ PROFILE_OF = {
     # backward: Q, dO, O, K, V, lse read; dQ, dK, dV written
     "b2": ("backward_bf16_config2.txt", ("bwd_dq_bf16_kernel", "bwd_dkdv_bf16_kernel"), 4 * 67108864 + 4 * 16777216 + 1048576),
     "b3r": ("backward_bf16_config3.txt", ("bwd_dq_bf16_kernel", "bwd_dkdv_bf16_kernel"), 4 * 67108864 + 4 * 16777216 + 1048576),
+    # the same tensors in fp32: twice the bytes
+    "b2f": ("backward_split_f32_config2.txt", ("bwd_split_kernel", "bwd_dq_bf16_kernel", "bwd_dkdv_bf16_kernel"),
+            4 * 134217728 + 4 * 33554432 + 1048576),
     "b2s": ("backward_bf16_stored_ds_config2.txt", ("bwd_rowstats_bf16_kernel", "bwd_dkdv_bf16_kernel", "bwd_dq_stream_kernel"),
             4 * 67108864 + 4 * 16777216 + 1048576),
     "b3": ("backward_bf16_stored_ds_config3.txt", ("bwd_rowstats_bf16_kernel", "bwd_dkdv_bf16_kernel", "bwd_dq_stream_kernel"),
