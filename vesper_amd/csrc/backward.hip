@@ -648,9 +648,9 @@ __global__ void __launch_bounds__(256, SPLIT ? 1 : 2) bwd_dkdv_bf16_kernel(BwdAr
     char* ds_tile = nullptr;
     int64_t ds_step_t = 0, ds_step_r = 0;   // to the next query tile; from the last query tile of a head to the first of the next
     if constexpr (SPILL) {
-        ds_step_t = (int64_t)a.n_kt32 * 2048;
-        ds_step_r = (int64_t)a.n_qt32 * ds_step_t - (int64_t)(n_qt - 1) * ds_step_t;
-        ds_tile = (char*)a.ds_tiles + ((((int64_t)b * a.Hq + kvh * a.n_rep) * a.n_qt32 + qt_begin) * a.n_kt32 + (key0 >> 5)) * 2048 + lane * 16;
+        ds_step_t = -(int64_t)a.n_kt32 * 2048;
+        ds_step_r = (int64_t)a.n_qt32 * a.n_kt32 * 2048 - (int64_t)(n_qt - 1) * ds_step_t;
+        ds_tile = (char*)a.ds_tiles + ((((int64_t)b * a.Hq + kvh * a.n_rep) * a.n_qt32 + qt_begin + n_qt - 1) * a.n_kt32 + (key0 >> 5)) * 2048 + lane * 16;
     }
     const float scale_log2 = a.scale * kLog2e;
 
@@ -667,7 +667,7 @@ __global__ void __launch_bounds__(256, SPLIT ? 1 : 2) bwd_dkdv_bf16_kernel(BwdAr
         }
     };
     auto load = [&](int it, auto buf) {
-        const int hq = kvh * a.n_rep + ld_r, qb = (qt_begin + ld_t) * kBT;
+        const int hq = kvh * a.n_rep + ld_r, qb = (qt_begin + (n_qt - 1 - ld_t)) * kBT;   // a head's query tiles from the last one down
         advance(ld_r, ld_t);
         dq_.load(tq(buf), (const uint16_t*)a.q + (int64_t)b * a.s_q[0] + (int64_t)hq * a.s_q[1] + (int64_t)qb * a.s_q[2], a.N - qb,
                  a.s_q[2], wave);
@@ -706,7 +706,7 @@ __global__ void __launch_bounds__(256, SPLIT ? 1 : 2) bwd_dkdv_bf16_kernel(BwdAr
             }
         }
         if constexpr (!RD) {
-            const int qb = (qt_begin + fi_t) * kBT;
+            const int qb = (qt_begin + (n_qt - 1 - fi_t)) * kBT;
             float lq[16];
 #pragma unroll
             for (int g = 0; g < 4; ++g) *(float4*)&lq[4 * g] = *(const float4*)&tl(buf)[8 * g + 4 * h];
