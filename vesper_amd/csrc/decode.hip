@@ -173,6 +173,47 @@ __device__ inline bool locate_work(const DecodeArgs& a, int item, int lane, int&
     return false;
 }
 
+// The (m, l, O^T) of a workgroup's four wavefronts, left in LDS per column, merged into one split-K partial per column.
+// First, one lane per column: the merged maximum, the four weights 2^(m_w - m), the merged sum and the partial's row
+// (once per column, not once per element: the weights are four exp2 and the row takes integer divisions).  Then one
+// element per thread: o = sum_w weight_w * O_w in wavefront order.  ZERO_FOR_EMPTY: a wavefront that saw no key of a
+// short split, or a column with no key in it, carries m = -inf, l = 0 and zero sums, and gets the weight 0 explicitly;
+// otherwise -inf is replaced by 0 as the reference point (a column without a key in this split: zero sums, m = -inf).
+template <int D, bool ZERO_FOR_EMPTY>
+__device__ inline void merge_waves_and_store(const DecodeArgs& a, const float (&sm_o)[kWaves][16][D + 4], const float (&sm_m)[kWaves][16],
+                                             const float (&sm_l)[kWaves][16], int b, int kvh, int split, int tid) {
+    __shared__ float sm_f[kWaves][16];
+    __shared__ int64_t sm_row[16];
+    const int ncol = column_count(a);
+    if (tid < ncol) {
+        const int hc = tid;
+        float mm = sm_m[0][hc];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) mm = fmaxf(mm, sm_m[w][hc]);
+        const float mm_ref = mm == -INFINITY ? 0.f : mm;
+        float ll = 0.f;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            const float f = ZERO_FOR_EMPTY ? (sm_m[w][hc] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(sm_m[w][hc] - mm))
+                                           : __builtin_amdgcn_exp2f(sm_m[w][hc] - mm_ref);
+            sm_f[w][hc] = f;
+            ll += f * sm_l[w][hc];
+        }
+        const int64_t row = partial_row(a, b, kvh, column_of(a, hc), split);
+        sm_row[hc] = row;
+        a.ws_ml[row * 2] = mm;
+        a.ws_ml[row * 2 + 1] = ll;
+    }
+    __syncthreads();
+    for (int i = tid; i < ncol * D; i += 256) {
+        const int hc = i / D, d = i % D;
+        float o = 0.f;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) o += sm_f[w][hc] * sm_o[w][hc][d];
+        a.ws_o[sm_row[hc] * D + d] = o;
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // bf16 cache
 // ---------------------------------------------------------------------------------------------
@@ -316,26 +357,7 @@ __global__ void __launch_bounds__(256, 2) decode_bf16_kernel(DecodeArgs a) {
         }
     }
     __syncthreads();
-    for (int i = tid; i < column_count(a) * D; i += 256) {
-        const int hc = i / D, d = i % D;
-        float mm = sm_m[0][hc];
-#pragma unroll
-        for (int w = 1; w < kWaves; ++w) mm = fmaxf(mm, sm_m[w][hc]);
-        const float mm_ref = mm == -INFINITY ? 0.f : mm;   // a column without a key in this split: zero sums, m = -inf
-        float o = 0.f, ll = 0.f;
-#pragma unroll
-        for (int w = 0; w < kWaves; ++w) {
-            const float f = __builtin_amdgcn_exp2f(sm_m[w][hc] - mm_ref);
-            o += f * sm_o[w][hc][d];
-            ll += f * sm_l[w][hc];
-        }
-        const int64_t row = partial_row(a, b, kvh, column_of(a, hc), split);
-        a.ws_o[row * D + d] = o;
-        if (d == 0) {
-            a.ws_ml[row * 2] = mm;
-            a.ws_ml[row * 2 + 1] = ll;
-        }
-    }
+    merge_waves_and_store<D, false>(a, sm_o, sm_m, sm_l, b, kvh, split, tid);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -534,26 +556,7 @@ __global__ void __launch_bounds__(256, 2) decode_q8_kernel(DecodeArgs a) {
         }
     }
     __syncthreads();
-    for (int i = tid; i < column_count(a) * D; i += 256) {
-        const int hc = i / D, d = i % D;
-        float mm = sm_m[0][hc];
-#pragma unroll
-        for (int w = 1; w < kWaves; ++w) mm = fmaxf(mm, sm_m[w][hc]);
-        const float mm_ref = mm == -INFINITY ? 0.f : mm;   // a column without a key in this split: zero sums, m = -inf
-        float o = 0.f, ll = 0.f;
-#pragma unroll
-        for (int w = 0; w < kWaves; ++w) {
-            const float f = __builtin_amdgcn_exp2f(sm_m[w][hc] - mm_ref);
-            o += f * sm_o[w][hc][d];
-            ll += f * sm_l[w][hc];
-        }
-        const int64_t row = partial_row(a, b, kvh, column_of(a, hc), split);
-        a.ws_o[row * D + d] = o;
-        if (d == 0) {
-            a.ws_ml[row * 2] = mm;
-            a.ws_ml[row * 2 + 1] = ll;
-        }
-    }
+    merge_waves_and_store<D, false>(a, sm_o, sm_m, sm_l, b, kvh, split, tid);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -820,26 +823,7 @@ __global__ void __launch_bounds__(256, 2) decode_f32_mfma_kernel(DecodeArgs a) {
         }
     }
     __syncthreads();
-    for (int i = tid; i < column_count(a) * D; i += 256) {
-        const int hc = i / D, d = i % D;
-        float mm = sm_m[0][hc];
-#pragma unroll
-        for (int w = 1; w < kWaves; ++w) mm = fmaxf(mm, sm_m[w][hc]);
-        float o = 0.f, ll = 0.f;
-#pragma unroll
-        for (int w = 0; w < kWaves; ++w) {
-            // a wavefront that saw no key of a short split, or a column with no key in it, carries m = -inf, l = 0 and zero sums
-            const float f = sm_m[w][hc] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(sm_m[w][hc] - mm);
-            o += f * sm_o[w][hc][d];
-            ll += f * sm_l[w][hc];
-        }
-        const int64_t row = partial_row(a, b, kvh, column_of(a, hc), split);
-        a.ws_o[row * D + d] = o;
-        if (d == 0) {
-            a.ws_ml[row * 2] = mm;
-            a.ws_ml[row * 2 + 1] = ll;
-        }
-    }
+    merge_waves_and_store<D, true>(a, sm_o, sm_m, sm_l, b, kvh, split, tid);
 }
 
 // ---------------------------------------------------------------------------------------------
