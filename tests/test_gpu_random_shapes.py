@@ -64,6 +64,29 @@ def test_decode_random_shapes(va, seed):
     G.assert_f32_close(out.cpu().numpy(), oracle_decode(q, k, v, lens), f"f32 {c} {lens}")
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_decode_random_shapes_with_many_query_heads_per_kv_head(va, seed):
+    # more than 16 query heads per kv head are served in column groups of 16 (bf16 / Q8_0 caches); 16 itself and the
+    # counts around a group boundary are the interesting ones
+    r = np.random.default_rng(7000 + seed)
+    Hkv, n_rep = int(r.choice([1, 2, 3])), int(r.choice([15, 16, 17, 24, 31, 32, 33, 40]))
+    B, S, D = int(r.integers(1, 4)), int(r.integers(1, 600)), int(r.choice([64, 128]))
+    Hq = Hkv * n_rep
+    lens = [int(x) for x in r.integers(0, S + 1, size=B)]
+    lens[int(r.integers(0, B))] = S
+    q, k, v = I.qkv(7500 + seed, B, Hq, Hkv, 1, S, D)
+    q, kb, vb = O.bf16_round(q), O.bf16_round(k), O.bf16_round(v)
+    sl = torch.tensor(lens, dtype=torch.int32, device=G.dev())
+    tag = f"B{B} Hq{Hq} Hkv{Hkv} S{S} D{D} {lens}"
+    out = va.decode_attention(G.to_bf16_dev(q), fill_cache(va, "bf16", kb, vb), seq_lens=sl)
+    G.assert_bf16_close(G.bf16_to_np(out), oracle_decode(q, kb, vb, lens), "bf16 " + tag)
+    kd, vd = O.q8_0_dequantize(*O.q8_0_quantize(k)), O.q8_0_dequantize(*O.q8_0_quantize(v))
+    out = va.decode_attention(G.to_bf16_dev(q), fill_cache(va, "q8_0", k, v), seq_lens=sl)
+    G.assert_bf16_close(G.bf16_to_np(out), oracle_decode(q, kd, vd, lens), "q8_0 " + tag)
+    out = va.decode_attention(G.f32_dev(q), fill_cache(va, "f32", k, v), seq_lens=sl)
+    G.assert_f32_close(out.cpu().numpy(), oracle_decode(q, k, v, lens), "f32 " + tag)
+
+
 @pytest.mark.parametrize("seed", range(12))
 def test_backward_random_shapes(va, seed):
     c = draw(5000 + seed, 200)
